@@ -1,0 +1,152 @@
+"""GPU parity tests of the HIP TQ8 linear path against the CPU oracle, through the C-ABI
+(ctypes).  Tolerances: rotation and dequantised weights bit-exact (the kernels keep the
+reference's fp32 operation order); layer outputs within 1e-3 relative L2 for fp32
+activations and 5e-3 for bf16/f16 activations."""
+import numpy as np
+import pytest
+
+import __graft_entry__ as entry
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tq():
+    return entry.load_package()
+
+
+def _rel(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+
+
+# ---------------------------------------------------------------- rotation
+@pytest.mark.parametrize("rows,cols,bs", [(1, 512, 512), (1, 384, 128), (4, 896, 128), (2, 4864, 256),
+                                          (3, 256, 64), (2, 64, 32), (5, 2048, 512), (3, 5120, 512),
+                                          (2, 4096, 1024), (2, 4096, 2048), (2, 96, 16), (3, 64, 2),
+                                          (2, 27648, 512)])
+def test_rotation_bit_exact(tq, oracle, rows, cols, bs):
+    rng = np.random.default_rng(rows * 1000 + cols + bs)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    for seed in (42, 0xCAFEBABE):
+        assert np.array_equal(tq.apply_wht_rotation(x, seed, bs), oracle.wht_forward(x, seed, bs))
+        assert np.array_equal(tq.apply_inverse_wht_rotation(x, seed, bs), oracle.wht_inverse(x, seed, bs))
+    rt = tq.apply_inverse_wht_rotation(tq.apply_wht_rotation(x, 42, bs), 42, bs)
+    assert np.abs(rt - x).max() < 1e-4                      # tests/unit/test_rotation.cpp:17-34
+
+
+def test_rotation_rejects_non_divisible(tq):
+    with pytest.raises(ValueError):
+        tq.apply_wht_rotation(np.zeros((1, 96), np.float32), 1, 64)
+
+
+# ------------------------------------------------------------- dequantiser
+MODES = {
+    "shared": dict(pb=4, rb=4, shared=True),
+    "dual": dict(pb=4, rb=4, shared=False),
+    "primary_only": dict(pb=4, rb=0, shared=False),
+    "shared_3bit_res": dict(pb=4, rb=3, shared=True),
+    "5+3shared": dict(pb=5, rb=3, shared=True),
+    "5+3dual": dict(pb=5, rb=3, shared=False),
+    "5+0": dict(pb=5, rb=0, shared=False),
+}
+SHAPES = [(64, 128, 128), (32, 128, 128), (16, 512, 256), (24, 384, 128), (16, 256, 256), (16, 896, 128),
+          (7, 2048, 512), (5, 4096, 512), (3, 5120, 512), (2, 18944, 512), (9, 64, 32), (4, 64, 16)]
+
+
+def _make(oracle, out, inf, bs, mode, seed=42, fitted=False):
+    m = MODES[mode]
+    w = oracle.lcg_matrix(out, inf, seed) if out * inf <= 1 << 16 else \
+        np.random.default_rng(seed).standard_normal((out, inf)).astype(np.float32) * 0.02
+    cbp = oracle.generate_codebook(m["pb"])
+    cbr = oracle.generate_codebook(m["rb"] if m["rb"] else 4)
+    if fitted:
+        cbp, cbr = oracle.fit_layer_codebooks(w, bs, m["pb"], m["rb"])
+    qw = oracle.quantize_weight(w, cbp, cbr, m["pb"], m["rb"], bs, m["shared"])
+    return qw, cbp, cbr
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("out,inf,bs", SHAPES)
+def test_dequantize_bit_exact(tq, oracle, mode, out, inf, bs):
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    got = tq.dequantize_weight_gpu(qw, cbp, cbr, bs)
+    want = oracle.dequantize_weight_cpu(qw, cbp, cbr, bs)
+    assert got.dtype == np.float32 and got.shape == (out, inf)
+    assert np.array_equal(got, want)
+
+
+def test_dequantize_fitted_codebooks_and_index_clamp(tq, oracle):
+    qw, cbp, cbr = _make(oracle, 48, 1024, 512, "shared", fitted=True)
+    assert np.array_equal(tq.dequantize_weight_gpu(qw, cbp, cbr, 512), oracle.dequantize_weight_cpu(qw, cbp, cbr, 512))
+    # 3-bit codebooks with 4-bit index planes: dual path clamps, LUT path zero-fills (src/dequantizer.cpp:94,144-150)
+    cb3 = oracle.generate_codebook(3)
+    rng = np.random.default_rng(0)
+    for seeds1 in (0, 1234):
+        q = oracle.QuantizedWeight(rng.integers(0, 256, (8, 256), dtype=np.uint8), rng.integers(0, 256, (8, 256), dtype=np.uint8),
+                                   rng.random(8, dtype=np.float32) + 0.5, np.array([99, seeds1, 128], np.uint32))
+        assert np.array_equal(tq.dequantize_weight_gpu(q, cb3, cb3, 128), oracle.dequantize_weight_cpu(q, cb3, cb3, 128))
+
+
+# ------------------------------------------------------------------ forward
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only", "shared_3bit_res"])
+@pytest.mark.parametrize("out,inf,bs", [(64, 128, 128), (32, 128, 128), (16, 512, 256), (24, 384, 128), (16, 896, 128),
+                                        (37, 2048, 512), (130, 4096, 512), (33, 5120, 512), (21, 3584, 512),
+                                        (9, 18944, 512), (5, 27648, 512), (9, 64, 32), (6, 64, 16)])
+@pytest.mark.parametrize("batch", [1, 2, 3, 4, 8])
+def test_forward_fp32(tq, oracle, mode, out, inf, bs, batch):
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    x = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    assert layer.in_features() == inf and layer.out_features() == out
+    y = layer.forward(x)
+    layer.close()
+    assert y.shape == (batch, out) and y.dtype == np.float32
+    want = oracle.linear_forward(qw, cbp, cbr, bs, x)
+    assert _rel(y, want) < 1e-3
+    assert np.abs(y - want).max() < 0.15                     # the reference's own bound, test_linear.cpp:135
+
+
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("xd", ["bf16", "f16"])
+@pytest.mark.parametrize("yd", ["f32", "bf16", "f16"])
+def test_forward_half_activations(tq, oracle, mode, xd, yd):
+    out, inf, bs, batch = 96, 2048, 512, 3
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    x32 = np.random.default_rng(5).standard_normal((batch, inf)).astype(np.float32)
+    if xd == "bf16":
+        xbits = oracle.f32_to_bf16_bits(x32); xin = oracle.bf16_bits_to_f32(xbits); xarg, xcode = xbits, tq.BF16
+    else:
+        xarg = x32.astype(np.float16); xin = xarg.astype(np.float32); xcode = tq.F16
+    ycode = {"f32": tq.F32, "bf16": tq.BF16, "f16": tq.F16}[yd]
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    y = layer.forward(xarg, xcode, ycode)
+    layer.close()
+    if yd == "bf16":
+        y = oracle.bf16_bits_to_f32(y)
+    y = y.astype(np.float32)
+    want = oracle.linear_forward(qw, cbp, cbr, bs, xin)
+    assert _rel(y, want) < 5e-3
+
+
+def test_forward_fitted_codebooks_match_dequant_matmul(tq, oracle):
+    qw, cbp, cbr = _make(oracle, 200, 2048, 512, "shared", fitted=True)
+    x = np.random.default_rng(1).standard_normal((1, 2048)).astype(np.float32)
+    y = tq.fused_dequant_matmul(qw, cbp, cbr, 512, x)
+    assert _rel(y, oracle.linear_forward(qw, cbp, cbr, 512, x)) < 1e-3
+
+
+def test_error_conventions(tq, oracle):
+    L = tq.lib()
+    assert L.tq_linear_in_features(None) == 0 and L.tq_linear_out_features(None) == 0
+    L.tq_linear_free(None)                                   # no-op
+    assert L.tq_linear_forward(None, None, 0, 1, None, 0, None) != 0
+    qw, cbp, cbr = _make(oracle, 8, 128, 128, "shared")
+    with pytest.raises(ValueError):
+        tq.TurboQuantLinear(256, 8, qw, cbp, cbr, 128)       # shape mismatch
+    with pytest.raises(ValueError):
+        tq.TurboQuantLinear(128, 8, qw, cbp, cbr, 96)        # block size does not divide
+    q5, c5, c3 = _make(oracle, 8, 128, 128, "5+3shared")
+    layer = tq.TurboQuantLinear(128, 8, q5, c5, c3, 128)
+    with pytest.raises(RuntimeError):
+        layer.forward(np.zeros((1, 128), np.float32))        # 5-bit: dequantise only
+    layer.close()

@@ -1,0 +1,189 @@
+"""Python binding (ctypes) of libturboquant_amd.so, the gfx950 TQ8 linear path.
+
+The names mirror the reference's C++ API for this path
+(include/turboquant/linear.h:11-35, include/turboquant/dequantizer.h:11-39,
+include/turboquant/quantizer.h:22-42).  Everything computes on the GPU through
+the C-ABI in include/turboquant_c/tq_linear.h; there is no CPU fallback, and a
+missing library is an ImportError-like RuntimeError, never a silent substitute.
+
+The directory name is not a Python identifier; load it with
+``importlib`` (see ``__graft_entry__.load_package``) under the module name
+``turboquant_mlx_core_amd``.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libturboquant_amd.so")
+
+F32, F16, BF16 = 0, 1, 2
+MODE_NAMES = {0: "primary_only", 1: "shared_lut", 2: "dual", 3: "shared_5bit",
+              4: "primary_only_5bit", 5: "dual_5bit"}
+
+_u8p = C.POINTER(C.c_uint8)
+_f32p = C.POINTER(C.c_float)
+_u32p = C.POINTER(C.c_uint32)
+_lib = None
+
+
+def build():
+    """Compile the HIP library in-tree (hipcc cross-compiles gfx950 without a GPU)."""
+    subprocess.check_call(["make", "-C", _HERE, "-B", "-j8"], stdout=subprocess.DEVNULL,
+                          stderr=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with `make -C {_HERE}`; "
+                               "there is no CPU fallback for the TQ8 linear path")
+        L = C.CDLL(LIB_PATH)
+        L.tq_last_error.restype = C.c_char_p
+        L.tq_linear_create.restype = C.c_void_p
+        L.tq_linear_create.argtypes = [C.c_int, C.c_int, _u8p, C.c_int, _u8p, C.c_int, _f32p, _u32p,
+                                       _f32p, C.c_int, _f32p, C.c_int, C.c_uint32]
+        L.tq_linear_create_from_device.restype = C.c_void_p
+        L.tq_linear_create_from_device.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                                   C.c_void_p, _u32p, _f32p, C.c_int, _f32p, C.c_int, C.c_uint32]
+        for name in ("tq_linear_in_features", "tq_linear_out_features", "tq_linear_mode"):
+            getattr(L, name).argtypes = [C.c_void_p]
+        L.tq_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
+        L.tq_linear_forward_host.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]
+        L.tq_linear_dequantize.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.tq_linear_dequantize_host.argtypes = [C.c_void_p, _f32p]
+        L.tq_linear_free.argtypes = [C.c_void_p]
+        L.tq_linear_free.restype = None
+        L.tq_wht_rotate.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_int, C.c_void_p]
+        L.tq_wht_rotate_host.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_int]
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().tq_last_error().decode()
+
+
+def _p(a, t):
+    return a.ctypes.data_as(t)
+
+
+_NP_DTYPE = {F32: np.float32, F16: np.float16, BF16: np.uint16}
+
+
+class TurboQuantLinear:
+    """Mirror of turboquant::TurboQuantLinear (include/turboquant/linear.h:11-35).
+
+    ``weights`` is any object with ``packed_primary``, ``packed_residual``, ``norms`` and
+    ``seeds`` numpy arrays (the reference's QuantizedWeight); codebooks are objects with a
+    ``centroids`` array.  bf16 arrays travel as uint16 bit patterns.
+    """
+
+    def __init__(self, in_features, out_features, weights, primary_codebook, residual_codebook, block_size):
+        pp = np.ascontiguousarray(weights.packed_primary, dtype=np.uint8)
+        pr = np.ascontiguousarray(weights.packed_residual, dtype=np.uint8)
+        norms = np.ascontiguousarray(weights.norms, dtype=np.float32)
+        seeds = np.ascontiguousarray(weights.seeds, dtype=np.uint32)
+        cp = np.ascontiguousarray(primary_codebook.centroids, dtype=np.float32)
+        cr = np.ascontiguousarray(residual_codebook.centroids, dtype=np.float32)
+        if pp.ndim != 2 or pr.ndim != 2 or pp.shape[0] != out_features or pr.shape[0] != out_features:
+            raise ValueError("packed tensors must be [out_features, cols]")
+        self._h = lib().tq_linear_create(in_features, out_features, _p(pp, _u8p), pp.shape[1], _p(pr, _u8p),
+                                         pr.shape[1], _p(norms, _f32p), _p(seeds, _u32p), _p(cp, _f32p), len(cp),
+                                         _p(cr, _f32p), len(cr), block_size)
+        if not self._h:
+            raise ValueError(last_error())
+
+    def in_features(self):
+        return lib().tq_linear_in_features(self._h)
+
+    def out_features(self):
+        return lib().tq_linear_out_features(self._h)
+
+    def mode(self):
+        return MODE_NAMES[lib().tq_linear_mode(self._h)]
+
+    def forward(self, x, x_dtype=F32, y_dtype=F32):
+        """x: numpy [batch, in] (float32, float16, or uint16 bf16 bits) -> numpy [batch, out]."""
+        x = np.ascontiguousarray(x, dtype=_NP_DTYPE[x_dtype])
+        if x.ndim != 2 or x.shape[1] != self.in_features():
+            raise ValueError("input must be [batch, in_features]")
+        y = np.empty((x.shape[0], self.out_features()), dtype=_NP_DTYPE[y_dtype])
+        rc = lib().tq_linear_forward_host(self._h, x.ctypes.data, x_dtype, x.shape[0], y.ctypes.data, y_dtype)
+        if rc != 0:
+            raise RuntimeError(last_error())
+        return y
+
+    def forward_device(self, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream=None):
+        """Asynchronous forward on raw device pointers (e.g. torch ``data_ptr()``)."""
+        rc = lib().tq_linear_forward(self._h, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream)
+        if rc != 0:
+            raise RuntimeError(last_error())
+
+    def dequantize(self):
+        """dequantize_weight_gpu: float32 [out, in]."""
+        w = np.empty((self.out_features(), self.in_features()), dtype=np.float32)
+        if lib().tq_linear_dequantize_host(self._h, _p(w, _f32p)) != 0:
+            raise RuntimeError(last_error())
+        return w
+
+    def dequantize_device(self, w_ptr, stream=None):
+        if lib().tq_linear_dequantize(self._h, w_ptr, stream) != 0:
+            raise RuntimeError(last_error())
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().tq_linear_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def fused_dequant_matmul(qw, primary_codebook, residual_codebook, block_size, x, x_dtype=F32, y_dtype=F32):
+    """Mirror of turboquant::fused_dequant_matmul (include/turboquant/dequantizer.h:33-39)."""
+    out = qw.packed_primary.shape[0]
+    inf = qw.packed_residual.shape[1] * 2
+    layer = TurboQuantLinear(inf, out, qw, primary_codebook, residual_codebook, block_size)
+    try:
+        return layer.forward(x, x_dtype, y_dtype)
+    finally:
+        layer.close()
+
+
+def dequantize_weight_gpu(qw, primary_codebook, residual_codebook, block_size):
+    """Mirror of turboquant::dequantize_weight_gpu (include/turboquant/dequantizer.h:19-25)."""
+    out = qw.packed_primary.shape[0]
+    inf = qw.packed_residual.shape[1] * 2
+    layer = TurboQuantLinear(inf, out, qw, primary_codebook, residual_codebook, block_size)
+    try:
+        return layer.dequantize()
+    finally:
+        layer.close()
+
+
+def _rotate(matrix, seed, block_size, inverse):
+    m = np.ascontiguousarray(matrix, dtype=np.float32)
+    if m.ndim != 2:
+        raise ValueError("matrix must be 2-D")
+    out = np.empty_like(m)
+    rc = lib().tq_wht_rotate_host(_p(m, _f32p), _p(out, _f32p), m.shape[0], m.shape[1], seed, block_size, inverse)
+    if rc != 0:
+        raise ValueError(last_error())
+    return out
+
+
+def apply_wht_rotation(matrix, seed, block_size):
+    """Mirror of turboquant::apply_wht_rotation (include/turboquant/quantizer.h:31-35)."""
+    return _rotate(matrix, seed, block_size, 0)
+
+
+def apply_inverse_wht_rotation(matrix, seed, block_size):
+    """Mirror of turboquant::apply_inverse_wht_rotation (include/turboquant/quantizer.h:37-42)."""
+    return _rotate(matrix, seed, block_size, 1)

@@ -1,0 +1,197 @@
+// Materialising dequantiser and stand-alone block rotation for gfx950.
+//
+// tq_dequant_kernel rebuilds the fp32 weight [out, in] from the packed indices and
+// follows the reference CPU dequantiser operation by operation
+// (src/dequantizer.cpp:52-256 with the inverse rotation of src/rotation.cpp:323-350):
+// lookup, * 1/sqrt(in), butterfly, * (1/sqrt(bs) * sign), [+ residual plane], * norm.
+// Every step is a single fp32 operation in the reference's order (this file is
+// compiled with -ffp-contract=off), so the output is bit-identical to the CPU path.
+//
+// One wave handles one (row, 2048-column slab); a lane owns 32 consecutive columns.
+#include "tq_device.h"
+
+namespace tq {
+
+constexpr int kDqWaves = 4;   // waves per workgroup
+
+__device__ __forceinline__ void unpack_nibbles(const uint4& P, uint32_t (&idx)[kChunk]) {
+    const uint32_t w[4] = {P.x, P.y, P.z, P.w};
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t byte = (w[d] >> (8 * j)) & 0xffu;
+            idx[8 * d + 2 * j]     = byte & 0x0fu;   // lo nibble = even column (src/dequantizer.cpp:46)
+            idx[8 * d + 2 * j + 1] = byte >> 4;      // hi nibble = odd column  (src/dequantizer.cpp:47)
+        }
+}
+
+__global__ __launch_bounds__(kDqWaves* kWave) void tq_dequant_kernel(LayerView L, float* __restrict__ Wout,
+                                                                      int chunks, int slabs) {
+    __shared__ float tab[256];
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) tab[i] = L.tables[i];
+    __syncthreads();
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const long long wid = (long long)blockIdx.x * kDqWaves + (threadIdx.x >> 6);
+    const int row = (int)(wid / slabs);
+    const int slab = (int)(wid % slabs);
+    if (row >= L.out_features) return;          // whole wave leaves together
+    const int chunk = slab * kWave + lane;
+    const bool active = chunk < chunks;
+    const int in = L.in_features;
+    const uint32_t bs = L.block_size;
+    const bool five = (L.mode >= kShared5);
+    const bool has_res = (L.mode != kPrimaryOnly && L.mode != kPrimaryOnly5);
+    const bool shared = (L.mode == kSharedLut || L.mode == kShared5);
+
+    uint32_t pi[kChunk], ri[kChunk];
+    float v[kChunk];
+    if (active) {
+        if (five) {
+            const uint4* p = reinterpret_cast<const uint4*>(L.packed_primary + (size_t)row * in + (size_t)chunk * 32);
+            const uint4 a = p[0], b = p[1];
+            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int d = 0; d < 8; ++d)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) pi[4 * d + j] = (w[d] >> (8 * j)) & 0xffu;
+        } else {
+            unpack_nibbles(*reinterpret_cast<const uint4*>(L.packed_primary + (size_t)row * (in >> 1) + (size_t)chunk * 16), pi);
+        }
+        if (has_res)
+            unpack_nibbles(*reinterpret_cast<const uint4*>(L.packed_residual + (size_t)row * (in >> 1) + (size_t)chunk * 16), ri);
+    }
+
+    const uint32_t col0 = ((uint32_t)chunk * kChunk) & (bs - 1);
+    const float nrm = L.norms[row];
+
+    if (L.mode == kSharedLut) {
+        // path A: 256-entry table of centroid sums (src/dequantizer.cpp:136-184)
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) v[k] = active ? tab[(ri[k] << 4) | pi[k]] * L.inv_scale : 0.0f;
+    } else {
+        const int roff = five ? 32 : 16;
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) {
+            float c = 0.0f;
+            if (active) {
+                c = tab[five ? (pi[k] > 31u ? 31u : pi[k]) : pi[k]];
+                if (shared) c = c + tab[roff + ri[k]];       // path B (src/dequantizer.cpp:186-212)
+            }
+            v[k] = c * L.inv_scale;
+        }
+    }
+    fwht_lane32(v, bs, lane);
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) v[k] *= L.inv_sqrt_bs * sign_of(L.seed_primary, (col0 + k) & (bs - 1));
+
+    if (has_res && !shared) {
+        // path C second plane (src/dequantizer.cpp:220-245)
+        const int roff = five ? 32 : 16;
+        float u[kChunk];
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) u[k] = active ? tab[roff + ri[k]] * L.inv_scale : 0.0f;
+        fwht_lane32(u, bs, lane);
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) {
+            u[k] *= L.inv_sqrt_bs * sign_of(L.seed_residual, (col0 + k) & (bs - 1));
+            v[k] = v[k] + u[k];
+        }
+    }
+
+    if (active) {
+        float4* dst = reinterpret_cast<float4*>(Wout + (size_t)row * in + (size_t)chunk * kChunk);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            dst[i] = make_float4(v[4 * i] * nrm, v[4 * i + 1] * nrm, v[4 * i + 2] * nrm, v[4 * i + 3] * nrm);
+    }
+}
+
+hipError_t launch_dequant(const LayerView& L, float* w, hipStream_t stream) {
+    const int chunks = L.in_features / kChunk;
+    const int slabs = (chunks + kWave - 1) / kWave;
+    const long long waves = (long long)L.out_features * slabs;
+    const long long grid = (waves + kDqWaves - 1) / kDqWaves;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(tq_dequant_kernel, dim3((unsigned)grid), dim3(kDqWaves * kWave), 0, stream, L, w, chunks, slabs);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Block rotation of an fp32 matrix (reference src/rotation.cpp:291-350).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kDqWaves* kWave) void tq_wht_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                                  int rows, int cols, int chunks, int slabs,
+                                                                  uint32_t seed, uint32_t bs, float inv_sqrt_bs,
+                                                                  int inverse) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const long long wid = (long long)blockIdx.x * kDqWaves + (threadIdx.x >> 6);
+    const int row = (int)(wid / slabs);
+    const int slab = (int)(wid % slabs);
+    if (row >= rows) return;
+    const int chunk = slab * kWave + lane;
+    const bool active = chunk < chunks;
+    const uint32_t col0 = ((uint32_t)chunk * kChunk) & (bs - 1);
+
+    float v[kChunk];
+    if (active) {
+        load_chunk(in, kF32, (size_t)row * cols + (size_t)chunk * kChunk, v);
+    } else {
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) v[k] = 0.0f;
+    }
+    if (!inverse) {
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) v[k] *= sign_of(seed, (col0 + k) & (bs - 1));
+    }
+    fwht_lane32(v, bs, lane);
+    if (!inverse) {
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) v[k] *= inv_sqrt_bs;
+    } else {
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) v[k] *= inv_sqrt_bs * sign_of(seed, (col0 + k) & (bs - 1));
+    }
+    if (active) {
+        float4* dst = reinterpret_cast<float4*>(out + (size_t)row * cols + (size_t)chunk * kChunk);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dst[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+    }
+}
+
+hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t seed,
+                      uint32_t block_size, float inv_sqrt_bs, int inverse, hipStream_t stream) {
+    const int chunks = cols / kChunk;
+    const int slabs = (chunks + kWave - 1) / kWave;
+    const long long waves = (long long)rows * slabs;
+    const long long grid = (waves + kDqWaves - 1) / kDqWaves;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(tq_wht_kernel, dim3((unsigned)grid), dim3(kDqWaves * kWave), 0, stream,
+                       in, out, rows, cols, chunks, slabs, seed, block_size, inv_sqrt_bs, inverse);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// "Does the residual plane hold any non-zero byte" (src/dequantizer.cpp:118-128)
+// for tensors that already live on the GPU.
+// ---------------------------------------------------------------------------
+__global__ void tq_any_nonzero_kernel(const uint8_t* __restrict__ data, size_t n, int* flag) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint32_t acc = 0;
+    const size_t n16 = n / 16;
+    const uint4* p = reinterpret_cast<const uint4*>(data);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) {
+        const uint4 t = p[i];
+        acc |= t.x | t.y | t.z | t.w;
+    }
+    for (size_t i = n16 * 16 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) acc |= data[i];
+    if (acc) atomicOr(flag, 1);
+}
+
+hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream) {
+    hipLaunchKernelGGL(tq_any_nonzero_kernel, dim3(1024), dim3(256), 0, stream, data, n, flag_dev);
+    return hipGetLastError();
+}
+
+}  // namespace tq

@@ -1,0 +1,146 @@
+// Internal declarations shared by the gfx950 kernels and the C-ABI layer.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tq {
+
+// Activation / output element types (same numbering as TQ_DTYPE_* in tq_linear.h).
+enum : int { kF32 = 0, kF16 = 1, kBF16 = 2 };
+
+// Decode modes (same numbering as TQ_MODE_* in tq_linear.h).
+enum : int {
+    kPrimaryOnly = 0, kSharedLut = 1, kDual = 2,
+    kShared5 = 3, kPrimaryOnly5 = 4, kDual5 = 5
+};
+
+constexpr int kWave = 64;          // gfx950 wavefront width
+constexpr int kChunk = 32;         // columns owned by one lane (16 packed bytes)
+constexpr int kSlab = kWave * kChunk;   // columns covered by one wave
+
+// Device-side description of one TQ8 layer.
+struct LayerView {
+    const uint8_t* packed_primary;   // [out, in/2] nibble pairs (or [out, in] bytes for 5-bit)
+    const uint8_t* packed_residual;  // [out, in/2]
+    const float*   norms;            // [out]
+    const float*   tables;           // decode tables, layout depends on mode (see build_tables)
+    int out_features;
+    int in_features;
+    uint32_t block_size;
+    uint32_t seed_primary;
+    uint32_t seed_residual;
+    int mode;
+    float inv_scale;                 // 1/sqrt(in), computed on the host as the reference does
+    float inv_sqrt_bs;               // 1/sqrt(block_size), host computed
+};
+
+// Launchers (tq_gemv.hip, tq_dequant.hip).  All return hipError_t of the launch.
+hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch,
+                       void* y, int y_dtype, int num_cus, hipStream_t stream);
+hipError_t launch_dequant(const LayerView& L, float* w, hipStream_t stream);
+hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t seed,
+                      uint32_t block_size, float inv_sqrt_bs, int inverse, hipStream_t stream);
+hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream);
+
+// True when the fast wave-per-slab kernels can handle this shape.
+inline bool shape_supported(int in_features, uint32_t block_size) {
+    if (in_features <= 0 || in_features % kChunk != 0) return false;
+    if (block_size < 2 || block_size > 2048 || (block_size & (block_size - 1))) return false;
+    if (in_features % (int)block_size != 0) return false;
+    if (in_features > 16 * kSlab) return false;
+    return true;
+}
+
+// ---------------------------------------------------------------------------
+// Device helpers
+// ---------------------------------------------------------------------------
+
+// +-1 from a u32 hash of (seed, index inside the block); reference
+// src/rotation.cpp:32-42 and metal/turboquant_dequant_mm.metal:57-61.
+__device__ __forceinline__ float sign_of(uint32_t seed, uint32_t index) {
+    uint32_t h = seed * 2654435761u + index * 2246822519u;
+    h ^= h >> 16;
+    h *= 0x45d9f3bu;
+    h ^= h >> 16;
+    return (h & 1u) ? 1.0f : -1.0f;
+}
+
+// Unnormalised natural-order Walsh-Hadamard butterfly over a block that is
+// spread as 32 consecutive values per lane over bs/32 neighbouring lanes
+// (or lives entirely inside the lane when bs <= 32).  Stage order and the
+// (a+b, a-b) convention are those of reference src/rotation.cpp:14-25, so the
+// result is bit-identical to the CPU butterfly.
+__device__ __forceinline__ void fwht_lane32(float (&v)[kChunk], uint32_t bs, int lane) {
+#pragma unroll
+    for (int h = 1; h < kChunk; h <<= 1) {
+        if ((uint32_t)h < bs) {
+#pragma unroll
+            for (int i = 0; i < kChunk; i += 2 * h) {
+#pragma unroll
+                for (int j = i; j < i + h; ++j) {
+                    float a = v[j], b = v[j + h];
+                    v[j] = a + b;
+                    v[j + h] = a - b;
+                }
+            }
+        }
+    }
+    for (uint32_t m = 1; m * kChunk < bs; m <<= 1) {
+        const bool upper = (lane & (int)m) != 0;
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) {
+            float p = __shfl_xor(v[k], (int)m, kWave);
+            v[k] = upper ? (p - v[k]) : (v[k] + p);
+        }
+    }
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) {
+    return __builtin_bit_cast(float, b << 16);
+}
+
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// Load the 32 consecutive activations a lane owns and widen them to fp32.
+__device__ __forceinline__ void load_chunk(const void* base, int dtype, size_t elem_offset,
+                                           float (&v)[kChunk]) {
+    if (dtype == kF32) {
+        const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(base) + elem_offset);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float4 t = p[i];
+            v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+        }
+    } else {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + elem_offset);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4 t = p[i];
+            uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (dtype == kBF16) {
+                    v[8 * i + 2 * j]     = bf16_bits_to_float(w[j] & 0xffffu);
+                    v[8 * i + 2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+                } else {
+                    v[8 * i + 2 * j]     = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] & 0xffffu));
+                    v[8 * i + 2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] >> 16));
+                }
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void store_scalar(void* base, int dtype, size_t idx, float v) {
+    if (dtype == kF32) static_cast<float*>(base)[idx] = v;
+    else if (dtype == kBF16) static_cast<uint16_t*>(base)[idx] = float_to_bf16_bits(v);
+    else static_cast<_Float16*>(base)[idx] = (_Float16)v;
+}
+
+}  // namespace tq

@@ -1,0 +1,306 @@
+// C-ABI of the TQ8 linear path (declared in include/turboquant_c/tq_linear.h).
+// Host-side logic only: argument checks, mode inference exactly as the reference
+// does it (src/dequantizer.cpp:72-75,118-133,674-675), decode-table construction,
+// device buffer ownership and kernel dispatch.  Nothing here computes on the CPU:
+// a missing GPU or a failed HIP call is reported as an error.
+#include "turboquant_c/tq_linear.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "tq_device.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+void set_error(const std::string& msg) { g_last_error = msg; }
+
+bool hip_ok(hipError_t e, const char* what) {
+    if (e == hipSuccess) return true;
+    set_error(std::string(what) + ": " + hipGetErrorString(e));
+    return false;
+}
+
+int device_cu_count() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+size_t dtype_size(int dt) { return dt == TQ_DTYPE_F32 ? 4 : 2; }
+bool dtype_valid(int dt) { return dt == TQ_DTYPE_F32 || dt == TQ_DTYPE_F16 || dt == TQ_DTYPE_BF16; }
+
+}  // namespace
+
+struct tq_linear_s {
+    tq::LayerView view{};
+    uint8_t* d_primary = nullptr;
+    uint8_t* d_residual = nullptr;
+    float* d_norms = nullptr;
+    float* d_tables = nullptr;
+    int primary_cols = 0;
+    int residual_cols = 0;
+    // Staging for the *_host entry points, grown on demand.
+    void* d_stage_x = nullptr; size_t stage_x_bytes = 0;
+    void* d_stage_y = nullptr; size_t stage_y_bytes = 0;
+
+    ~tq_linear_s() {
+        if (d_primary) (void)hipFree(d_primary);
+        if (d_residual) (void)hipFree(d_residual);
+        if (d_norms) (void)hipFree(d_norms);
+        if (d_tables) (void)hipFree(d_tables);
+        if (d_stage_x) (void)hipFree(d_stage_x);
+        if (d_stage_y) (void)hipFree(d_stage_y);
+    }
+};
+
+namespace {
+
+// Decode tables as 256 floats.
+//   shared 4-bit : lut[(r << 4) | p] = cP[p] + cR[r], zero where p >= n_primary
+//                  (src/dequantizer.cpp:144-150, 669-688)
+//   other 4-bit  : [0..15] primary, [16..31] residual, index clamped to the last
+//                  centroid (src/dequantizer.cpp:94,103,229)
+//   5-bit primary: [0..31] primary, [32..47] residual, clamped likewise
+void build_tables(int mode, const float* cbp, int np, const float* cbr, int nr, float* t) {
+    std::memset(t, 0, 256 * sizeof(float));
+    if (mode == tq::kSharedLut) {
+        for (int r = 0; r < 16; ++r)
+            for (int p = 0; p < np && p < 16; ++p)
+                t[(r << 4) | p] = cbp[p] + cbr[r < nr ? r : nr - 1];
+        return;
+    }
+    const bool five = mode >= tq::kShared5;
+    const int pn = five ? 32 : 16;
+    for (int i = 0; i < pn; ++i) t[i] = cbp[i < np ? i : np - 1];
+    for (int i = 0; i < 16; ++i) t[pn + i] = cbr[i < nr ? i : nr - 1];
+}
+
+bool ensure_stage(void** buf, size_t* have, size_t need) {
+    if (*have >= need) return true;
+    if (*buf) { (void)hipFree(*buf); *buf = nullptr; *have = 0; }
+    if (!hip_ok(hipMalloc(buf, need), "hipMalloc(staging)")) return false;
+    *have = need;
+    return true;
+}
+
+tq_linear_t create_impl(int in_features, int out_features,
+                        const uint8_t* pp, int primary_cols,
+                        const uint8_t* pr, int residual_cols,
+                        const float* norms, const uint32_t* seeds,
+                        const float* cbp, int np, const float* cbr, int nr,
+                        uint32_t block_size, bool from_device) {
+    if (!pp || !pr || !norms || !seeds || !cbp || !cbr) { set_error("tq_linear_create: NULL argument"); return nullptr; }
+    if (in_features <= 0 || out_features <= 0 || np <= 0 || nr <= 0 || np > 32 || nr > 16) {
+        set_error("tq_linear_create: bad dimensions"); return nullptr;
+    }
+    // Shape inference as the reference does it (src/dequantizer.cpp:72-75).
+    const bool five = (primary_cols == residual_cols * 2);
+    const int in_inferred = five ? primary_cols : primary_cols * 2;
+    if (in_inferred != in_features || residual_cols * 2 != in_features) {
+        set_error("tq_linear_create: packed shapes do not match in_features"); return nullptr;
+    }
+    if (block_size == 0 || in_features % (int)block_size != 0) {
+        set_error("tq_linear_create: in_features must be divisible by block_size"); return nullptr;
+    }
+    if (!tq::shape_supported(in_features, block_size)) {
+        set_error("tq_linear_create: unsupported shape (need in_features % 32 == 0, in_features <= 32768, "
+                  "power-of-two block_size in [2, 2048])");
+        return nullptr;
+    }
+
+    tq_linear_s* h = new (std::nothrow) tq_linear_s();
+    if (!h) { set_error("tq_linear_create: out of host memory"); return nullptr; }
+    const size_t pbytes = (size_t)out_features * primary_cols;
+    const size_t rbytes = (size_t)out_features * residual_cols;
+    const hipMemcpyKind kind = from_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice;
+    bool ok = hip_ok(hipMalloc((void**)&h->d_primary, pbytes), "hipMalloc(packed_primary)") &&
+              hip_ok(hipMalloc((void**)&h->d_residual, rbytes), "hipMalloc(packed_residual)") &&
+              hip_ok(hipMalloc((void**)&h->d_norms, (size_t)out_features * sizeof(float)), "hipMalloc(norms)") &&
+              hip_ok(hipMalloc((void**)&h->d_tables, 256 * sizeof(float)), "hipMalloc(tables)") &&
+              hip_ok(hipMemcpy(h->d_primary, pp, pbytes, kind), "copy packed_primary") &&
+              hip_ok(hipMemcpy(h->d_residual, pr, rbytes, kind), "copy packed_residual") &&
+              hip_ok(hipMemcpy(h->d_norms, norms, (size_t)out_features * sizeof(float), kind), "copy norms");
+    if (!ok) { delete h; return nullptr; }
+
+    // Residual presence: any non-zero byte (src/dequantizer.cpp:118-128).
+    bool has_residual = false;
+    if (from_device) {
+        int* d_flag = nullptr; int flag = 0;
+        ok = hip_ok(hipMalloc((void**)&d_flag, sizeof(int)), "hipMalloc(flag)") &&
+             hip_ok(hipMemset(d_flag, 0, sizeof(int)), "hipMemset(flag)") &&
+             hip_ok(tq::launch_any_nonzero(h->d_residual, rbytes, d_flag, nullptr), "any_nonzero") &&
+             hip_ok(hipMemcpy(&flag, d_flag, sizeof(int), hipMemcpyDeviceToHost), "copy flag");
+        if (d_flag) (void)hipFree(d_flag);
+        if (!ok) { delete h; return nullptr; }
+        has_residual = flag != 0;
+    } else {
+        for (size_t i = 0; i < rbytes; ++i) if (pr[i] != 0) { has_residual = true; break; }
+    }
+    const bool shared = (seeds[1] == 0 && has_residual);          // src/dequantizer.cpp:133
+    int mode;
+    if (!has_residual) mode = five ? tq::kPrimaryOnly5 : tq::kPrimaryOnly;
+    else if (shared)   mode = five ? tq::kShared5 : tq::kSharedLut;
+    else               mode = five ? tq::kDual5 : tq::kDual;
+
+    float tables[256];
+    build_tables(mode, cbp, np, cbr, nr, tables);
+    if (!hip_ok(hipMemcpy(h->d_tables, tables, sizeof(tables), hipMemcpyHostToDevice), "copy tables")) {
+        delete h; return nullptr;
+    }
+
+    h->primary_cols = primary_cols;
+    h->residual_cols = residual_cols;
+    tq::LayerView& v = h->view;
+    v.packed_primary = h->d_primary;
+    v.packed_residual = h->d_residual;
+    v.norms = h->d_norms;
+    v.tables = h->d_tables;
+    v.out_features = out_features;
+    v.in_features = in_features;
+    v.block_size = block_size;
+    v.seed_primary = seeds[0];
+    v.seed_residual = seeds[1];
+    v.mode = mode;
+    v.inv_scale = 1.0f / std::sqrt(static_cast<float>(in_features));      // src/dequantizer.cpp:76
+    v.inv_sqrt_bs = 1.0f / std::sqrt(static_cast<float>(block_size));     // src/rotation.cpp:333
+    return h;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* tq_last_error(void) { return g_last_error.c_str(); }
+
+tq_linear_t tq_linear_create(int in_features, int out_features,
+                             const uint8_t* packed_primary_host, int primary_cols,
+                             const uint8_t* packed_residual_host, int residual_cols,
+                             const float* norms_host, const uint32_t* seeds_host,
+                             const float* cb_primary_host, int n_primary,
+                             const float* cb_residual_host, int n_residual,
+                             uint32_t block_size) {
+    try {
+        return create_impl(in_features, out_features, packed_primary_host, primary_cols,
+                           packed_residual_host, residual_cols, norms_host, seeds_host,
+                           cb_primary_host, n_primary, cb_residual_host, n_residual, block_size, false);
+    } catch (...) { set_error("tq_linear_create: exception"); return nullptr; }
+}
+
+tq_linear_t tq_linear_create_from_device(int in_features, int out_features,
+                             const uint8_t* packed_primary_dev, int primary_cols,
+                             const uint8_t* packed_residual_dev, int residual_cols,
+                             const float* norms_dev, const uint32_t* seeds_host,
+                             const float* cb_primary_host, int n_primary,
+                             const float* cb_residual_host, int n_residual,
+                             uint32_t block_size) {
+    try {
+        return create_impl(in_features, out_features, packed_primary_dev, primary_cols,
+                           packed_residual_dev, residual_cols, norms_dev, seeds_host,
+                           cb_primary_host, n_primary, cb_residual_host, n_residual, block_size, true);
+    } catch (...) { set_error("tq_linear_create_from_device: exception"); return nullptr; }
+}
+
+int tq_linear_in_features(tq_linear_t h) { return h ? h->view.in_features : 0; }
+int tq_linear_out_features(tq_linear_t h) { return h ? h->view.out_features : 0; }
+int tq_linear_mode(tq_linear_t h) { return h ? h->view.mode : 0; }
+
+int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
+                      void* y_dev, int y_dtype, void* stream) {
+    try {
+        if (!h || !x_dev || !y_dev) { set_error("tq_linear_forward: NULL argument"); return 1; }
+        if (batch <= 0 || !dtype_valid(x_dtype) || !dtype_valid(y_dtype)) {
+            set_error("tq_linear_forward: bad batch or dtype"); return 1;
+        }
+        if (h->view.mode >= tq::kShared5) {
+            set_error("tq_linear_forward: 5-bit primary is not supported by the fused kernels"); return 1;
+        }
+        return hip_ok(tq::launch_gemv(h->view, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(),
+                                      static_cast<hipStream_t>(stream)), "tq_gemv launch") ? 0 : 1;
+    } catch (...) { set_error("tq_linear_forward: exception"); return 1; }
+}
+
+int tq_linear_forward_host(tq_linear_t h, const void* x_host, int x_dtype, int batch,
+                           void* y_host, int y_dtype) {
+    try {
+        if (!h || !x_host || !y_host) { set_error("tq_linear_forward_host: NULL argument"); return 1; }
+        if (batch <= 0 || !dtype_valid(x_dtype) || !dtype_valid(y_dtype)) {
+            set_error("tq_linear_forward_host: bad batch or dtype"); return 1;
+        }
+        const size_t xb = (size_t)batch * h->view.in_features * dtype_size(x_dtype);
+        const size_t yb = (size_t)batch * h->view.out_features * dtype_size(y_dtype);
+        if (!ensure_stage(&h->d_stage_x, &h->stage_x_bytes, xb)) return 1;
+        if (!ensure_stage(&h->d_stage_y, &h->stage_y_bytes, yb)) return 1;
+        if (!hip_ok(hipMemcpy(h->d_stage_x, x_host, xb, hipMemcpyHostToDevice), "copy x")) return 1;
+        if (tq_linear_forward(h, h->d_stage_x, x_dtype, batch, h->d_stage_y, y_dtype, nullptr) != 0) return 1;
+        if (!hip_ok(hipMemcpy(y_host, h->d_stage_y, yb, hipMemcpyDeviceToHost), "copy y")) return 1;
+        return 0;
+    } catch (...) { set_error("tq_linear_forward_host: exception"); return 1; }
+}
+
+int tq_linear_dequantize(tq_linear_t h, float* w_dev, void* stream) {
+    try {
+        if (!h || !w_dev) { set_error("tq_linear_dequantize: NULL argument"); return 1; }
+        return hip_ok(tq::launch_dequant(h->view, w_dev, static_cast<hipStream_t>(stream)), "tq_dequant launch") ? 0 : 1;
+    } catch (...) { set_error("tq_linear_dequantize: exception"); return 1; }
+}
+
+int tq_linear_dequantize_host(tq_linear_t h, float* w_host) {
+    try {
+        if (!h || !w_host) { set_error("tq_linear_dequantize_host: NULL argument"); return 1; }
+        const size_t bytes = (size_t)h->view.out_features * h->view.in_features * sizeof(float);
+        float* d = nullptr;
+        if (!hip_ok(hipMalloc((void**)&d, bytes), "hipMalloc(weight)")) return 1;
+        bool ok = tq_linear_dequantize(h, d, nullptr) == 0 &&
+                  hip_ok(hipMemcpy(w_host, d, bytes, hipMemcpyDeviceToHost), "copy weight");
+        (void)hipFree(d);
+        return ok ? 0 : 1;
+    } catch (...) { set_error("tq_linear_dequantize_host: exception"); return 1; }
+}
+
+void tq_linear_free(tq_linear_t h) {
+    if (!h) return;
+    delete h;
+}
+
+int tq_wht_rotate(const float* in_dev, float* out_dev, int rows, int cols,
+                  uint32_t seed, uint32_t block_size, int inverse, void* stream) {
+    try {
+        if (!in_dev || !out_dev || rows <= 0 || cols <= 0) { set_error("tq_wht_rotate: bad argument"); return 1; }
+        if (block_size == 0 || cols % (int)block_size != 0) {
+            set_error("tq_wht_rotate: in_features must be divisible by block_size"); return 1;
+        }
+        if (!tq::shape_supported(cols, block_size)) { set_error("tq_wht_rotate: unsupported shape"); return 1; }
+        const float inv_sqrt_bs = 1.0f / std::sqrt(static_cast<float>(block_size));
+        return hip_ok(tq::launch_wht(in_dev, out_dev, rows, cols, seed, block_size, inv_sqrt_bs, inverse,
+                                     static_cast<hipStream_t>(stream)), "tq_wht launch") ? 0 : 1;
+    } catch (...) { set_error("tq_wht_rotate: exception"); return 1; }
+}
+
+int tq_wht_rotate_host(const float* in_host, float* out_host, int rows, int cols,
+                       uint32_t seed, uint32_t block_size, int inverse) {
+    try {
+        if (!in_host || !out_host || rows <= 0 || cols <= 0) { set_error("tq_wht_rotate_host: bad argument"); return 1; }
+        const size_t bytes = (size_t)rows * cols * sizeof(float);
+        float* d = nullptr;
+        if (!hip_ok(hipMalloc((void**)&d, bytes), "hipMalloc(matrix)")) return 1;
+        bool ok = hip_ok(hipMemcpy(d, in_host, bytes, hipMemcpyHostToDevice), "copy in") &&
+                  tq_wht_rotate(d, d, rows, cols, seed, block_size, inverse, nullptr) == 0 &&
+                  hip_ok(hipMemcpy(out_host, d, bytes, hipMemcpyDeviceToHost), "copy out");
+        (void)hipFree(d);
+        return ok ? 0 : 1;
+    } catch (...) { set_error("tq_wht_rotate_host: exception"); return 1; }
+}
+
+}  // extern "C"
