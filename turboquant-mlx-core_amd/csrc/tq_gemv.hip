@@ -29,30 +29,61 @@ struct GemvArgs {
     int W, S;        // slabs per row, row streams per workgroup
     int groups;      // ceil(out / R)
     int iters;       // uniform trip count: ceil(groups / (gridDim.x * S))
+    int share_x;     // rotate the activations once per workgroup and pass them through LDS
     float out_scale; // inv_scale * inv_sqrt_bs
 };
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 128-bit streaming load (weights are read exactly once).
+__device__ __forceinline__ uint4 load_stream16(const uint8_t* p) {
+    const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+
 template <int CTRL>
-__device__ __forceinline__ float dpp_add(float v) {
-    int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
-    return v + __builtin_bit_cast(float, moved);
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
 
-// Sum over the 64 lanes of a wave; the result is uniform.
-__device__ __forceinline__ float wave_sum(float v) {
-    v = dpp_add<0xB1>(v);    // quad_perm [1,0,3,2]
-    v = dpp_add<0x4E>(v);    // quad_perm [2,3,0,1]
-    v = dpp_add<0x141>(v);   // row_half_mirror
-    v = dpp_add<0x140>(v);   // row_mirror
-    int iv = __builtin_bit_cast(int, v);
-    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));
-    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));
-    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
-    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
-    return (r0 + r1) + (r2 + r3);
+// Value held by lane (lane ^ MASK).
+template <int MASK>
+__device__ __forceinline__ float lane_xor(float v) {
+    if constexpr (MASK == 1) return dpp_mov<0xB1>(v);        // quad_perm [1,0,3,2]
+    else if constexpr (MASK == 2) return dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (MASK == 8) return dpp_mov<0x128>(v);  // row_ror:8
+    else return __shfl_xor(v, MASK, kWave);
 }
 
-// LDS byte address of table entry `byte j of idx`, private column of this lane:
+// Transposed wave reduction of N per-lane partial sums (N a power of two <= 16):
+// afterwards lane l holds the sum over all 64 lanes of value (l % N).  Every
+// exchange step halves the number of live values, so the cost is about
+// N + log2(64) shuffles instead of N * log2(64).
+template <int N, int MASK>
+__device__ __forceinline__ float reduce_rec(float (&cur)[N], int lane) {
+    if constexpr (N == 1) {
+        float v = cur[0];
+        if constexpr (MASK <= 1) v += lane_xor<1>(v);
+        if constexpr (MASK <= 2) v += lane_xor<2>(v);
+        if constexpr (MASK <= 4) v += dpp_mov<0x124>(v);     // row_ror:4; with row_ror:8 below: l, l+4, l+8, l+12
+        if constexpr (MASK <= 8) v += lane_xor<8>(v);
+        if constexpr (MASK <= 16) v += lane_xor<16>(v);
+        v += lane_xor<32>(v);
+        return v;
+    } else {
+        float nxt[N / 2];
+        const bool up = (lane & MASK) != 0;
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            const float keep = up ? cur[2 * i + 1] : cur[2 * i];
+            const float give = up ? cur[2 * i] : cur[2 * i + 1];
+            nxt[i] = keep + lane_xor<MASK>(give);
+        }
+        return reduce_rec<N / 2, MASK * 2>(nxt, lane);
+    }
+}
+
+// LDS byte address of table entry `byte J of idx`, private column of this lane:
 // (entry << 8) | (lane << 2), built by one byte permute.
 template <int J>
 __device__ __forceinline__ uint32_t entry_addr(uint32_t idx_bytes, uint32_t laneoff) {
@@ -63,64 +94,51 @@ __device__ __forceinline__ float lds_f32(const char* lds, uint32_t byte_addr) {
     return *reinterpret_cast<const float*>(lds + byte_addr);
 }
 
-// One row, shared-rotation 4-bit mode: a single 256-entry table indexed by
-// (residual_nibble << 4) | primary_nibble  (reference src/dequantizer.cpp:144-169).
-template <int NB>
-__device__ __forceinline__ void row_lut256(const uint4& P, const uint4& Q, const float (&xt)[NB][kChunk],
-                                           float (&acc)[NB], const char* lds, uint32_t laneoff) {
+// Centroid values of the 32 columns a lane owns, from one 16-entry table
+// (TABLE_OFF selects it) or from the 256-entry sum table of shared rotation
+// (reference src/dequantizer.cpp:144-169: index = residual_nibble << 4 | primary_nibble).
+template <bool LUT256, int TABLE_OFF>
+__device__ __forceinline__ void lookup32(const uint4& P, const uint4& Q, const char* lds, uint32_t laneoff,
+                                         float (&val)[kChunk]) {
     const uint32_t pw[4] = {P.x, P.y, P.z, P.w};
     const uint32_t rw[4] = {Q.x, Q.y, Q.z, Q.w};
+    uint32_t ce[4], co[4];
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-        const uint32_t ce = ((rw[d] << 4) & 0xF0F0F0F0u) | (pw[d] & 0x0F0F0F0Fu);          // even columns
-        const uint32_t co = (rw[d] & 0xF0F0F0F0u) | ((pw[d] >> 4) & 0x0F0F0F0Fu);         // odd columns
-        float le[4], lo[4];
-        le[0] = lds_f32(lds, entry_addr<0>(ce, laneoff)); lo[0] = lds_f32(lds, entry_addr<0>(co, laneoff));
-        le[1] = lds_f32(lds, entry_addr<1>(ce, laneoff)); lo[1] = lds_f32(lds, entry_addr<1>(co, laneoff));
-        le[2] = lds_f32(lds, entry_addr<2>(ce, laneoff)); lo[2] = lds_f32(lds, entry_addr<2>(co, laneoff));
-        le[3] = lds_f32(lds, entry_addr<3>(ce, laneoff)); lo[3] = lds_f32(lds, entry_addr<3>(co, laneoff));
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                acc[b] = __builtin_fmaf(le[j], xt[b][8 * d + 2 * j], acc[b]);
-                acc[b] = __builtin_fmaf(lo[j], xt[b][8 * d + 2 * j + 1], acc[b]);
-            }
+        if constexpr (LUT256) {
+            ce[d] = ((rw[d] << 4) & 0xF0F0F0F0u) | (pw[d] & 0x0F0F0F0Fu);     // even columns
+            co[d] = (rw[d] & 0xF0F0F0F0u) | ((pw[d] >> 4) & 0x0F0F0F0Fu);    // odd columns
+        } else {
+            ce[d] = pw[d] & 0x0F0F0F0Fu;
+            co[d] = (pw[d] >> 4) & 0x0F0F0F0Fu;
         }
+    }
+    const char* tab = lds + TABLE_OFF;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        val[8 * d + 0] = lds_f32(tab, entry_addr<0>(ce[d], laneoff));
+        val[8 * d + 1] = lds_f32(tab, entry_addr<0>(co[d], laneoff));
+        val[8 * d + 2] = lds_f32(tab, entry_addr<1>(ce[d], laneoff));
+        val[8 * d + 3] = lds_f32(tab, entry_addr<1>(co[d], laneoff));
+        val[8 * d + 4] = lds_f32(tab, entry_addr<2>(ce[d], laneoff));
+        val[8 * d + 5] = lds_f32(tab, entry_addr<2>(co[d], laneoff));
+        val[8 * d + 6] = lds_f32(tab, entry_addr<3>(ce[d], laneoff));
+        val[8 * d + 7] = lds_f32(tab, entry_addr<3>(co[d], laneoff));
     }
 }
 
-// One row, one 16-entry table (primary or residual plane) at LDS offset TABLE_OFF.
-template <int NB, int TABLE_OFF>
-__device__ __forceinline__ void row_tab16(const uint4& P, const float (&xt)[NB][kChunk],
-                                          float (&acc)[NB], const char* lds, uint32_t laneoff) {
-    const uint32_t pw[4] = {P.x, P.y, P.z, P.w};
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        const uint32_t ce = pw[d] & 0x0F0F0F0Fu;
-        const uint32_t co = (pw[d] >> 4) & 0x0F0F0F0Fu;
-        float le[4], lo[4];
-        le[0] = lds_f32(lds + TABLE_OFF, entry_addr<0>(ce, laneoff)); lo[0] = lds_f32(lds + TABLE_OFF, entry_addr<0>(co, laneoff));
-        le[1] = lds_f32(lds + TABLE_OFF, entry_addr<1>(ce, laneoff)); lo[1] = lds_f32(lds + TABLE_OFF, entry_addr<1>(co, laneoff));
-        le[2] = lds_f32(lds + TABLE_OFF, entry_addr<2>(ce, laneoff)); lo[2] = lds_f32(lds + TABLE_OFF, entry_addr<2>(co, laneoff));
-        le[3] = lds_f32(lds + TABLE_OFF, entry_addr<3>(ce, laneoff)); lo[3] = lds_f32(lds + TABLE_OFF, entry_addr<3>(co, laneoff));
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                acc[b] = __builtin_fmaf(le[j], xt[b][8 * d + 2 * j], acc[b]);
-                acc[b] = __builtin_fmaf(lo[j], xt[b][8 * d + 2 * j + 1], acc[b]);
-            }
-        }
-    }
-}
-
-constexpr int kLut256Bytes = 256 * 256;   // 256 entries x 64 lanes x 4 B
+constexpr int kLut256Bytes = 256 * 256;          // 256 entries x 64 lanes x 4 B
 constexpr int kTab16Bytes = 16 * 256;
+constexpr int kPartialBytes = 2 * 16 * 16 * 4;   // [2 buffers][<=16 waves][<=16 values]
+constexpr int kShareBytes = 4 * kSlab * 4;       // activation hand-over: up to 4 slab images
 
 template <int MODE>
 __host__ __device__ constexpr int table_bytes() {
     return MODE == kSharedLut ? kLut256Bytes : (MODE == kDual ? 2 * kTab16Bytes : kTab16Bytes);
+}
+template <int MODE>
+__host__ __device__ constexpr int table_region_bytes() {
+    return table_bytes<MODE>() > kShareBytes ? table_bytes<MODE>() : kShareBytes;
 }
 
 // Rotated activations of this lane's chunk for one batch row: H (s (.) x).
@@ -141,120 +159,153 @@ __device__ __forceinline__ void rotate_chunk(const void* x, int x_dtype, size_t 
 
 template <int MODE, int NB, int R, int MAXT>
 __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
-    extern __shared__ __align__(16) char smem[];
-    constexpr int kTable = table_bytes<MODE>();
-    float* partial = reinterpret_cast<float*>(smem + kTable);   // [2][S][W][R*NB]
+    constexpr int kRegion = table_region_bytes<MODE>();
+    constexpr int V = R * NB;                       // sums produced per row group
+    __shared__ __align__(16) char smem[kRegion + kPartialBytes];
+    float* partial = reinterpret_cast<float*>(smem + kRegion);   // [2][waves][V]
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int slab = wave % a.W;
     const int stream = wave / a.W;
     const int chunk = slab * kWave + lane;
     const bool active = chunk < a.chunks;
+    const int chunk_c = active ? chunk : a.chunks - 1;      // idle lanes re-read a valid chunk; their xt is 0
     const uint32_t laneoff = (uint32_t)lane << 2;
     const int out = a.L.out_features;
     const size_t row_bytes = (size_t)a.L.in_features >> 1;
-    const bool use_res = (MODE != kPrimaryOnly);
+    constexpr bool use_res = (MODE != kPrimaryOnly);
 
     const long long gs = (long long)blockIdx.x * a.S + stream;
     const long long ts = (long long)gridDim.x * a.S;
     const int g_begin = (int)(gs * a.groups / ts);
     const int g_end = (int)((gs + 1) * a.groups / ts);
 
-    const uint8_t* pp = a.L.packed_primary + (size_t)chunk * 16;
-    const uint8_t* pr = a.L.packed_residual + (size_t)chunk * 16;
+    const uint8_t* pp = a.L.packed_primary + (size_t)chunk_c * 16;
+    const uint8_t* pr = a.L.packed_residual + (size_t)chunk_c * 16;
 
     uint4 P[2][R], Q[2][R];
     auto fetch = [&](int buf, int g) {
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            const int r = g * R + i;
-            if (active && g < g_end && r < out) {
-                P[buf][i] = *reinterpret_cast<const uint4*>(pp + (size_t)r * row_bytes);
-                if (use_res) Q[buf][i] = *reinterpret_cast<const uint4*>(pr + (size_t)r * row_bytes);
-            } else {
-                P[buf][i] = make_uint4(0, 0, 0, 0);
-                if (use_res) Q[buf][i] = make_uint4(0, 0, 0, 0);
-            }
+            int r = g * R + i;
+            r = r < out ? r : out - 1;                      // rows past the end re-read the last row; never stored
+            P[buf][i] = load_stream16(pp + (size_t)r * row_bytes);
+            if constexpr (use_res)
+                Q[buf][i] = load_stream16(pr + (size_t)r * row_bytes);
+            else
+                Q[buf][i] = make_uint4(0, 0, 0, 0);
         }
     };
 
     // First weight fetch goes out before the prologue so its latency overlaps it.
     fetch(0, g_begin);
 
+    // Rotated activations, kept in registers for the whole kernel.
+    float xt[NB][kChunk];
+    float xr[NB][kChunk];   // second rotation, dual mode only
+    if (a.share_x) {
+        // One stream rotates, every stream of the workgroup picks the result up from LDS
+        // (value k of lane l at float index k*64 + l: conflict-free both ways).
+        float* xs = reinterpret_cast<float*>(smem);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (stream == 0) {
+                rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
+                             a.L.seed_primary, a.L.block_size, lane, xt[b]);
+#pragma unroll
+                for (int k = 0; k < kChunk; ++k) xs[slab * kSlab + k * kWave + lane] = xt[b][k];
+            }
+            __syncthreads();
+            if (stream != 0) {
+#pragma unroll
+                for (int k = 0; k < kChunk; ++k) xt[b][k] = xs[slab * kSlab + k * kWave + lane];
+            }
+            __syncthreads();
+            if constexpr (MODE == kDual) {
+                if (stream == 0) {
+                    rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
+                                 a.L.seed_residual, a.L.block_size, lane, xr[b]);
+#pragma unroll
+                    for (int k = 0; k < kChunk; ++k) xs[slab * kSlab + k * kWave + lane] = xr[b][k];
+                }
+                __syncthreads();
+                if (stream != 0) {
+#pragma unroll
+                    for (int k = 0; k < kChunk; ++k) xr[b][k] = xs[slab * kSlab + k * kWave + lane];
+                }
+                __syncthreads();
+            }
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
+                         a.L.seed_primary, a.L.block_size, lane, xt[b]);
+            if constexpr (MODE == kDual)
+                rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
+                             a.L.seed_residual, a.L.block_size, lane, xr[b]);
+        }
+    }
+
     // Decode tables -> LDS, one private column per lane.
     {
-        const int entries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
+        constexpr int entries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
         float4* dst = reinterpret_cast<float4*>(smem);
         for (int i = tid; i < entries * 16; i += blockDim.x) {
             const float v = a.L.tables[i >> 4];
             dst[i] = make_float4(v, v, v, v);
         }
     }
-
-    // Rotated activations, kept in registers for the whole kernel.
-    float xt[NB][kChunk];
-    float xr[NB][kChunk];   // second rotation, dual mode only
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
-        rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
-                     a.L.seed_primary, a.L.block_size, lane, xt[b]);
-        if constexpr (MODE == kDual)
-            rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
-                         a.L.seed_residual, a.L.block_size, lane, xr[b]);
-    }
     __syncthreads();
 
     auto consume = [&](int buf, int g, int it) {
-        float acc[R][NB];
+        float acc[V];
 #pragma unroll
         for (int i = 0; i < R; ++i) {
+            float val[kChunk];
+            lookup32<MODE == kSharedLut, 0>(P[buf][i], Q[buf][i], smem, laneoff, val);
 #pragma unroll
-            for (int b = 0; b < NB; ++b) acc[i][b] = 0.0f;
-            if constexpr (MODE == kSharedLut) {
-                row_lut256<NB>(P[buf][i], Q[buf][i], xt, acc[i], smem, laneoff);
-            } else {
-                row_tab16<NB, 0>(P[buf][i], xt, acc[i], smem, laneoff);
-                if constexpr (MODE == kDual) row_tab16<NB, kTab16Bytes>(Q[buf][i], xr, acc[i], smem, laneoff);
+            for (int b = 0; b < NB; ++b) {
+                float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+                for (int k = 0; k < kChunk; k += 2) {
+                    s0 = __builtin_fmaf(val[k], xt[b][k], s0);
+                    s1 = __builtin_fmaf(val[k + 1], xt[b][k + 1], s1);
+                }
+                acc[i * NB + b] = s0 + s1;
+            }
+            if constexpr (MODE == kDual) {
+                lookup32<false, kTab16Bytes>(Q[buf][i], Q[buf][i], smem, laneoff, val);
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < kChunk; k += 2) {
+                        s0 = __builtin_fmaf(val[k], xr[b][k], s0);
+                        s1 = __builtin_fmaf(val[k + 1], xr[b][k + 1], s1);
+                    }
+                    acc[i * NB + b] += s0 + s1;
+                }
             }
         }
-        float sums[R][NB];
-#pragma unroll
-        for (int i = 0; i < R; ++i)
-#pragma unroll
-            for (int b = 0; b < NB; ++b) sums[i][b] = wave_sum(acc[i][b]);
+        // Lane l < V now gets the wave total of value l = i*NB + b.
+        const float total = reduce_rec<V, 1>(acc, lane);
+        const int i = lane / NB, b = lane % NB;
+        const int r = g * R + i;
+        const bool owner = lane < V && g < g_end && r < out;
 
         if (a.W == 1) {
-            if (lane == 0 && g < g_end) {
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    const int r = g * R + i;
-                    if (r < out) {
-                        const float s = a.out_scale * a.L.norms[r];
-#pragma unroll
-                        for (int b = 0; b < NB; ++b)
-                            store_scalar(a.y, a.y_dtype, (size_t)b * out + r, sums[i][b] * s);
-                    }
-                }
-            }
+            if (owner) store_scalar(a.y, a.y_dtype, (size_t)b * out + r, total * (a.out_scale * a.L.norms[r]));
         } else {
-            float* slot = partial + (size_t)(it & 1) * a.S * a.W * (R * NB) + (size_t)stream * a.W * (R * NB);
-            if (lane == 0) {
-#pragma unroll
-                for (int i = 0; i < R; ++i)
-#pragma unroll
-                    for (int b = 0; b < NB; ++b) slot[slab * (R * NB) + i * NB + b] = sums[i][b];
-            }
+            float* buf_base = partial + (it & 1) * (16 * 16);
+            if (lane < V) buf_base[wave * V + lane] = total;
             __syncthreads();
-            if (slab == 0 && lane < R * NB && g < g_end) {
-                const int i = lane / NB, b = lane % NB;
-                const int r = g * R + i;
-                if (r < out) {
-                    float t = 0.0f;
-                    for (int w = 0; w < a.W; ++w) t += slot[w * (R * NB) + lane];
-                    store_scalar(a.y, a.y_dtype, (size_t)b * out + r, t * (a.out_scale * a.L.norms[r]));
-                }
+            if (slab == 0 && owner) {
+                float t = 0.0f;
+                for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * V + lane];
+                store_scalar(a.y, a.y_dtype, (size_t)b * out + r, t * (a.out_scale * a.L.norms[r]));
             }
         }
     };
@@ -272,16 +323,8 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
 }
 
 template <int MODE, int NB, int R, int MAXT>
-static hipError_t launch_one(const GemvArgs& a, int grid, int threads, size_t lds, hipStream_t stream) {
-    auto kern = tq_gemv_kernel<MODE, NB, R, MAXT>;
-    static thread_local bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, a);
+static hipError_t launch_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
+    hipLaunchKernelGGL((tq_gemv_kernel<MODE, NB, R, MAXT>), dim3(grid), dim3(threads), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -294,6 +337,7 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     a.S = (a.W >= 8) ? 1 : (8 / a.W);
     const int threads = a.W * a.S * kWave;
     const int max_grid = num_cus * 2;
+    a.share_x = (a.S > 1 && a.W * kSlab * 4 <= kShareBytes) ? 1 : 0;
 
     // Largest row-group size that still gives every resident stream work.
     int R = 4;
@@ -304,12 +348,11 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     if (grid < 1) grid = 1;
     const long long ts = (long long)grid * a.S;
     a.iters = (int)((a.groups + ts - 1) / ts);
-    const size_t lds = (size_t)table_bytes<MODE>() + (size_t)2 * a.S * a.W * R * NB * sizeof(float);
 
     switch (R) {
-        case 4: return launch_one<MODE, NB, 4, MAXT>(a, grid, threads, lds, stream);
-        case 2: return launch_one<MODE, NB, 2, MAXT>(a, grid, threads, lds, stream);
-        default: return launch_one<MODE, NB, 1, MAXT>(a, grid, threads, lds, stream);
+        case 4: return launch_one<MODE, NB, 4, MAXT>(a, grid, threads, stream);
+        case 2: return launch_one<MODE, NB, 2, MAXT>(a, grid, threads, stream);
+        default: return launch_one<MODE, NB, 1, MAXT>(a, grid, threads, stream);
     }
 }
 
