@@ -47,7 +47,20 @@ __global__ __launch_bounds__(kDqWaves* kWave) void tq_dequant_kernel(LayerView L
 
     uint32_t pi[kChunk], ri[kChunk];
     float v[kChunk];
-    if (active) {
+    if (active && L.mode == kSharedLut) {
+        // combined plane: one byte per weight, residual nibble high, primary nibble low
+        const uint4* p = reinterpret_cast<const uint4*>(L.packed_combined + (size_t)row * in + (size_t)chunk * 32);
+        const uint4 a = p[0], b = p[1];
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t c = (w[d] >> (8 * j)) & 0xffu;
+                pi[4 * d + j] = c & 0x0fu;
+                ri[4 * d + j] = c >> 4;
+            }
+    } else if (active) {
         if (five) {
             const uint4* p = reinterpret_cast<const uint4*>(L.packed_primary + (size_t)row * in + (size_t)chunk * 32);
             const uint4 a = p[0], b = p[1];
@@ -187,6 +200,26 @@ __global__ void tq_any_nonzero_kernel(const uint8_t* __restrict__ data, size_t n
     }
     for (size_t i = n16 * 16 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) acc |= data[i];
     if (acc) atomicOr(flag, 1);
+}
+
+// Interleave the two nibble planes into one byte per weight (residual high, primary low),
+// the layout the shared-rotation GEMV streams.  One thread per packed byte pair.
+__global__ void tq_combine_planes_kernel(const uint8_t* __restrict__ primary, const uint8_t* __restrict__ residual,
+                                         uint16_t* __restrict__ combined, size_t plane_bytes) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < plane_bytes; i += stride) {
+        const uint32_t pb = primary[i], rb = residual[i];
+        const uint32_t even = (pb & 0x0fu) | ((rb & 0x0fu) << 4);   // src/dequantizer.cpp:163
+        const uint32_t odd = (pb >> 4) | (rb & 0xf0u);              // src/dequantizer.cpp:168
+        combined[i] = (uint16_t)(even | (odd << 8));
+    }
+}
+
+hipError_t launch_combine_planes(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,
+                                 size_t plane_bytes, hipStream_t stream) {
+    hipLaunchKernelGGL(tq_combine_planes_kernel, dim3(2048), dim3(256), 0, stream, primary, residual,
+                       reinterpret_cast<uint16_t*>(combined), plane_bytes);
+    return hipGetLastError();
 }
 
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream) {

@@ -23,6 +23,9 @@ constexpr int kSlab = kWave * kChunk;   // columns covered by one wave
 struct LayerView {
     const uint8_t* packed_primary;   // [out, in/2] nibble pairs (or [out, in] bytes for 5-bit)
     const uint8_t* packed_residual;  // [out, in/2]
+    const uint8_t* packed_combined;  // shared-rotation 4-bit mode only: [out, in], one byte per weight =
+                                     // residual_nibble << 4 | primary_nibble (the LUT index of reference
+                                     // src/dequantizer.cpp:163-169); the two planes above are then NULL
     const float*   norms;            // [out]
     const float*   tables;           // decode tables, layout depends on mode (see build_tables)
     int out_features;
@@ -42,6 +45,8 @@ hipError_t launch_dequant(const LayerView& L, float* w, hipStream_t stream);
 hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t seed,
                       uint32_t block_size, float inv_sqrt_bs, int inverse, hipStream_t stream);
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream);
+hipError_t launch_combine_planes(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,
+                                 size_t plane_bytes, hipStream_t stream);
 
 // True when the fast wave-per-slab kernels can handle this shape.
 inline bool shape_supported(int in_features, uint32_t block_size) {
@@ -66,17 +71,42 @@ __device__ __forceinline__ float sign_of(uint32_t seed, uint32_t index) {
     return (h & 1u) ? 1.0f : -1.0f;
 }
 
-// Unnormalised natural-order Walsh-Hadamard butterfly over a block that is
-// spread as 32 consecutive values per lane over bs/32 neighbouring lanes
-// (or lives entirely inside the lane when bs <= 32).  Stage order and the
-// (a+b, a-b) convention are those of reference src/rotation.cpp:14-25, so the
-// result is bit-identical to the CPU butterfly.
-__device__ __forceinline__ void fwht_lane32(float (&v)[kChunk], uint32_t bs, int lane) {
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
+// Value held by lane (lane ^ MASK).
+template <int MASK>
+__device__ __forceinline__ float lane_xor(float v) {
+    if constexpr (MASK == 1) return dpp_mov<0xB1>(v);        // quad_perm [1,0,3,2]
+    else if constexpr (MASK == 2) return dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (MASK == 8) return dpp_mov<0x128>(v);  // row_ror:8
+    else return __shfl_xor(v, MASK, kWave);
+}
+
+// One cross-lane butterfly stage over N values per lane: the lower lane of a pair
+// gets a+b, the upper lane a-b.  fma(v, +-1, partner) is exact, so the result is
+// bit-identical to the add/sub of the CPU butterfly.
+template <int MASK, int N>
+__device__ __forceinline__ void butterfly_lanes(float (&v)[N], int lane) {
+    const float sgn = (lane & MASK) ? -1.0f : 1.0f;
 #pragma unroll
-    for (int h = 1; h < kChunk; h <<= 1) {
+    for (int k = 0; k < N; ++k) v[k] = __builtin_fmaf(v[k], sgn, lane_xor<MASK>(v[k]));
+}
+
+// Unnormalised natural-order Walsh-Hadamard butterfly over a block that is
+// spread as N consecutive values per lane over bs/N neighbouring lanes (or lives
+// entirely inside the lane when bs <= N).  Stage order and the (a+b, a-b)
+// convention are those of reference src/rotation.cpp:14-25, so the result is
+// bit-identical to the CPU butterfly.
+template <int N>
+__device__ __forceinline__ void fwht_lanes(float (&v)[N], uint32_t bs, int lane) {
+#pragma unroll
+    for (int h = 1; h < N; h <<= 1) {
         if ((uint32_t)h < bs) {
 #pragma unroll
-            for (int i = 0; i < kChunk; i += 2 * h) {
+            for (int i = 0; i < N; i += 2 * h) {
 #pragma unroll
                 for (int j = i; j < i + h; ++j) {
                     float a = v[j], b = v[j + h];
@@ -86,14 +116,16 @@ __device__ __forceinline__ void fwht_lane32(float (&v)[kChunk], uint32_t bs, int
             }
         }
     }
-    for (uint32_t m = 1; m * kChunk < bs; m <<= 1) {
-        const bool upper = (lane & (int)m) != 0;
-#pragma unroll
-        for (int k = 0; k < kChunk; ++k) {
-            float p = __shfl_xor(v[k], (int)m, kWave);
-            v[k] = upper ? (p - v[k]) : (v[k] + p);
-        }
-    }
+    if ((uint32_t)N * 1 < bs) butterfly_lanes<1, N>(v, lane);
+    if ((uint32_t)N * 2 < bs) butterfly_lanes<2, N>(v, lane);
+    if ((uint32_t)N * 4 < bs) butterfly_lanes<4, N>(v, lane);
+    if ((uint32_t)N * 8 < bs) butterfly_lanes<8, N>(v, lane);
+    if ((uint32_t)N * 16 < bs) butterfly_lanes<16, N>(v, lane);
+    if ((uint32_t)N * 32 < bs) butterfly_lanes<32, N>(v, lane);
+}
+
+__device__ __forceinline__ void fwht_lane32(float (&v)[kChunk], uint32_t bs, int lane) {
+    fwht_lanes<kChunk>(v, bs, lane);
 }
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) {

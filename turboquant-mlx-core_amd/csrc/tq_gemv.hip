@@ -17,6 +17,7 @@
 // one private 4-byte column per lane (entry pitch 256 B), so lookups never conflict
 // and the LDS byte address is assembled with a single v_perm_b32.
 #include "tq_device.h"
+#include <cstdlib>
 
 namespace tq {
 
@@ -27,9 +28,8 @@ struct GemvArgs {
     int x_dtype, y_dtype;
     int chunks;      // in / 32
     int W, S;        // slabs per row, row streams per workgroup
-    int groups;      // ceil(out / R)
-    int iters;       // uniform trip count: ceil(groups / (gridDim.x * S))
-    int share_x;     // rotate the activations once per workgroup and pass them through LDS
+    int groups;      // unused
+    int iters;       // uniform trip count: ceil(longest row range / R)
     float out_scale; // inv_scale * inv_sqrt_bs
 };
 
@@ -39,20 +39,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 load_stream16(const uint8_t* p) {
     const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
     return make_uint4(t.x, t.y, t.z, t.w);
-}
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_mov(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-
-// Value held by lane (lane ^ MASK).
-template <int MASK>
-__device__ __forceinline__ float lane_xor(float v) {
-    if constexpr (MASK == 1) return dpp_mov<0xB1>(v);        // quad_perm [1,0,3,2]
-    else if constexpr (MASK == 2) return dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
-    else if constexpr (MASK == 8) return dpp_mov<0x128>(v);  // row_ror:8
-    else return __shfl_xor(v, MASK, kWave);
 }
 
 // Transposed wave reduction of N per-lane partial sums (N a power of two <= 16):
@@ -94,158 +80,234 @@ __device__ __forceinline__ float lds_f32(const char* lds, uint32_t byte_addr) {
     return *reinterpret_cast<const float*>(lds + byte_addr);
 }
 
-// Centroid values of the 32 columns a lane owns, from one 16-entry table
-// (TABLE_OFF selects it) or from the 256-entry sum table of shared rotation
-// (reference src/dequantizer.cpp:144-169: index = residual_nibble << 4 | primary_nibble).
+// Centroid values of the 32 columns a lane owns.
+//   LUT256: P, Q are the lane's 32 combined bytes (residual_nibble << 4 | primary_nibble, one per
+//           column); each byte indexes the 256-entry sum table of shared rotation
+//           (reference src/dequantizer.cpp:144-169).
+//   else  : P holds 32 nibbles of one plane (lo nibble = even column); 16-entry table at TABLE_OFF.
 template <bool LUT256, int TABLE_OFF>
 __device__ __forceinline__ void lookup32(const uint4& P, const uint4& Q, const char* lds, uint32_t laneoff,
                                          float (&val)[kChunk]) {
-    const uint32_t pw[4] = {P.x, P.y, P.z, P.w};
-    const uint32_t rw[4] = {Q.x, Q.y, Q.z, Q.w};
-    uint32_t ce[4], co[4];
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        if constexpr (LUT256) {
-            ce[d] = ((rw[d] << 4) & 0xF0F0F0F0u) | (pw[d] & 0x0F0F0F0Fu);     // even columns
-            co[d] = (rw[d] & 0xF0F0F0F0u) | ((pw[d] >> 4) & 0x0F0F0F0Fu);    // odd columns
-        } else {
-            ce[d] = pw[d] & 0x0F0F0F0Fu;
-            co[d] = (pw[d] >> 4) & 0x0F0F0F0Fu;
-        }
-    }
     const char* tab = lds + TABLE_OFF;
+    if constexpr (LUT256) {
+        const uint32_t w[8] = {P.x, P.y, P.z, P.w, Q.x, Q.y, Q.z, Q.w};
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        val[8 * d + 0] = lds_f32(tab, entry_addr<0>(ce[d], laneoff));
-        val[8 * d + 1] = lds_f32(tab, entry_addr<0>(co[d], laneoff));
-        val[8 * d + 2] = lds_f32(tab, entry_addr<1>(ce[d], laneoff));
-        val[8 * d + 3] = lds_f32(tab, entry_addr<1>(co[d], laneoff));
-        val[8 * d + 4] = lds_f32(tab, entry_addr<2>(ce[d], laneoff));
-        val[8 * d + 5] = lds_f32(tab, entry_addr<2>(co[d], laneoff));
-        val[8 * d + 6] = lds_f32(tab, entry_addr<3>(ce[d], laneoff));
-        val[8 * d + 7] = lds_f32(tab, entry_addr<3>(co[d], laneoff));
+        for (int d = 0; d < 8; ++d) {
+            val[4 * d + 0] = lds_f32(tab, entry_addr<0>(w[d], laneoff));
+            val[4 * d + 1] = lds_f32(tab, entry_addr<1>(w[d], laneoff));
+            val[4 * d + 2] = lds_f32(tab, entry_addr<2>(w[d], laneoff));
+            val[4 * d + 3] = lds_f32(tab, entry_addr<3>(w[d], laneoff));
+        }
+    } else {
+        const uint32_t pw[4] = {P.x, P.y, P.z, P.w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t ce = pw[d] & 0x0F0F0F0Fu;
+            const uint32_t co = (pw[d] >> 4) & 0x0F0F0F0Fu;
+            val[8 * d + 0] = lds_f32(tab, entry_addr<0>(ce, laneoff));
+            val[8 * d + 1] = lds_f32(tab, entry_addr<0>(co, laneoff));
+            val[8 * d + 2] = lds_f32(tab, entry_addr<1>(ce, laneoff));
+            val[8 * d + 3] = lds_f32(tab, entry_addr<1>(co, laneoff));
+            val[8 * d + 4] = lds_f32(tab, entry_addr<2>(ce, laneoff));
+            val[8 * d + 5] = lds_f32(tab, entry_addr<2>(co, laneoff));
+            val[8 * d + 6] = lds_f32(tab, entry_addr<3>(ce, laneoff));
+            val[8 * d + 7] = lds_f32(tab, entry_addr<3>(co, laneoff));
+        }
     }
 }
 
 constexpr int kLut256Bytes = 256 * 256;          // 256 entries x 64 lanes x 4 B
 constexpr int kTab16Bytes = 16 * 256;
+constexpr int kRegionBytes = kLut256Bytes;       // decode tables; doubles as activation hand-over space
+constexpr int kRegionFloats = kRegionBytes / 4;
 constexpr int kPartialBytes = 2 * 16 * 16 * 4;   // [2 buffers][<=16 waves][<=16 values]
-constexpr int kShareBytes = 4 * kSlab * 4;       // activation hand-over: up to 4 slab images
+constexpr int kTile = 512;                       // columns rotated by one wave in the prologue (8 per lane)
 
-template <int MODE>
-__host__ __device__ constexpr int table_bytes() {
-    return MODE == kSharedLut ? kLut256Bytes : (MODE == kDual ? 2 * kTab16Bytes : kTab16Bytes);
-}
-template <int MODE>
-__host__ __device__ constexpr int table_region_bytes() {
-    return table_bytes<MODE>() > kShareBytes ? table_bytes<MODE>() : kShareBytes;
-}
-
-// Rotated activations of this lane's chunk for one batch row: H (s (.) x).
-__device__ __forceinline__ void rotate_chunk(const void* x, int x_dtype, size_t row_off, int chunk,
-                                             bool active, uint32_t seed, uint32_t bs, int lane,
-                                             float (&v)[kChunk]) {
+// Rotate one 512-column tile of an activation row: lane owns 8 consecutive columns.
+// Valid for block sizes up to 512 (a block never straddles a tile).
+__device__ __forceinline__ void rotate_tile(const void* x, int x_dtype, size_t row_off, int col, bool active,
+                                            uint32_t seed, uint32_t bs, int lane, float (&v)[8]) {
     if (active) {
-        load_chunk(x, x_dtype, row_off + (size_t)chunk * kChunk, v);
-        const uint32_t col0 = ((uint32_t)chunk * kChunk) & (bs - 1);
+        if (x_dtype == kF32) {
+            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(x) + row_off + col);
+            const float4 a = p[0], b = p[1];
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        } else {
+            const uint4 t = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + row_off + col);
+            const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
-        for (int k = 0; k < kChunk; ++k) v[k] *= sign_of(seed, (col0 + k) & (bs - 1));
+            for (int j = 0; j < 4; ++j) {
+                if (x_dtype == kBF16) {
+                    v[2 * j]     = bf16_bits_to_float(w[j] & 0xffffu);
+                    v[2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+                } else {
+                    v[2 * j]     = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] & 0xffffu));
+                    v[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] >> 16));
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] *= sign_of(seed, ((uint32_t)col + j) & (bs - 1));
     } else {
 #pragma unroll
-        for (int k = 0; k < kChunk; ++k) v[k] = 0.0f;
+        for (int j = 0; j < 8; ++j) v[j] = 0.0f;
     }
-    fwht_lane32(v, bs, lane);
+    fwht_lanes<8>(v, bs, lane);
+}
+
+// Column ownership.  A lane owns two runs of 16 columns inside its wave's 2048-column slab:
+//   SPLIT (combined byte plane): columns 16*lane.. and 1024 + 16*lane..  so that each of the
+//          lane's two 16-byte loads is contiguous across the wave (1 KB per load instruction);
+//   else  (nibble planes): columns 32*lane.. and 32*lane + 16..  (one 16-byte load per plane).
+// Value k (0..31) of lane l sits at float index k*64 + l of the slab's staging image.
+template <bool SPLIT>
+__device__ __forceinline__ int stage_index(int col_in_slab) {
+    if constexpr (SPLIT) {
+        const int h = col_in_slab >> 10, rem = col_in_slab & 1023;
+        return ((h << 4) + (rem & 15)) * kWave + (rem >> 4);
+    } else {
+        return (col_in_slab & 31) * kWave + (col_in_slab >> 5);
+    }
+}
+
+// Rotated activations H (s (.) x) of one batch row for every lane of the workgroup.
+// The waves rotate 512-column tiles cooperatively (block sizes up to 512), or run the
+// butterfly stage by stage in LDS (larger blocks), and each lane then picks up the 32
+// values of the columns it owns.  Rows wider than the staging space are handled in
+// passes of 8 slabs.
+template <bool SPLIT>
+__device__ __forceinline__ void rotate_row_shared(const void* x, int x_dtype, size_t row_off, int in_features,
+                                                  uint32_t seed, uint32_t bs, float* stage,
+                                                  int wave, int nwaves, int lane, int slab,
+                                                  bool act_a, bool act_b, float (&xt)[kChunk]) {
+    const int tiles = (in_features + kTile - 1) / kTile;
+    constexpr int kTilesPerPass = kRegionFloats / kTile;       // 32 tiles = 8 slabs
+    for (int t0 = 0; t0 < tiles; t0 += kTilesPerPass) {
+        const int t1 = (t0 + kTilesPerPass < tiles) ? t0 + kTilesPerPass : tiles;
+        const int col_base = t0 * kTile;
+        if (bs <= (uint32_t)kTile) {
+            for (int t = t0 + wave; t < t1; t += nwaves) {
+                const int col = t * kTile + lane * 8;
+                float v[8];
+                rotate_tile(x, x_dtype, row_off, col, col < in_features, seed, bs, lane, v);
+                const int rel = col - col_base;
+                float* dst = stage + (rel >> 11) * kSlab + stage_index<SPLIT>(rel & (kSlab - 1));
+#pragma unroll
+                for (int j = 0; j < 8; ++j) dst[j * kWave] = v[j];      // 8 columns stay inside one 16-run
+            }
+            __syncthreads();
+        } else {
+            // Generic path: signed activations in natural order, one butterfly stage per barrier
+            // (same (a+b, a-b) pairs and stage order as reference src/rotation.cpp:14-25).
+            const int ncols = ((t1 * kTile < in_features) ? t1 * kTile : in_features) - col_base;
+            const int tid = wave * kWave + lane, nthreads = nwaves * kWave;
+            for (int c = tid; c < ncols; c += nthreads) {
+                const size_t e = row_off + col_base + c;
+                float v;
+                if (x_dtype == kF32) v = static_cast<const float*>(x)[e];
+                else if (x_dtype == kBF16) v = bf16_bits_to_float(static_cast<const uint16_t*>(x)[e]);
+                else v = (float)static_cast<const _Float16*>(x)[e];
+                stage[c] = v * sign_of(seed, (uint32_t)(col_base + c) & (bs - 1));
+            }
+            __syncthreads();
+            for (uint32_t h = 1; h < bs; h <<= 1) {
+                for (int q = tid; q < (ncols >> 1); q += nthreads) {
+                    const int i = ((q / (int)h) * 2 * (int)h) + (q % (int)h);
+                    const float u = stage[i], w = stage[i + h];
+                    stage[i] = u + w;
+                    stage[i + h] = u - w;
+                }
+                __syncthreads();
+            }
+        }
+        const int s_rel = slab - (t0 >> 2);
+        if (s_rel >= 0 && s_rel < (kTilesPerPass >> 2)) {
+            if (bs <= (uint32_t)kTile) {
+                const float* src = stage + s_rel * kSlab + lane;
+#pragma unroll
+                for (int k = 0; k < kChunk; ++k)
+                    xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
+            } else {
+                const int ca = s_rel * kSlab + (SPLIT ? 16 * lane : 32 * lane);
+                const int cb = SPLIT ? ca + 1024 : ca + 16;
+#pragma unroll
+                for (int k = 0; k < 16; ++k) {
+                    xt[k] = act_a ? stage[ca + k] : 0.0f;
+                    xt[16 + k] = act_b ? stage[cb + k] : 0.0f;
+                }
+            }
+        }
+        __syncthreads();
+    }
 }
 
 template <int MODE, int NB, int R, int MAXT>
 __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
-    constexpr int kRegion = table_region_bytes<MODE>();
     constexpr int V = R * NB;                       // sums produced per row group
-    __shared__ __align__(16) char smem[kRegion + kPartialBytes];
-    float* partial = reinterpret_cast<float*>(smem + kRegion);   // [2][waves][V]
+    __shared__ __align__(16) char smem[kRegionBytes + kPartialBytes];
+    float* partial = reinterpret_cast<float*>(smem + kRegionBytes);   // [2][waves][V]
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = blockDim.x >> 6;
     const int slab = wave % a.W;
     const int stream = wave / a.W;
-    const int chunk = slab * kWave + lane;
-    const bool active = chunk < a.chunks;
-    const int chunk_c = active ? chunk : a.chunks - 1;      // idle lanes re-read a valid chunk; their xt is 0
+    // Shared-rotation mode streams the combined plane (one byte per weight); the other modes
+    // stream 16 B from each nibble plane.  See stage_index for the column ownership.
+    constexpr bool combined = (MODE == kSharedLut);
+    const int col_a = slab * kSlab + (combined ? 16 * lane : 32 * lane);
+    const int col_b = combined ? col_a + 1024 : col_a + 16;
+    const bool act_a = col_a < a.L.in_features, act_b = col_b < a.L.in_features;
     const uint32_t laneoff = (uint32_t)lane << 2;
     const int out = a.L.out_features;
-    const size_t row_bytes = (size_t)a.L.in_features >> 1;
+    const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
     constexpr bool use_res = (MODE != kPrimaryOnly);
 
+    // Contiguous row range of this stream.
     const long long gs = (long long)blockIdx.x * a.S + stream;
     const long long ts = (long long)gridDim.x * a.S;
-    const int g_begin = (int)(gs * a.groups / ts);
-    const int g_end = (int)((gs + 1) * a.groups / ts);
+    const int r_begin = (int)(gs * out / ts);
+    const int r_end = (int)((gs + 1) * out / ts);
 
-    const uint8_t* pp = a.L.packed_primary + (size_t)chunk_c * 16;
-    const uint8_t* pr = a.L.packed_residual + (size_t)chunk_c * 16;
+    // Idle runs re-read a valid address; their rotated activations are 0.
+    const uint8_t* pp = combined ? a.L.packed_combined + (act_a ? col_a : 0) : a.L.packed_primary + (act_a ? (col_a >> 1) : 0);
+    const uint8_t* pr = combined ? a.L.packed_combined + (act_b ? col_b : 0) : a.L.packed_residual + (act_a ? (col_a >> 1) : 0);
 
     uint4 P[2][R], Q[2][R];
-    auto fetch = [&](int buf, int g) {
+    auto fetch = [&](int buf, int r0) {
+        if (r0 + R <= r_end) {                               // wave-uniform: a full group, straight-line
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            int r = g * R + i;
-            r = r < out ? r : out - 1;                      // rows past the end re-read the last row; never stored
-            P[buf][i] = load_stream16(pp + (size_t)r * row_bytes);
-            if constexpr (use_res)
-                Q[buf][i] = load_stream16(pr + (size_t)r * row_bytes);
-            else
-                Q[buf][i] = make_uint4(0, 0, 0, 0);
+            for (int i = 0; i < R; ++i) {
+                P[buf][i] = load_stream16(pp + (size_t)(r0 + i) * row_bytes);
+                if constexpr (use_res) Q[buf][i] = load_stream16(pr + (size_t)(r0 + i) * row_bytes);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                if (r0 + i < r_end) {
+                    P[buf][i] = load_stream16(pp + (size_t)(r0 + i) * row_bytes);
+                    if constexpr (use_res) Q[buf][i] = load_stream16(pr + (size_t)(r0 + i) * row_bytes);
+                }
+            }
         }
     };
 
     // First weight fetch goes out before the prologue so its latency overlaps it.
-    fetch(0, g_begin);
+    fetch(0, r_begin);
 
     // Rotated activations, kept in registers for the whole kernel.
     float xt[NB][kChunk];
     float xr[NB][kChunk];   // second rotation, dual mode only
-    if (a.share_x) {
-        // One stream rotates, every stream of the workgroup picks the result up from LDS
-        // (value k of lane l at float index k*64 + l: conflict-free both ways).
-        float* xs = reinterpret_cast<float*>(smem);
+    {
+        float* stage = reinterpret_cast<float*>(smem);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            if (stream == 0) {
-                rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
-                             a.L.seed_primary, a.L.block_size, lane, xt[b]);
-#pragma unroll
-                for (int k = 0; k < kChunk; ++k) xs[slab * kSlab + k * kWave + lane] = xt[b][k];
-            }
-            __syncthreads();
-            if (stream != 0) {
-#pragma unroll
-                for (int k = 0; k < kChunk; ++k) xt[b][k] = xs[slab * kSlab + k * kWave + lane];
-            }
-            __syncthreads();
-            if constexpr (MODE == kDual) {
-                if (stream == 0) {
-                    rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
-                                 a.L.seed_residual, a.L.block_size, lane, xr[b]);
-#pragma unroll
-                    for (int k = 0; k < kChunk; ++k) xs[slab * kSlab + k * kWave + lane] = xr[b][k];
-                }
-                __syncthreads();
-                if (stream != 0) {
-#pragma unroll
-                    for (int k = 0; k < kChunk; ++k) xr[b][k] = xs[slab * kSlab + k * kWave + lane];
-                }
-                __syncthreads();
-            }
-        }
-    } else {
-#pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
-                         a.L.seed_primary, a.L.block_size, lane, xt[b]);
+            rotate_row_shared<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, a.L.in_features, a.L.seed_primary,
+                                        a.L.block_size, stage, wave, nwaves, lane, slab, act_a, act_b, xt[b]);
             if constexpr (MODE == kDual)
-                rotate_chunk(a.x, a.x_dtype, (size_t)b * a.L.in_features, chunk, active,
-                             a.L.seed_residual, a.L.block_size, lane, xr[b]);
+                rotate_row_shared<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, a.L.in_features, a.L.seed_residual,
+                                            a.L.block_size, stage, wave, nwaves, lane, slab, act_a, act_b, xr[b]);
         }
     }
 
@@ -260,41 +322,52 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     }
     __syncthreads();
 
-    auto consume = [&](int buf, int g, int it) {
-        float acc[V];
+    auto decode_row = [&](int buf, int i, float (&acc)[V]) {
+        float val[kChunk];
+        lookup32<MODE == kSharedLut, 0>(P[buf][i], Q[buf][i], smem, laneoff, val);
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            float val[kChunk];
-            lookup32<MODE == kSharedLut, 0>(P[buf][i], Q[buf][i], smem, laneoff, val);
+        for (int b = 0; b < NB; ++b) {
+            float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kChunk; k += 2) {
+                s0 = __builtin_fmaf(val[k], xt[b][k], s0);
+                s1 = __builtin_fmaf(val[k + 1], xt[b][k + 1], s1);
+            }
+            acc[i * NB + b] = s0 + s1;
+        }
+        if constexpr (MODE == kDual) {
+            lookup32<false, kTab16Bytes>(Q[buf][i], Q[buf][i], smem, laneoff, val);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
                 for (int k = 0; k < kChunk; k += 2) {
-                    s0 = __builtin_fmaf(val[k], xt[b][k], s0);
-                    s1 = __builtin_fmaf(val[k + 1], xt[b][k + 1], s1);
+                    s0 = __builtin_fmaf(val[k], xr[b][k], s0);
+                    s1 = __builtin_fmaf(val[k + 1], xr[b][k + 1], s1);
                 }
-                acc[i * NB + b] = s0 + s1;
+                acc[i * NB + b] += s0 + s1;
             }
-            if constexpr (MODE == kDual) {
-                lookup32<false, kTab16Bytes>(Q[buf][i], Q[buf][i], smem, laneoff, val);
+        }
+    };
+
+    auto consume = [&](int buf, int r0, int it) {
+        float acc[V];
+        if (r0 + R <= r_end) {                               // wave-uniform: a full group, straight-line
 #pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    float s0 = 0.0f, s1 = 0.0f;
+            for (int i = 0; i < R; ++i) decode_row(buf, i, acc);
+        } else {                                             // ragged end of the range: skip missing rows
 #pragma unroll
-                    for (int k = 0; k < kChunk; k += 2) {
-                        s0 = __builtin_fmaf(val[k], xr[b][k], s0);
-                        s1 = __builtin_fmaf(val[k + 1], xr[b][k + 1], s1);
-                    }
-                    acc[i * NB + b] += s0 + s1;
-                }
+            for (int i = 0; i < R; ++i) {
+#pragma unroll
+                for (int b = 0; b < NB; ++b) acc[i * NB + b] = 0.0f;
+                if (r0 + i < r_end) decode_row(buf, i, acc);
             }
         }
         // Lane l < V now gets the wave total of value l = i*NB + b.
         const float total = reduce_rec<V, 1>(acc, lane);
         const int i = lane / NB, b = lane % NB;
-        const int r = g * R + i;
-        const bool owner = lane < V && g < g_end && r < out;
+        const int r = r0 + i;
+        const bool owner = lane < V && r < r_end;
 
         if (a.W == 1) {
             if (owner) store_scalar(a.y, a.y_dtype, (size_t)b * out + r, total * (a.out_scale * a.L.norms[r]));
@@ -310,14 +383,16 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
         }
     };
 
-    // Double-buffered main loop (unrolled by two so the buffers are static).
+    // Double-buffered main loop (unrolled by two so the buffers are static).  The
+    // trip count is uniform over the grid; a stream whose range ends early skips
+    // the work of the missing rows.
     for (int it = 0; it < a.iters; it += 2) {
-        const int g0 = g_begin + it;
-        fetch(1, g0 + 1);
-        consume(0, g0, it);
+        const int r0 = r_begin + it * R;
+        fetch(1, r0 + R);
+        consume(0, r0, it);
         if (it + 1 < a.iters) {
-            fetch(0, g0 + 2);
-            consume(1, g0 + 1, it + 1);
+            fetch(0, r0 + 2 * R);
+            consume(1, r0 + R, it + 1);
         }
     }
 }
@@ -336,18 +411,19 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     if (a.W * kWave > MAXT) return hipErrorInvalidValue;
     a.S = (a.W >= 8) ? 1 : (8 / a.W);
     const int threads = a.W * a.S * kWave;
-    const int max_grid = num_cus * 2;
-    a.share_x = (a.S > 1 && a.W * kSlab * 4 <= kShareBytes) ? 1 : 0;
+    int max_grid = num_cus * 2;
+    if (const char* e = getenv("TQ_GEMV_GRID")) { int v = atoi(e); if (v > 0) max_grid = v; }
 
-    // Largest row-group size that still gives every resident stream work.
-    int R = 4;
-    while (R > 1 && (long long)((out + R - 1) / R) < (long long)max_grid * a.S) R >>= 1;
-    a.groups = (out + R - 1) / R;
-    int grid = (a.groups + a.S - 1) / a.S;
+    int grid = (out + a.S - 1) / a.S;
     if (grid > max_grid) grid = max_grid;
     if (grid < 1) grid = 1;
     const long long ts = (long long)grid * a.S;
-    a.iters = (int)((a.groups + ts - 1) / ts);
+    const int max_rows = (int)((out + ts - 1) / ts);        // longest row range of any stream
+    // Four rows per group only where the register budget allows it without spilling.
+    int R = (max_rows >= 4 && MAXT <= 512) ? 4 : (max_rows >= 2 ? 2 : 1);
+    if (const char* e = getenv("TQ_GEMV_R")) { int v = atoi(e); if (v == 1 || v == 2 || v == 4) R = v; }
+    a.groups = 0;
+    a.iters = (max_rows + R - 1) / R;
 
     switch (R) {
         case 4: return launch_one<MODE, NB, 4, MAXT>(a, grid, threads, stream);
@@ -378,6 +454,7 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
         } else {
             if (left >= 4 && W <= 8)      { step = 4; e = launch_nb<MODE, 4, 512>(a, num_cus, stream); }
             else if (left >= 2 && W <= 8) { step = 2; e = launch_nb<MODE, 2, 512>(a, num_cus, stream); }
+            else if (W <= 8 && getenv("TQ_GEMV_512")) { step = 1; e = launch_nb<MODE, 1, 512>(a, num_cus, stream); }
             else                          { step = 1; e = launch_nb<MODE, 1, 1024>(a, num_cus, stream); }
         }
         if (e != hipSuccess) return e;

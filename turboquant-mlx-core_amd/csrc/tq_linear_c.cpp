@@ -47,6 +47,7 @@ struct tq_linear_s {
     tq::LayerView view{};
     uint8_t* d_primary = nullptr;
     uint8_t* d_residual = nullptr;
+    uint8_t* d_combined = nullptr;
     float* d_norms = nullptr;
     float* d_tables = nullptr;
     int primary_cols = 0;
@@ -58,6 +59,7 @@ struct tq_linear_s {
     ~tq_linear_s() {
         if (d_primary) (void)hipFree(d_primary);
         if (d_residual) (void)hipFree(d_residual);
+        if (d_combined) (void)hipFree(d_combined);
         if (d_norms) (void)hipFree(d_norms);
         if (d_tables) (void)hipFree(d_tables);
         if (d_stage_x) (void)hipFree(d_stage_x);
@@ -160,11 +162,23 @@ tq_linear_t create_impl(int in_features, int out_features,
         delete h; return nullptr;
     }
 
+    if (mode == tq::kSharedLut) {
+        // The shared-rotation kernels stream one byte per weight; interleave the planes once and drop them.
+        const size_t cbytes = (size_t)out_features * in_features;
+        ok = hip_ok(hipMalloc((void**)&h->d_combined, cbytes), "hipMalloc(packed_combined)") &&
+             hip_ok(tq::launch_combine_planes(h->d_primary, h->d_residual, h->d_combined, pbytes, nullptr), "combine_planes") &&
+             hip_ok(hipDeviceSynchronize(), "combine_planes sync");
+        if (!ok) { delete h; return nullptr; }
+        (void)hipFree(h->d_primary); h->d_primary = nullptr;
+        (void)hipFree(h->d_residual); h->d_residual = nullptr;
+    }
+
     h->primary_cols = primary_cols;
     h->residual_cols = residual_cols;
     tq::LayerView& v = h->view;
     v.packed_primary = h->d_primary;
     v.packed_residual = h->d_residual;
+    v.packed_combined = h->d_combined;
     v.norms = h->d_norms;
     v.tables = h->d_tables;
     v.out_features = out_features;
