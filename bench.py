@@ -116,6 +116,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-extra", action="store_true", help="measure the headline configuration only")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy three times (reference reading for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -186,6 +187,9 @@ def main():
 
     # ---- secondary configuration of the metric: 4096 x 4096 fp32, batch 1 ------------
     extra = {}
+    if args.skip_extra:
+        finish(args, torch, extra, result)
+        return
     out1, in1 = 4096, 4096
     copies = 32                         # 32 x 16.8 MB > 256 MB of last-level cache: HBM-resident timing
     handles = [make_layer(tq, torch, out1, in1, bs, seed=100 + i)[0] for i in range(copies)]
@@ -200,6 +204,10 @@ def main():
                                        "hbm_frac": B1 / (us_hbm * 1e-6) / 1e9 / HBM_PEAK_GBS}
     for h in handles:
         tq.lib().tq_linear_free(h)
+    finish(args, torch, extra, result)
+
+
+def finish(args, torch, extra, result):
     if args.copy_calibration:
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
