@@ -150,3 +150,30 @@ def test_error_conventions(tq, oracle):
     with pytest.raises(RuntimeError):
         layer.forward(np.zeros((1, 128), np.float32))        # 5-bit: dequantise only
     layer.close()
+
+
+# ------------------------------------------------------------------ prefill
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("out,inf,bs,batch", [(64, 128, 128, 16), (300, 512, 256, 37), (513, 2048, 512, 64),
+                                              (256, 5120, 512, 300), (1000, 896 * 2, 128, 17)])
+def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, batch):
+    """batch >= 16 with 16-bit activations takes the MFMA path (bf16 weight tiles, bf16 rotated
+    activations, fp32 accumulation): 5e-3 relative L2 against dequantise + fp32 matmul."""
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    x32 = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
+    xbits = oracle.f32_to_bf16_bits(x32)
+    want = oracle.linear_forward(qw, cbp, cbr, bs, oracle.bf16_bits_to_f32(xbits))
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    y = layer.forward(xbits, tq.BF16, tq.F32)
+    yb = oracle.bf16_bits_to_f32(layer.forward(xbits, tq.BF16, tq.BF16))
+    y16 = layer.forward(x32.astype(np.float16), tq.F16, tq.F32)
+    layer.close()
+    assert y.shape == (batch, out)
+    assert _rel(y, want) < 5e-3
+    assert _rel(yb, want) < 7e-3                      # plus bf16 rounding of the outputs
+    assert _rel(y16, oracle.linear_forward(qw, cbp, cbr, bs, x32.astype(np.float16).astype(np.float32))) < 5e-3
+    # every row of the batch must agree with the batch-1 kernel on the same row
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    y1 = layer.forward(xbits[3:4], tq.BF16, tq.F32)
+    layer.close()
+    assert _rel(y[3:4], y1) < 5e-3

@@ -42,6 +42,11 @@ struct LayerView {
 hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch,
                        void* y, int y_dtype, int num_cus, hipStream_t stream);
 hipError_t launch_dequant(const LayerView& L, float* w, hipStream_t stream);
+// Prefill (tq_prefill.hip): rotate the activations to bf16 in `workspace`, then dequant + MFMA GEMM.
+bool prefill_supported(const LayerView& L, int x_dtype, int batch);
+size_t prefill_workspace_bytes(const LayerView& L, int batch);
+hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
+                          void* workspace, hipStream_t stream);
 hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t seed,
                       uint32_t block_size, float inv_sqrt_bs, int inverse, hipStream_t stream);
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream);

@@ -55,6 +55,8 @@ struct tq_linear_s {
     // Staging for the *_host entry points, grown on demand.
     void* d_stage_x = nullptr; size_t stage_x_bytes = 0;
     void* d_stage_y = nullptr; size_t stage_y_bytes = 0;
+    // Rotated-activation workspace of the prefill path, grown on demand.
+    void* d_work = nullptr; size_t work_bytes = 0;
 
     ~tq_linear_s() {
         if (d_primary) (void)hipFree(d_primary);
@@ -64,6 +66,7 @@ struct tq_linear_s {
         if (d_tables) (void)hipFree(d_tables);
         if (d_stage_x) (void)hipFree(d_stage_x);
         if (d_stage_y) (void)hipFree(d_stage_y);
+        if (d_work) (void)hipFree(d_work);
     }
 };
 
@@ -239,6 +242,13 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
         }
         if (h->view.mode >= tq::kShared5) {
             set_error("tq_linear_forward: 5-bit primary is not supported by the fused kernels"); return 1;
+        }
+        if (tq::prefill_supported(h->view, x_dtype, batch)) {
+            // Dense contraction: rotate once, dequantise tiles to bf16 in LDS, MFMA.  The first call
+            // with a larger batch allocates the rotated-activation workspace (not capturable in a graph).
+            if (!ensure_stage(&h->d_work, &h->work_bytes, tq::prefill_workspace_bytes(h->view, batch))) return 1;
+            return hip_ok(tq::launch_prefill(h->view, x_dev, x_dtype, batch, y_dev, y_dtype, h->d_work,
+                                             static_cast<hipStream_t>(stream)), "tq_prefill launch") ? 0 : 1;
         }
         return hip_ok(tq::launch_gemv(h->view, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(),
                                       static_cast<hipStream_t>(stream)), "tq_gemv launch") ? 0 : 1;
