@@ -59,6 +59,17 @@ def lib():
         L.tq_linear_free.restype = None
         L.tq_wht_rotate.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_int, C.c_void_p]
         L.tq_wht_rotate_host.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_int]
+        L.tq_generate_codebook.argtypes = [C.c_int, _f32p, _f32p]
+        L.tq_best_block_size.restype = C.c_uint32
+        L.tq_best_block_size.argtypes = [C.c_int, C.c_uint32]
+        L.tq_quantize_weight.argtypes = [C.c_void_p, C.c_int, C.c_int, _f32p, C.c_int, _f32p, C.c_int, C.c_int, C.c_int,
+                                         C.c_uint32, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, _u32p]
+        L.tq_quantize_weight_host.argtypes = [_f32p, C.c_int, C.c_int, _f32p, C.c_int, _f32p, C.c_int, C.c_int, C.c_int,
+                                              C.c_uint32, C.c_int, _u8p, _u8p, _f32p, _u32p]
+        L.tq_fit_layer_codebooks.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_uint32, C.c_int, C.c_int, _f32p, C.c_int,
+                                             C.c_int, _f32p, _f32p]
+        L.tq_fit_layer_codebooks_host.argtypes = [_f32p, C.c_int, C.c_int, C.c_uint32, C.c_int, C.c_int, _f32p, C.c_int,
+                                                  C.c_int, _f32p, _f32p]
         _lib = L
     return _lib
 
@@ -187,3 +198,73 @@ def apply_wht_rotation(matrix, seed, block_size):
 def apply_inverse_wht_rotation(matrix, seed, block_size):
     """Mirror of turboquant::apply_inverse_wht_rotation (include/turboquant/quantizer.h:37-42)."""
     return _rotate(matrix, seed, block_size, 1)
+
+
+class Codebook:
+    """Mirror of turboquant::Codebook (include/turboquant/codebook.h:24-29)."""
+
+    def __init__(self, centroids, bits):
+        self.centroids = np.ascontiguousarray(centroids, dtype=np.float32)
+        self.bits = int(bits)
+        self.boundaries = ((self.centroids[:-1] + self.centroids[1:]) * np.float32(0.5)).astype(np.float32)
+
+
+def generate_codebook(bits):
+    """Mirror of turboquant::generate_codebook (include/turboquant/codebook.h:33)."""
+    c = np.empty(32, dtype=np.float32)
+    n = lib().tq_generate_codebook(bits, _p(c, _f32p), None)
+    if n < 0:
+        raise ValueError(last_error())
+    return Codebook(c[:n].copy(), bits)
+
+
+class QuantizedWeight:
+    """Mirror of turboquant::QuantizedWeight (include/turboquant/quantizer.h:22-27), numpy tensors."""
+
+    def __init__(self, packed_primary, packed_residual, norms, seeds):
+        self.packed_primary = packed_primary
+        self.packed_residual = packed_residual
+        self.norms = norms
+        self.seeds = seeds
+
+
+def quantize_weight(weight, primary_codebook, residual_codebook, primary_bits=4, residual_bits=4,
+                    block_size=512, shared_rotation=False):
+    """Mirror of turboquant::quantize_weight (include/turboquant/quantizer.h:54-60) on the GPU."""
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    if w.ndim != 2:
+        raise ValueError("weight must be [out, in]")
+    out, inf = w.shape
+    pp = np.empty((out, inf // 2 if primary_bits <= 4 else inf), dtype=np.uint8)
+    pr = np.empty((out, inf // 2), dtype=np.uint8)
+    norms = np.empty(out, dtype=np.float32)
+    seeds = np.empty(3, dtype=np.uint32)
+    cp = np.ascontiguousarray(primary_codebook.centroids, dtype=np.float32)
+    cr = np.ascontiguousarray(residual_codebook.centroids, dtype=np.float32)
+    rc = lib().tq_quantize_weight_host(_p(w, _f32p), out, inf, _p(cp, _f32p), len(cp), _p(cr, _f32p), len(cr),
+                                       primary_bits, residual_bits, block_size, int(shared_rotation),
+                                       _p(pp, _u8p), _p(pr, _u8p), _p(norms, _f32p), _p(seeds, _u32p))
+    if rc != 0:
+        raise ValueError(last_error())
+    return QuantizedWeight(pp, pr, norms, seeds)
+
+
+def fit_layer_codebooks(weight, block_size, primary_bits=4, residual_bits=4, global_primary=None, iterations=100):
+    """Per-layer codebooks as the reference's converter fits them (src/converter.cpp:291-372)."""
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    g = global_primary if global_primary is not None else generate_codebook(primary_bits)
+    gc = np.ascontiguousarray(g.centroids, dtype=np.float32)
+    cp = np.empty(32, dtype=np.float32)
+    cr = np.empty(32, dtype=np.float32)
+    rc = lib().tq_fit_layer_codebooks_host(_p(w, _f32p), w.shape[0], w.shape[1], block_size, primary_bits,
+                                           residual_bits, _p(gc, _f32p), len(gc), iterations, _p(cp, _f32p), _p(cr, _f32p))
+    if rc != 0:
+        raise ValueError(last_error())
+    cbp = Codebook(cp[:1 << primary_bits].copy(), primary_bits)
+    cbr = Codebook(cr[:1 << residual_bits].copy(), residual_bits) if residual_bits > 0 else generate_codebook(4)
+    return cbp, cbr
+
+
+def best_block_size(in_features, max_block_size=512):
+    """Block-size rule of the reference's converter (src/converter.cpp:228-240)."""
+    return int(lib().tq_best_block_size(in_features, max_block_size))

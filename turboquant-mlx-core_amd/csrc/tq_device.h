@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string>
 
 namespace tq {
 
@@ -52,6 +53,29 @@ hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t 
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream);
 hipError_t launch_combine_planes(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,
                                  size_t plane_bytes, hipStream_t stream);
+
+// Host-side error reporting shared by the C-ABI translation units (thread-local message).
+void set_error(const std::string& msg);
+bool hip_ok(hipError_t e, const char* what);
+
+// Offline quantizer (tq_quantize.hip).
+struct QuantArgsHost {
+    const float* w; float* orig_norm; double* recon_partial; float* scaled_out;
+    uint8_t* packed_primary; uint8_t* packed_residual;
+    const float* tables;     // device: [0..31] cP, [32..62] bP, [64..79] cR, [80..94] bR
+    int out, in, n_primary, n_residual, primary_bits, residual_bits, shared_rotation;
+    uint32_t bs, seed_p, seed_r;
+    float scale_factor, inv_scale, inv_sqrt_bs;
+    int quantize;            // 0: only emit the rotated * sqrt(in) samples
+};
+hipError_t launch_row_norms(const float* w, float* norms, int out, int in, hipStream_t stream);
+hipError_t launch_derive_seeds(const float* w, size_t n_floats, uint32_t* seeds_dev, hipStream_t stream);
+hipError_t launch_quantize_rows(const QuantArgsHost& h, hipStream_t stream);
+hipError_t launch_finish_norms(const float* orig, const double* partial, float* norms, int out, int slabs,
+                               hipStream_t stream);
+hipError_t launch_lloyd_pass(const float* data, size_t n, const float* bounds_dev, int nc, int subtract,
+                             const float* gcent_dev, const float* gbounds_dev, int ngc,
+                             double* part_sum, unsigned long long* part_cnt, int workgroups, hipStream_t stream);
 
 // True when the fast wave-per-slab kernels can handle this shape.
 inline bool shape_supported(int in_features, uint32_t block_size) {

@@ -15,9 +15,10 @@
 #include "tq_device.h"
 
 namespace {
-
 thread_local std::string g_last_error;
+}
 
+namespace tq {
 void set_error(const std::string& msg) { g_last_error = msg; }
 
 bool hip_ok(hipError_t e, const char* what) {
@@ -25,6 +26,11 @@ bool hip_ok(hipError_t e, const char* what) {
     set_error(std::string(what) + ": " + hipGetErrorString(e));
     return false;
 }
+}  // namespace tq
+
+namespace {
+using tq::set_error;
+using tq::hip_ok;
 
 int device_cu_count() {
     static int cus = 0;
