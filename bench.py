@@ -30,28 +30,48 @@ def algorithmic_bytes(out, inf, batch, x_bytes, y_bytes):
     return out * inf + 4 * out + 128 + batch * inf * x_bytes + batch * out * y_bytes
 
 
-def make_layer(tq, torch, out, inf, bs, seed, shared=True):
-    """Synthetic TQ8 tensors generated on the GPU: uniformly random 4-bit indices in both
-    planes, corrected norms ~U(0.5, 1.5)*0.02*sqrt(in), analytic 4-bit codebooks."""
+def make_layer(tq, torch, out, inf, bs, seed, sigma, shared=True, per_layer_codebooks=False):
+    """Synthetic layer of BASELINE.json's recipe, produced entirely on the GPU: fp32 weights
+    ~N(0, sigma^2) with 1% of the entries drawn from sigma * Student-t(3) (torch Philox generator,
+    seeded), quantized by this library's GPU quantizer (the reference's quantize_weight pipeline)
+    with analytic or per-layer Lloyd-Max codebooks."""
     import ctypes as C
     import numpy as np
+    f32p, u32p = C.POINTER(C.c_float), C.POINTER(C.c_uint32)
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
-    pp = torch.randint(0, 256, (out, inf // 2), dtype=torch.uint8, device="cuda", generator=g)
-    pr = torch.randint(0, 256, (out, inf // 2), dtype=torch.uint8, device="cuda", generator=g)
-    norms = (torch.rand(out, device="cuda", generator=g) + 0.5) * (0.02 * inf ** 0.5)
-    cb = np.array([-2.732590, -2.069017, -1.618046, -1.256231, -0.942340, -0.656759, -0.388048, -0.128395,
-                   0.128395, 0.388048, 0.656759, 0.942340, 1.256231, 1.618046, 2.069017, 2.732590], np.float32)
-    seeds = np.array([0xCAFEBABE, 0 if shared else 0x1234567, bs], np.uint32)
+    w = torch.randn(out, inf, device="cuda", generator=g) * sigma
+    g.manual_seed(seed + 1)
+    mask = torch.rand(out, inf, device="cuda", generator=g) < 0.01
+    z = torch.randn(4, int(mask.sum().item()), device="cuda", generator=g)
+    w[mask] = sigma * z[0] / torch.sqrt((z[1] ** 2 + z[2] ** 2 + z[3] ** 2) / 3.0)
+    del mask, z
     L = tq.lib()
+    cbp = np.empty(32, np.float32)
+    cbr = np.empty(32, np.float32)
+    L.tq_generate_codebook(4, cbp.ctypes.data_as(f32p), None)
+    L.tq_generate_codebook(4, cbr.ctypes.data_as(f32p), None)
+    if per_layer_codebooks:
+        glob = cbp.copy()
+        if L.tq_fit_layer_codebooks(w.data_ptr(), out, inf, bs, 4, 4, glob.ctypes.data_as(f32p), 16, 100,
+                                    cbp.ctypes.data_as(f32p), cbr.ctypes.data_as(f32p)) != 0:
+            raise RuntimeError(tq.last_error())
+    pp = torch.empty(out, inf // 2, dtype=torch.uint8, device="cuda")
+    pr = torch.empty(out, inf // 2, dtype=torch.uint8, device="cuda")
+    norms = torch.empty(out, dtype=torch.float32, device="cuda")
+    seeds = np.zeros(3, np.uint32)
+    if L.tq_quantize_weight(w.data_ptr(), out, inf, cbp.ctypes.data_as(f32p), 16, cbr.ctypes.data_as(f32p), 16,
+                            4, 4, bs, int(shared), pp.data_ptr(), pr.data_ptr(), norms.data_ptr(),
+                            seeds.ctypes.data_as(u32p)) != 0:
+        raise RuntimeError(tq.last_error())
+    del w
     h = L.tq_linear_create_from_device(inf, out, pp.data_ptr(), inf // 2, pr.data_ptr(), inf // 2, norms.data_ptr(),
-                                       seeds.ctypes.data_as(C.POINTER(C.c_uint32)),
-                                       cb.ctypes.data_as(C.POINTER(C.c_float)), 16,
-                                       cb.ctypes.data_as(C.POINTER(C.c_float)), 16, bs)
+                                       seeds.ctypes.data_as(u32p), cbp.ctypes.data_as(f32p), 16,
+                                       cbr.ctypes.data_as(f32p), 16, bs)
     if not h:
         raise RuntimeError(tq.last_error())
     torch.cuda.synchronize()
-    return h, dict(pp=pp, pr=pr, norms=norms, cb=cb, seeds=seeds)
+    return h, dict(pp=pp, pr=pr, norms=norms, cbp=cbp[:16].copy(), cbr=cbr[:16].copy(), seeds=seeds)
 
 
 def time_graph(tq, torch, handles, x, y, xcode, batch, steps, warmup):
@@ -92,17 +112,17 @@ def cpu_baseline(torch, tensors, out, inf, bs, x_f32):
     pp = tensors["pp"].cpu().numpy()
     pr = tensors["pr"].cpu().numpy()
     norms = tensors["norms"].cpu().numpy()
-    cb = o.Codebook(tensors["cb"], 4)
+    cbp, cbr = o.Codebook(tensors["cbp"], 4), o.Codebook(tensors["cbr"], 4)
     qw = o.QuantizedWeight(pp, pr, norms, tensors["seeds"])
     o.set_threads(1)
     t0 = time.perf_counter()
-    W = o.dequantize_weight_cpu(qw, cb, cb, bs)
+    W = o.dequantize_weight_cpu(qw, cbp, cbr, bs)
     y = o.matmul_xwT(x_f32, W, acc_double=False)
     dt = time.perf_counter() - t0
     threads = min(16, os.cpu_count() or 1)
     o.set_threads(threads)
     t0 = time.perf_counter()
-    W = o.dequantize_weight_cpu(qw, cb, cb, bs)
+    W = o.dequantize_weight_cpu(qw, cbp, cbr, bs)
     y_mt = o.matmul_xwT(x_f32, W, acc_double=False)
     dt_mt = time.perf_counter() - t0
     o.set_threads(1)
@@ -137,7 +157,8 @@ def main():
 
     # ---- headline: lm_head 151936 x 2048, bf16 x, fp32 y, batch 1 -------------------
     out, inf, bs = 151936, 2048, 512
-    handle, tensors = make_layer(tq, torch, out, inf, bs, seed=0xCAFEBABE + 1)
+    handle, tensors = make_layer(tq, torch, out, inf, bs, seed=0xCAFEBABE + 1, sigma=0.02, shared=True,
+                                 per_layer_codebooks=True)
     g = torch.Generator(device="cuda"); g.manual_seed(0xCAFEBABE + 3)
     x = torch.randn(1, inf, device="cuda", generator=g).to(torch.bfloat16)
     y = torch.empty(1, out, device="cuda", dtype=torch.float32)
@@ -158,8 +179,9 @@ def main():
         "scaling": "weak",
         "vs_baseline": (1e6 / us) / REFERENCE_PUBLISHED_TOK_S,
         "dtype": "f32",
-        "data": "synthetic: uniformly random 4-bit primary/residual indices, random row norms, analytic "
-                "16-entry codebooks, bf16 N(0,1) activations; all generated on the GPU",
+        "data": "synthetic: fp32 weights N(0,0.02^2) with 1% Student-t(3) tails, quantized on the GPU by this "
+                "library's TQ8 quantizer with per-layer Lloyd-Max codebooks (shared rotation, block 512); "
+                "bf16 N(0,1) activations",
         "config": {"workload": "Qwen2.5-0.5B lm_head as TQ8 linear 151936x2048, shared rotation, block 512, "
                                "x bf16 [1,2048], y f32 [1,151936]",
                    "baseline_note": "vs_baseline divides by the reference's published 47.3 tok/s (Apple Silicon)"},
@@ -192,7 +214,7 @@ def main():
         return
     out1, in1 = 4096, 4096
     copies = 32                         # 32 x 16.8 MB > 256 MB of last-level cache: HBM-resident timing
-    handles = [make_layer(tq, torch, out1, in1, bs, seed=100 + i)[0] for i in range(copies)]
+    handles = [make_layer(tq, torch, out1, in1, bs, seed=100 + 2 * i, sigma=0.02, shared=True)[0] for i in range(copies)]
     x1 = torch.randn(1, in1, device="cuda", generator=g)
     y1 = torch.empty(1, out1, device="cuda", dtype=torch.float32)
     steps1 = max(args.steps, copies) // copies * copies
@@ -204,6 +226,40 @@ def main():
                                        "hbm_frac": B1 / (us_hbm * 1e-6) / 1e9 / HBM_PEAK_GBS}
     for h in handles:
         tq.lib().tq_linear_free(h)
+    # the library default of the reference is dual rotation (include/turboquant/quantizer.h:15)
+    handles = [make_layer(tq, torch, out1, in1, bs, seed=300 + 2 * i, sigma=0.02, shared=False)[0] for i in range(copies)]
+    us_dual = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
+    extra["gemv_4096x4096_f32_bs1_dual_rotation"] = {"us_per_layer_hbm_resident": us_dual,
+                                                     "hbm_frac": B1 / (us_dual * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    for h in handles:
+        tq.lib().tq_linear_free(h)
+    del handles
+    torch.cuda.empty_cache()
+
+    # ---- prefill: Qwen2.5-32B up-projection 27648 x 5120, M = 512 and 2048, bf16 in / bf16 out ----
+    outp, inp = 27648, 5120
+    hp, _ = make_layer(tq, torch, outp, inp, bs, seed=500, sigma=0.01, shared=True, per_layer_codebooks=True)
+    for M in (512, 2048):
+        xp = torch.randn(M, inp, device="cuda", generator=g).to(torch.bfloat16)
+        yp = torch.empty(M, outp, device="cuda", dtype=torch.bfloat16)
+        L = tq.lib()
+        for _ in range(2):
+            if L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None) != 0:
+                raise RuntimeError(tq.last_error())
+        torch.cuda.synchronize()
+        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 10
+        st.record()
+        for _ in range(reps):
+            L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None)
+        en.record()
+        torch.cuda.synchronize()
+        usp = st.elapsed_time(en) * 1e3 / reps
+        flops = 2.0 * M * outp * inp
+        extra[f"prefill_27648x5120_M{M}_bf16"] = {"us_per_layer": usp, "tflops": flops / usp / 1e6,
+                                                  "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
+                                                  "includes": "activation rotation kernel + dequant/MFMA GEMM kernel"}
+    tq.lib().tq_linear_free(hp)
     finish(args, torch, extra, result)
 
 
