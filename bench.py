@@ -22,6 +22,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152403.7 KiB + 632.3 KiB.
+MEASURED_TRAFFIC_BYTES = 312770253
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
 
@@ -187,7 +190,7 @@ def main():
                    "baseline_note": "vs_baseline divides by the reference's published 47.3 tok/s (Apple Silicon)"},
         "us_per_layer": us,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "tq_gemv_kernel<shared,1,2,1024>", "algorithmic_bytes": B},
     }
 
