@@ -241,7 +241,7 @@ __device__ __forceinline__ void rotate_row_shared(const void* x, int x_dtype, si
     }
 }
 
-template <int MODE, int NB, int R, int MAXT>
+template <int MODE, int NB, int R, int MAXT, int NS>
 __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     constexpr int V = R * NB;                       // sums produced per row group
     __shared__ __align__(16) char smem[kRegionBytes + kPartialBytes];
@@ -271,30 +271,40 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     const int r_end = (int)((gs + 1) * out / ts);
 
     // Idle runs re-read a valid address; their rotated activations are 0.
-    const uint8_t* pp = combined ? a.L.packed_combined + (act_a ? col_a : 0) : a.L.packed_primary + (act_a ? (col_a >> 1) : 0);
-    const uint8_t* pr = combined ? a.L.packed_combined + (act_b ? col_b : 0) : a.L.packed_residual + (act_a ? (col_a >> 1) : 0);
+    // Row bases are wave-uniform (scalar); the lane adds a fixed 32-bit byte offset.
+    const uint8_t* pp = combined ? a.L.packed_combined : a.L.packed_primary;
+    const uint8_t* pr = combined ? a.L.packed_combined : a.L.packed_residual;
+    const uint32_t off_p = combined ? (uint32_t)(act_a ? col_a : 0) : (uint32_t)(act_a ? (col_a >> 1) : 0);
+    const uint32_t off_r = combined ? (uint32_t)(act_b ? col_b : 0) : off_p;
 
-    uint4 P[2][R], Q[2][R];
+    uint4 P[NS][R], Q[NS][R];                 // NS-stage register ring of row groups in flight
+    float nrm[NS];                            // norm of the row this lane will store (lanes < V)
     auto fetch = [&](int buf, int r0) {
         if (r0 + R <= r_end) {                               // wave-uniform: a full group, straight-line
 #pragma unroll
             for (int i = 0; i < R; ++i) {
-                P[buf][i] = load_stream16(pp + (size_t)(r0 + i) * row_bytes);
-                if constexpr (use_res) Q[buf][i] = load_stream16(pr + (size_t)(r0 + i) * row_bytes);
+                const size_t rb = (size_t)(r0 + i) * row_bytes;
+                P[buf][i] = load_stream16(pp + rb + off_p);
+                if constexpr (use_res) Q[buf][i] = load_stream16(pr + rb + off_r);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < R; ++i) {
                 if (r0 + i < r_end) {
-                    P[buf][i] = load_stream16(pp + (size_t)(r0 + i) * row_bytes);
-                    if constexpr (use_res) Q[buf][i] = load_stream16(pr + (size_t)(r0 + i) * row_bytes);
+                    const size_t rb = (size_t)(r0 + i) * row_bytes;
+                    P[buf][i] = load_stream16(pp + rb + off_p);
+                    if constexpr (use_res) Q[buf][i] = load_stream16(pr + rb + off_r);
                 }
             }
         }
+        // The norm travels with its rows so the store at the end of the group never waits on memory.
+        const int rn = r0 + (lane % V) / NB;
+        nrm[buf] = a.L.norms[rn < out ? rn : out - 1];
     };
 
-    // First weight fetch goes out before the prologue so its latency overlaps it.
-    fetch(0, r_begin);
+    // The first NS-1 groups go out before the prologue so their latency overlaps it.
+#pragma unroll
+    for (int u = 0; u < NS - 1; ++u) fetch(u, r_begin + u * R);
 
     // Rotated activations, kept in registers for the whole kernel.
     float xt[NB][kChunk];
@@ -352,6 +362,7 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
 
     auto consume = [&](int buf, int r0, int it) {
         float acc[V];
+        const float row_scale = a.out_scale * nrm[buf];
         if (r0 + R <= r_end) {                               // wave-uniform: a full group, straight-line
 #pragma unroll
             for (int i = 0; i < R; ++i) decode_row(buf, i, acc);
@@ -370,7 +381,7 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
         const bool owner = lane < V && r < r_end;
 
         if (a.W == 1) {
-            if (owner) store_scalar(a.y, a.y_dtype, (size_t)b * out + r, total * (a.out_scale * a.L.norms[r]));
+            if (owner) store_scalar(a.y, a.y_dtype, (size_t)b * out + r, total * row_scale);
         } else {
             float* buf_base = partial + (it & 1) * (16 * 16);
             if (lane < V) buf_base[wave * V + lane] = total;
@@ -378,28 +389,30 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
             if (slab == 0 && owner) {
                 float t = 0.0f;
                 for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * V + lane];
-                store_scalar(a.y, a.y_dtype, (size_t)b * out + r, t * (a.out_scale * a.L.norms[r]));
+                store_scalar(a.y, a.y_dtype, (size_t)b * out + r, t * row_scale);
             }
         }
     };
 
-    // Double-buffered main loop (unrolled by two so the buffers are static).  The
-    // trip count is uniform over the grid; a stream whose range ends early skips
-    // the work of the missing rows.
-    for (int it = 0; it < a.iters; it += 2) {
-        const int r0 = r_begin + it * R;
-        fetch(1, r0 + R);
-        consume(0, r0, it);
-        if (it + 1 < a.iters) {
-            fetch(0, r0 + 2 * R);
-            consume(1, r0 + R, it + 1);
+    // Main loop over the register ring (unrolled NS times so the stages are static): group it+NS-1
+    // is requested while group it is decoded, which keeps NS-1 groups of loads in flight per wave.
+    // The trip count is uniform over the grid; a stream whose range ends early skips the work of
+    // the missing rows.
+    for (int it0 = 0; it0 < a.iters; it0 += NS) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            const int it = it0 + u;
+            if (it < a.iters) {
+                fetch((u + NS - 1) % NS, r_begin + (it + NS - 1) * R);
+                consume(u, r_begin + it * R, it);
+            }
         }
     }
 }
 
-template <int MODE, int NB, int R, int MAXT>
+template <int MODE, int NB, int R, int MAXT, int NS>
 static hipError_t launch_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
-    hipLaunchKernelGGL((tq_gemv_kernel<MODE, NB, R, MAXT>), dim3(grid), dim3(threads), 0, stream, a);
+    hipLaunchKernelGGL((tq_gemv_kernel<MODE, NB, R, MAXT, NS>), dim3(grid), dim3(threads), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -425,10 +438,16 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     a.groups = 0;
     a.iters = (max_rows + R - 1) / R;
 
+    int ns = 2;
+    if (const char* e = getenv("TQ_GEMV_NS")) ns = atoi(e);
+    if (NB == 1 && MODE != kDual && R == 2 && ns == 3) return launch_one<MODE, NB, 2, MAXT, 3>(a, grid, threads, stream);
+    if (NB == 1 && MODE != kDual && R == 2 && ns == 4) return launch_one<MODE, NB, 2, MAXT, 4>(a, grid, threads, stream);
+    if (NB == 1 && MODE != kDual && R == 1 && ns == 4) return launch_one<MODE, NB, 1, MAXT, 4>(a, grid, threads, stream);
+    if (NB == 1 && MODE != kDual && R == 1 && ns == 8) return launch_one<MODE, NB, 1, MAXT, 8>(a, grid, threads, stream);
     switch (R) {
-        case 4: return launch_one<MODE, NB, 4, MAXT>(a, grid, threads, stream);
-        case 2: return launch_one<MODE, NB, 2, MAXT>(a, grid, threads, stream);
-        default: return launch_one<MODE, NB, 1, MAXT>(a, grid, threads, stream);
+        case 4: return launch_one<MODE, NB, 4, MAXT, 2>(a, grid, threads, stream);
+        case 2: return launch_one<MODE, NB, 2, MAXT, 2>(a, grid, threads, stream);
+        default: return launch_one<MODE, NB, 1, MAXT, 2>(a, grid, threads, stream);
     }
 }
 
