@@ -118,23 +118,38 @@ __device__ __forceinline__ void lookup32(const uint4& P, const uint4& Q, const c
 
 constexpr int kLut256Bytes = 256 * 256;          // 256 entries x 64 lanes x 4 B
 constexpr int kTab16Bytes = 16 * 256;
-constexpr int kRegionBytes = kLut256Bytes;       // decode tables; doubles as activation hand-over space
+constexpr int kRegionBytes = kLut256Bytes;       // decode tables
 constexpr int kRegionFloats = kRegionBytes / 4;
 constexpr int kPartialBytes = 2 * 16 * 16 * 4;   // [2 buffers][<=16 waves][<=16 values]
+constexpr int kStageBytes = kSlab * 4;           // one slab image of rotated activations
 constexpr int kTile = 512;                       // columns rotated by one wave in the prologue (8 per lane)
 
 // Rotate one 512-column tile of an activation row: lane owns 8 consecutive columns.
-// Valid for block sizes up to 512 (a block never straddles a tile).
-__device__ __forceinline__ void rotate_tile(const void* x, int x_dtype, size_t row_off, int col, bool active,
+// Valid for block sizes up to 512 (a block never straddles a tile).  The raw load is split
+// from the arithmetic so that a wave can have the loads of all its tiles in flight at once.
+struct TileRaw { uint4 a, b; };
+
+__device__ __forceinline__ TileRaw load_tile_raw(const void* x, int x_dtype, size_t row_off, int col) {
+    TileRaw r;
+    if (x_dtype == kF32) {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const float*>(x) + row_off + col);
+        r.a = p[0]; r.b = p[1];
+    } else {
+        r.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + row_off + col);
+        r.b = make_uint4(0, 0, 0, 0);
+    }
+    return r;
+}
+
+__device__ __forceinline__ void rotate_tile(const TileRaw& raw, int x_dtype, int col, bool active,
                                             uint32_t seed, uint32_t bs, int lane, float (&v)[8]) {
     if (active) {
         if (x_dtype == kF32) {
-            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(x) + row_off + col);
-            const float4 a = p[0], b = p[1];
-            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            const uint32_t w[8] = {raw.a.x, raw.a.y, raw.a.z, raw.a.w, raw.b.x, raw.b.y, raw.b.z, raw.b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = __builtin_bit_cast(float, w[j]);
         } else {
-            const uint4 t = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + row_off + col);
-            const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+            const uint32_t w[4] = {raw.a.x, raw.a.y, raw.a.z, raw.a.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if (x_dtype == kBF16) {
@@ -170,81 +185,116 @@ __device__ __forceinline__ int stage_index(int col_in_slab) {
     }
 }
 
-// Rotated activations H (s (.) x) of one batch row for every lane of the workgroup.
-// The waves rotate 512-column tiles cooperatively (block sizes up to 512), or run the
-// butterfly stage by stage in LDS (larger blocks), and each lane then picks up the 32
-// values of the columns it owns.  Rows wider than the staging space are handled in
-// passes of 8 slabs.
-template <bool SPLIT>
-__device__ __forceinline__ void rotate_row_shared(const void* x, int x_dtype, size_t row_off, int in_features,
-                                                  uint32_t seed, uint32_t bs, float* stage,
-                                                  int wave, int nwaves, int lane, int slab,
-                                                  bool act_a, bool act_b, float (&xt)[kChunk]) {
-    const int tiles = (in_features + kTile - 1) / kTile;
-    constexpr int kTilesPerPass = kRegionFloats / kTile;       // 32 tiles = 8 slabs
-    for (int t0 = 0; t0 < tiles; t0 += kTilesPerPass) {
-        const int t1 = (t0 + kTilesPerPass < tiles) ? t0 + kTilesPerPass : tiles;
-        const int col_base = t0 * kTile;
-        if (bs <= (uint32_t)kTile) {
-            for (int t = t0 + wave; t < t1; t += nwaves) {
-                const int col = t * kTile + lane * 8;
-                float v[8];
-                rotate_tile(x, x_dtype, row_off, col, col < in_features, seed, bs, lane, v);
-                const int rel = col - col_base;
-                float* dst = stage + (rel >> 11) * kSlab + stage_index<SPLIT>(rel & (kSlab - 1));
+// Load 16 consecutive activations and widen them to fp32.
+__device__ __forceinline__ void load_run16(const void* x, int x_dtype, size_t elem, float (&v)[16]) {
+    if (x_dtype == kF32) {
+        const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(x) + elem);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) dst[j * kWave] = v[j];      // 8 columns stay inside one 16-run
-            }
-            __syncthreads();
-        } else {
-            // Generic path: signed activations in natural order, one butterfly stage per barrier
-            // (same (a+b, a-b) pairs and stage order as reference src/rotation.cpp:14-25).
-            const int ncols = ((t1 * kTile < in_features) ? t1 * kTile : in_features) - col_base;
-            const int tid = wave * kWave + lane, nthreads = nwaves * kWave;
-            for (int c = tid; c < ncols; c += nthreads) {
-                const size_t e = row_off + col_base + c;
-                float v;
-                if (x_dtype == kF32) v = static_cast<const float*>(x)[e];
-                else if (x_dtype == kBF16) v = bf16_bits_to_float(static_cast<const uint16_t*>(x)[e]);
-                else v = (float)static_cast<const _Float16*>(x)[e];
-                stage[c] = v * sign_of(seed, (uint32_t)(col_base + c) & (bs - 1));
-            }
-            __syncthreads();
-            for (uint32_t h = 1; h < bs; h <<= 1) {
-                for (int q = tid; q < (ncols >> 1); q += nthreads) {
-                    const int i = ((q / (int)h) * 2 * (int)h) + (q % (int)h);
-                    const float u = stage[i], w = stage[i + h];
-                    stage[i] = u + w;
-                    stage[i + h] = u - w;
+        for (int i = 0; i < 4; ++i) {
+            const float4 t = p[i];
+            v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+        }
+    } else {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + elem);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint4 t = p[i];
+            const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (x_dtype == kBF16) {
+                    v[8 * i + 2 * j]     = bf16_bits_to_float(w[j] & 0xffffu);
+                    v[8 * i + 2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+                } else {
+                    v[8 * i + 2 * j]     = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] & 0xffffu));
+                    v[8 * i + 2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] >> 16));
                 }
-                __syncthreads();
             }
         }
-        const int s_rel = slab - (t0 >> 2);
-        if (s_rel >= 0 && s_rel < (kTilesPerPass >> 2)) {
-            if (bs <= (uint32_t)kTile) {
-                const float* src = stage + s_rel * kSlab + lane;
+    }
+}
+
+// Rotated activations H (s (.) x) of the columns one lane owns, computed by the wave on its own
+// (no LDS, no barrier): used when a workgroup has few row streams, so nothing would be shared.
+// Split ownership: the two 16-column runs are transformed as 16 values per lane; a 2048-column
+// block additionally pairs the runs in a last stage.  Block sizes up to 2048.
+template <bool SPLIT>
+__device__ __forceinline__ void rotate_private(const void* x, int x_dtype, size_t row_off, int col_a, int col_b,
+                                               bool act_a, bool act_b, uint32_t seed, uint32_t bs, int lane,
+                                               float (&xt)[kChunk]) {
+    if constexpr (SPLIT) {
+        float va[16], vb[16];
+        if (act_a) {
+            load_run16(x, x_dtype, row_off + col_a, va);
 #pragma unroll
-                for (int k = 0; k < kChunk; ++k)
-                    xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
-            } else {
-                const int ca = s_rel * kSlab + (SPLIT ? 16 * lane : 32 * lane);
-                const int cb = SPLIT ? ca + 1024 : ca + 16;
+            for (int k = 0; k < 16; ++k) va[k] *= sign_of(seed, ((uint32_t)col_a + k) & (bs - 1));
+        } else {
 #pragma unroll
-                for (int k = 0; k < 16; ++k) {
-                    xt[k] = act_a ? stage[ca + k] : 0.0f;
-                    xt[16 + k] = act_b ? stage[cb + k] : 0.0f;
-                }
-            }
+            for (int k = 0; k < 16; ++k) va[k] = 0.0f;
+        }
+        if (act_b) {
+            load_run16(x, x_dtype, row_off + col_b, vb);
+#pragma unroll
+            for (int k = 0; k < 16; ++k) vb[k] *= sign_of(seed, ((uint32_t)col_b + k) & (bs - 1));
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) vb[k] = 0.0f;
+        }
+        const uint32_t bsr = bs > 1024u ? 1024u : bs;     // stages inside one 1024-column run
+        fwht_lanes<16>(va, bsr, lane);
+        fwht_lanes<16>(vb, bsr, lane);
+        if (bs > 1024u) {                                  // h = 1024: column c pairs with c + 1024
+#pragma unroll
+            for (int k = 0; k < 16; ++k) { const float p = va[k], q = vb[k]; va[k] = p + q; vb[k] = p - q; }
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k) { xt[k] = va[k]; xt[16 + k] = vb[k]; }
+    } else {
+        if (act_a) {
+            load_chunk(x, x_dtype, row_off + col_a, xt);
+#pragma unroll
+            for (int k = 0; k < kChunk; ++k) xt[k] *= sign_of(seed, ((uint32_t)col_a + k) & (bs - 1));
+        } else {
+#pragma unroll
+            for (int k = 0; k < kChunk; ++k) xt[k] = 0.0f;
+        }
+        fwht_lane32(xt, bs, lane);
+    }
+}
+
+// Shared variant for narrow layers (at most 8 tiles = 2 slabs, block sizes up to 512): wave t
+// rotates 512-column tile t (8 values per lane), the slabs are handed over one at a time
+// through an 8 KB staging image (value k of lane l at float index k*64 + l), and every wave picks
+// up the 32 values of its own columns.  `raw` must hold tile `wave`'s activations.
+template <bool SPLIT>
+__device__ __forceinline__ void rotate_shared(const TileRaw& raw, int x_dtype, int in_features, int W,
+                                              uint32_t seed, uint32_t bs, float* stage, int wave, int lane,
+                                              int slab, bool act_a, bool act_b, float (&xt)[kChunk]) {
+    const int col = wave * kTile + lane * 8;
+    const bool mine = wave * kTile < in_features;           // wave-uniform
+    float v[8];
+    if (mine) rotate_tile(raw, x_dtype, col, col < in_features, seed, bs, lane, v);
+    for (int p = 0; p < W; ++p) {
+        if (p > 0) __syncthreads();                          // previous slab image has been read
+        if (mine && (wave >> 2) == p) {
+            float* dst = stage + stage_index<SPLIT>(col & (kSlab - 1));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dst[j * kWave] = v[j];      // 8 columns stay inside one 16-run
         }
         __syncthreads();
+        if (slab == p) {
+            const float* src = stage + lane;
+#pragma unroll
+            for (int k = 0; k < kChunk; ++k)
+                xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
+        }
     }
 }
 
 template <int MODE, int NB, int R, int MAXT, int NS>
 __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     constexpr int V = R * NB;                       // sums produced per row group
-    __shared__ __align__(16) char smem[kRegionBytes + kPartialBytes];
+    __shared__ __align__(16) char smem[kRegionBytes + kPartialBytes + kStageBytes];
     float* partial = reinterpret_cast<float*>(smem + kRegionBytes);   // [2][waves][V]
 
     const int tid = threadIdx.x;
@@ -306,19 +356,15 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
 #pragma unroll
     for (int u = 0; u < NS - 1; ++u) fetch(u, r_begin + u * R);
 
-    // Rotated activations, kept in registers for the whole kernel.
-    float xt[NB][kChunk];
-    float xr[NB][kChunk];   // second rotation, dual mode only
-    {
-        float* stage = reinterpret_cast<float*>(smem);
+    // Prologue.  Everything that has to come from memory is requested first (weights above, then
+    // the activation tile of the shared path and the table values), so the latencies overlap.
+    const bool shared_rot = (a.S >= 4 && a.L.block_size <= (uint32_t)kTile);      // W <= 2: at most 8 tiles
+    TileRaw raw[NB];
+    if (shared_rot) {
+        const int col = wave * kTile + lane * 8;
 #pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            rotate_row_shared<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, a.L.in_features, a.L.seed_primary,
-                                        a.L.block_size, stage, wave, nwaves, lane, slab, act_a, act_b, xt[b]);
-            if constexpr (MODE == kDual)
-                rotate_row_shared<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, a.L.in_features, a.L.seed_residual,
-                                            a.L.block_size, stage, wave, nwaves, lane, slab, act_a, act_b, xr[b]);
-        }
+        for (int b = 0; b < NB; ++b)
+            if (col < a.L.in_features) raw[b] = load_tile_raw(a.x, a.x_dtype, (size_t)b * a.L.in_features, col);
     }
 
     // Decode tables -> LDS, one private column per lane.
@@ -330,7 +376,34 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
             dst[i] = make_float4(v, v, v, v);
         }
     }
-    __syncthreads();
+
+    // Rotated activations, kept in registers for the whole kernel.
+    float xt[NB][kChunk];
+    float xr[NB][kChunk];   // second rotation, dual mode only
+    if (shared_rot) {
+        float* stage = reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (b > 0) __syncthreads();
+            rotate_shared<combined>(raw[b], a.x_dtype, a.L.in_features, a.W, a.L.seed_primary, a.L.block_size,
+                                    stage, wave, lane, slab, act_a, act_b, xt[b]);
+            if constexpr (MODE == kDual) {
+                __syncthreads();
+                rotate_shared<combined>(raw[b], a.x_dtype, a.L.in_features, a.W, a.L.seed_residual, a.L.block_size,
+                                        stage, wave, lane, slab, act_a, act_b, xr[b]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            rotate_private<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, col_a, col_b, act_a, act_b,
+                                     a.L.seed_primary, a.L.block_size, lane, xt[b]);
+            if constexpr (MODE == kDual)
+                rotate_private<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, col_a, col_b, act_a, act_b,
+                                         a.L.seed_residual, a.L.block_size, lane, xr[b]);
+        }
+    }
+    __syncthreads();                                          // tables visible to every wave
 
     auto decode_row = [&](int buf, int i, float (&acc)[V]) {
         float val[kChunk];
@@ -424,7 +497,9 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     if (a.W * kWave > MAXT) return hipErrorInvalidValue;
     a.S = (a.W >= 8) ? 1 : (8 / a.W);
     const int threads = a.W * a.S * kWave;
-    int max_grid = num_cus * 2;
+    // Two workgroups per CU fit (LDS, registers) up to 8 waves each; wider rows run one per CU so
+    // the prologue is not repeated in a second round.
+    int max_grid = (a.W > 8) ? num_cus : num_cus * 2;
     if (const char* e = getenv("TQ_GEMV_GRID")) { int v = atoi(e); if (v > 0) max_grid = v; }
 
     int grid = (out + a.S - 1) / a.S;
@@ -433,7 +508,8 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     const long long ts = (long long)grid * a.S;
     const int max_rows = (int)((out + ts - 1) / ts);        // longest row range of any stream
     // Four rows per group only where the register budget allows it without spilling.
-    int R = (max_rows >= 4 && MAXT <= 512) ? 4 : (max_rows >= 2 ? 2 : 1);
+    int R = (max_rows >= 4 && MAXT <= 512 && NB < 4) ? 4 : (max_rows >= 2 ? 2 : 1);
+    if (MODE == kDual && MAXT > 512) R = 1;
     if (const char* e = getenv("TQ_GEMV_R")) { int v = atoi(e); if (v == 1 || v == 2 || v == 4) R = v; }
     a.groups = 0;
     a.iters = (max_rows + R - 1) / R;
