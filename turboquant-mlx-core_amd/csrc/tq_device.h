@@ -105,13 +105,30 @@ __device__ __forceinline__ float dpp_mov(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
 
-// Value held by lane (lane ^ MASK).
+// Value held by lane (lane ^ MASK), without touching LDS:
+//   1, 2 : DPP quad_perm;  4 : row_shr:4 / row_shl:4 written under complementary bank masks;
+//   8    : DPP row_ror:8;  16, 32 : v_permlane16_swap / v_permlane32_swap (gfx950) plus a select.
 template <int MASK>
 __device__ __forceinline__ float lane_xor(float v) {
     if constexpr (MASK == 1) return dpp_mov<0xB1>(v);        // quad_perm [1,0,3,2]
     else if constexpr (MASK == 2) return dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (MASK == 4) {
+        const int iv = __builtin_bit_cast(int, v);
+        int a = __builtin_amdgcn_update_dpp(iv, iv, 0x114, 0xf, 0xa, false);   // row_shr:4 -> lanes with bit 2 set
+        a = __builtin_amdgcn_update_dpp(a, iv, 0x104, 0xf, 0x5, false);        // row_shl:4 -> lanes with bit 2 clear
+        return __builtin_bit_cast(float, a);
+    }
     else if constexpr (MASK == 8) return dpp_mov<0x128>(v);  // row_ror:8
-    else return __shfl_xor(v, MASK, kWave);
+    else if constexpr (MASK == 16) {
+        const unsigned u = __builtin_bit_cast(unsigned, v);
+        const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+        return __builtin_bit_cast(float, (__lane_id() & 16) ? r[0] : r[1]);
+    } else {
+        static_assert(MASK == 32, "lane_xor: unsupported mask");
+        const unsigned u = __builtin_bit_cast(unsigned, v);
+        const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        return __builtin_bit_cast(float, (__lane_id() & 32) ? r[0] : r[1]);
+    }
 }
 
 // One cross-lane butterfly stage over N values per lane: the lower lane of a pair

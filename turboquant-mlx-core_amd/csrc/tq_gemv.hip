@@ -28,7 +28,6 @@ struct GemvArgs {
     int x_dtype, y_dtype;
     int chunks;      // in / 32
     int W, S;        // slabs per row, row streams per workgroup
-    int groups;      // unused
     int iters;       // uniform trip count: ceil(longest row range / R)
     float out_scale; // inv_scale * inv_sqrt_bs
 };
@@ -214,31 +213,32 @@ __device__ __forceinline__ void load_run16(const void* x, int x_dtype, size_t el
     }
 }
 
+// The 32 activations of the columns one lane owns (two runs of 16, or 32 consecutive), as fp32.
+template <bool SPLIT>
+__device__ __forceinline__ void load_owned(const void* x, int x_dtype, size_t row_off, int col_a, int col_b,
+                                           bool act_a, bool act_b, float (&xin)[kChunk]) {
+    float va[16], vb[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) { va[k] = 0.0f; vb[k] = 0.0f; }
+    if (act_a) load_run16(x, x_dtype, row_off + col_a, va);
+    if (act_b) load_run16(x, x_dtype, row_off + col_b, vb);
+#pragma unroll
+    for (int k = 0; k < 16; ++k) { xin[k] = va[k]; xin[16 + k] = vb[k]; }
+}
+
 // Rotated activations H (s (.) x) of the columns one lane owns, computed by the wave on its own
 // (no LDS, no barrier): used when a workgroup has few row streams, so nothing would be shared.
 // Split ownership: the two 16-column runs are transformed as 16 values per lane; a 2048-column
 // block additionally pairs the runs in a last stage.  Block sizes up to 2048.
 template <bool SPLIT>
-__device__ __forceinline__ void rotate_private(const void* x, int x_dtype, size_t row_off, int col_a, int col_b,
-                                               bool act_a, bool act_b, uint32_t seed, uint32_t bs, int lane,
-                                               float (&xt)[kChunk]) {
+__device__ __forceinline__ void rotate_private(const float (&xin)[kChunk], int col_a, int col_b,
+                                               uint32_t seed, uint32_t bs, int lane, float (&xt)[kChunk]) {
     if constexpr (SPLIT) {
         float va[16], vb[16];
-        if (act_a) {
-            load_run16(x, x_dtype, row_off + col_a, va);
 #pragma unroll
-            for (int k = 0; k < 16; ++k) va[k] *= sign_of(seed, ((uint32_t)col_a + k) & (bs - 1));
-        } else {
-#pragma unroll
-            for (int k = 0; k < 16; ++k) va[k] = 0.0f;
-        }
-        if (act_b) {
-            load_run16(x, x_dtype, row_off + col_b, vb);
-#pragma unroll
-            for (int k = 0; k < 16; ++k) vb[k] *= sign_of(seed, ((uint32_t)col_b + k) & (bs - 1));
-        } else {
-#pragma unroll
-            for (int k = 0; k < 16; ++k) vb[k] = 0.0f;
+        for (int k = 0; k < 16; ++k) {
+            va[k] = xin[k] * sign_of(seed, ((uint32_t)col_a + k) & (bs - 1));
+            vb[k] = xin[16 + k] * sign_of(seed, ((uint32_t)col_b + k) & (bs - 1));
         }
         const uint32_t bsr = bs > 1024u ? 1024u : bs;     // stages inside one 1024-column run
         fwht_lanes<16>(va, bsr, lane);
@@ -250,14 +250,8 @@ __device__ __forceinline__ void rotate_private(const void* x, int x_dtype, size_
 #pragma unroll
         for (int k = 0; k < 16; ++k) { xt[k] = va[k]; xt[16 + k] = vb[k]; }
     } else {
-        if (act_a) {
-            load_chunk(x, x_dtype, row_off + col_a, xt);
 #pragma unroll
-            for (int k = 0; k < kChunk; ++k) xt[k] *= sign_of(seed, ((uint32_t)col_a + k) & (bs - 1));
-        } else {
-#pragma unroll
-            for (int k = 0; k < kChunk; ++k) xt[k] = 0.0f;
-        }
+        for (int k = 0; k < kChunk; ++k) xt[k] = xin[k] * sign_of(seed, ((uint32_t)col_a + k) & (bs - 1));
         fwht_lane32(xt, bs, lane);
     }
 }
@@ -352,34 +346,48 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
         nrm[buf] = a.L.norms[rn < out ? rn : out - 1];
     };
 
-    // The first NS-1 groups go out before the prologue so their latency overlaps it.
+    // Prologue.  Everything that has to come from memory is requested up front, the small things
+    // first (table values, activations), then the first NS-1 weight groups: loads complete in
+    // order, so the prologue only waits for what it needs while the weights keep streaming in.
+    constexpr int kEntries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
+    constexpr int kPre = 8;
+    float tv[kPre];
 #pragma unroll
-    for (int u = 0; u < NS - 1; ++u) fetch(u, r_begin + u * R);
-
-    // Prologue.  Everything that has to come from memory is requested first (weights above, then
-    // the activation tile of the shared path and the table values), so the latencies overlap.
+    for (int k = 0; k < kPre; ++k) {
+        const int i = tid + k * (int)blockDim.x;
+        tv[k] = a.L.tables[(i < kEntries * 16 ? i : 0) >> 4];
+    }
+    constexpr bool kEarlyX = (NB == 1 && MODE != kDual);
     const bool shared_rot = (a.S >= 4 && a.L.block_size <= (uint32_t)kTile);      // W <= 2: at most 8 tiles
     TileRaw raw[NB];
+    float xt[NB][kChunk];   // rotated activations, kept in registers for the whole kernel
+    float xr[NB][kChunk];   // second rotation, dual mode only
     if (shared_rot) {
         const int col = wave * kTile + lane * 8;
 #pragma unroll
         for (int b = 0; b < NB; ++b)
             if (col < a.L.in_features) raw[b] = load_tile_raw(a.x, a.x_dtype, (size_t)b * a.L.in_features, col);
+    } else if constexpr (kEarlyX) {
+        load_owned<combined>(a.x, a.x_dtype, 0, col_a, col_b, act_a, act_b, xt[0]);
     }
+
+#pragma unroll
+    for (int u = 0; u < NS - 1; ++u) fetch(u, r_begin + u * R);
 
     // Decode tables -> LDS, one private column per lane.
     {
-        constexpr int entries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
         float4* dst = reinterpret_cast<float4*>(smem);
-        for (int i = tid; i < entries * 16; i += blockDim.x) {
+#pragma unroll
+        for (int k = 0; k < kPre; ++k) {
+            const int i = tid + k * (int)blockDim.x;
+            if (i < kEntries * 16) dst[i] = make_float4(tv[k], tv[k], tv[k], tv[k]);
+        }
+        for (int i = tid + kPre * (int)blockDim.x; i < kEntries * 16; i += blockDim.x) {
             const float v = a.L.tables[i >> 4];
             dst[i] = make_float4(v, v, v, v);
         }
     }
 
-    // Rotated activations, kept in registers for the whole kernel.
-    float xt[NB][kChunk];
-    float xr[NB][kChunk];   // second rotation, dual mode only
     if (shared_rot) {
         float* stage = reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes);
 #pragma unroll
@@ -396,11 +404,11 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     } else {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            rotate_private<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, col_a, col_b, act_a, act_b,
-                                     a.L.seed_primary, a.L.block_size, lane, xt[b]);
+            if constexpr (!kEarlyX)  // register budget: load late, one batch row at a time
+                load_owned<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, col_a, col_b, act_a, act_b, xt[b]);
             if constexpr (MODE == kDual)
-                rotate_private<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, col_a, col_b, act_a, act_b,
-                                         a.L.seed_residual, a.L.block_size, lane, xr[b]);
+                rotate_private<combined>(xt[b], col_a, col_b, a.L.seed_residual, a.L.block_size, lane, xr[b]);
+            rotate_private<combined>(xt[b], col_a, col_b, a.L.seed_primary, a.L.block_size, lane, xt[b]);
         }
     }
     __syncthreads();                                          // tables visible to every wave
@@ -499,8 +507,7 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     const int threads = a.W * a.S * kWave;
     // Two workgroups per CU fit (LDS, registers) up to 8 waves each; wider rows run one per CU so
     // the prologue is not repeated in a second round.
-    int max_grid = (a.W > 8) ? num_cus : num_cus * 2;
-    if (const char* e = getenv("TQ_GEMV_GRID")) { int v = atoi(e); if (v > 0) max_grid = v; }
+    const int max_grid = (a.W > 8) ? num_cus : num_cus * 2;
 
     int grid = (out + a.S - 1) / a.S;
     if (grid > max_grid) grid = max_grid;
@@ -510,16 +517,8 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     // Four rows per group only where the register budget allows it without spilling.
     int R = (max_rows >= 4 && MAXT <= 512 && NB < 4) ? 4 : (max_rows >= 2 ? 2 : 1);
     if (MODE == kDual && MAXT > 512) R = 1;
-    if (const char* e = getenv("TQ_GEMV_R")) { int v = atoi(e); if (v == 1 || v == 2 || v == 4) R = v; }
-    a.groups = 0;
     a.iters = (max_rows + R - 1) / R;
 
-    int ns = 2;
-    if (const char* e = getenv("TQ_GEMV_NS")) ns = atoi(e);
-    if (NB == 1 && MODE != kDual && R == 2 && ns == 3) return launch_one<MODE, NB, 2, MAXT, 3>(a, grid, threads, stream);
-    if (NB == 1 && MODE != kDual && R == 2 && ns == 4) return launch_one<MODE, NB, 2, MAXT, 4>(a, grid, threads, stream);
-    if (NB == 1 && MODE != kDual && R == 1 && ns == 4) return launch_one<MODE, NB, 1, MAXT, 4>(a, grid, threads, stream);
-    if (NB == 1 && MODE != kDual && R == 1 && ns == 8) return launch_one<MODE, NB, 1, MAXT, 8>(a, grid, threads, stream);
     switch (R) {
         case 4: return launch_one<MODE, NB, 4, MAXT, 2>(a, grid, threads, stream);
         case 2: return launch_one<MODE, NB, 2, MAXT, 2>(a, grid, threads, stream);
@@ -549,7 +548,6 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
         } else {
             if (left >= 4 && W <= 8)      { step = 4; e = launch_nb<MODE, 4, 512>(a, num_cus, stream); }
             else if (left >= 2 && W <= 8) { step = 2; e = launch_nb<MODE, 2, 512>(a, num_cus, stream); }
-            else if (W <= 8 && getenv("TQ_GEMV_512")) { step = 1; e = launch_nb<MODE, 1, 512>(a, num_cus, stream); }
             else                          { step = 1; e = launch_nb<MODE, 1, 1024>(a, num_cus, stream); }
         }
         if (e != hipSuccess) return e;
