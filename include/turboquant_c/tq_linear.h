@@ -110,6 +110,12 @@ int tq_linear_forward_host(tq_linear_t layer, const void* x_host, int x_dtype, i
 int tq_linear_dequantize(tq_linear_t layer, float* w_dev, void* stream);
 int tq_linear_dequantize_host(tq_linear_t layer, float* w_host);
 
+/* Same dequantisation with the fp32 result rounded to nearest-even into w_dtype
+ * (TQ_DTYPE_F32 / F16 / BF16): the cast src/turboquant_c_dequant.cpp:155-167 applies
+ * before it writes a weight back to a safetensors file, fused into the kernel's store. */
+int tq_linear_dequantize_as(tq_linear_t layer, void* w_dev, int w_dtype, void* stream);
+int tq_linear_dequantize_as_host(tq_linear_t layer, void* w_host, int w_dtype);
+
 /** Release the layer and its device buffers.  Safe to call with NULL. */
 void tq_linear_free(tq_linear_t layer);
 

@@ -79,6 +79,22 @@ int tq_fit_layer_codebooks_host(const float* weight_host, int out_features, int 
  */
 uint32_t tq_best_block_size(int in_features, uint32_t max_block_size);
 
+/* generate_codebook_from_data (reference src/codebook.cpp:99-143,284-302 -- the CPU form, which the
+ * converter's workers force): Lloyd-Max from the analytic initialisation, lower_bound bins,
+ * double-precision bin sums, at most `iterations` rounds, stop below a 1e-6 shift.  The
+ * assignment pass runs on the GPU.  n == 0 returns the analytic codebook.  Returns the number of
+ * centroids written, -1 on error.  boundaries_out may be NULL. */
+int tq_generate_codebook_from_data_host(const float* data_host, size_t n, int bits, int iterations,
+                                        float* centroids_out, float* boundaries_out);
+
+/* quantize / dequantize of reference src/codebook.cpp:284-321 as elementwise GPU maps over host
+ * buffers: lower_bound over the n_centroids-1 boundaries, clamp to the last bin; index -> centroid
+ * with the same clamp.  Return 0 on success. */
+int tq_codebook_quantize_host(const float* values_host, size_t n, const float* boundaries_host, int n_centroids,
+                              uint8_t* indices_host);
+int tq_codebook_dequantize_host(const uint8_t* indices_host, size_t n, const float* centroids_host, int n_centroids,
+                                float* values_host);
+
 #ifdef __cplusplus
 }
 #endif

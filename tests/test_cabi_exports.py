@@ -12,7 +12,7 @@ INCLUDE = os.path.join(entry.ROOT, "include")
 
 def _declared_functions():
     names = []
-    for path in glob.glob(os.path.join(INCLUDE, "**", "*.h"), recursive=True):
+    for path in glob.glob(os.path.join(INCLUDE, "turboquant_c", "*.h")):
         text = open(path).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         text = re.sub(r"//[^\n]*", "", text)
@@ -39,7 +39,7 @@ def test_library_exports_every_declared_symbol():
 def test_headers_compile_as_c():
     import subprocess
     import tempfile
-    headers = sorted(glob.glob(os.path.join(INCLUDE, "**", "*.h"), recursive=True))
+    headers = sorted(glob.glob(os.path.join(INCLUDE, "turboquant_c", "*.h")))
     with tempfile.TemporaryDirectory() as d:
         src = os.path.join(d, "t.c")
         with open(src, "w") as f:

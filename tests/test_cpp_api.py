@@ -1,0 +1,221 @@
+"""C++ API (include/turboquant/*.h), the 25-symbol C API (include/turboquant_c/turboquant_c.h)
+and the TQ8 safetensors layout.
+
+CPU part: the handle-based C entry points, and this library's safetensors reader/writer checked
+in both directions against the independent `safetensors` Python package.
+GPU part: a C++ program drives quantize_weight / TurboQuantLinear / dequantize_weight_gpu /
+write_tq_safetensors and its results are compared with the CPU oracle; tq_model_dequant is run
+on a model directory assembled here.
+"""
+import ctypes
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+from safetensors import safe_open
+from safetensors.numpy import load_file, save_file
+
+import __graft_entry__ as entry
+
+BIN = os.path.join(entry.ROOT, "tests", "cpp", "bin")
+
+
+def _run(name, *args):
+    exe = os.path.join(BIN, name)
+    assert os.path.exists(exe), "build the test programs first (python __graft_entry__.py)"
+    p = subprocess.run([exe, *args], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, f"{name} failed:\n{p.stdout}\n{p.stderr}"
+    return p.stdout
+
+
+def _metadata(path):
+    with safe_open(path, framework="np") as f:
+        return f.metadata() or {}
+
+
+# --------------------------------------------------------------------------- CPU
+def test_c_api_program(tmp_path):
+    """Reference tests/c_api/*.c cases, compiled as C99 against turboquant_c.h."""
+    assert "c api ok" in _run("test_c_api", str(tmp_path))
+
+
+def test_safetensors_reader_and_writer_against_python_package(tmp_path):
+    rng = np.random.default_rng(5)
+    tensors = {
+        "a.packed_primary": rng.integers(0, 256, (7, 16), dtype=np.uint8),
+        "a.norms": rng.standard_normal(7).astype(np.float32),
+        "a.seeds": np.array([0xDEADBEEF, 0, 512], dtype=np.uint32),
+        "half": rng.standard_normal((3, 5)).astype(np.float16),
+        "wide": rng.standard_normal((2, 2, 3)),
+        "i64": rng.integers(-2**40, 2**40, (4,), dtype=np.int64),
+        "flags": np.array([True, False, True]),
+        "scalar": np.array(3.5, dtype=np.float32),
+        "empty": np.zeros((0, 4), dtype=np.float32),
+        "unié\"quote\\": np.arange(6, dtype=np.int32).reshape(2, 3),
+    }
+    md = {"quantization_method": "turboquant", "note": "line\nbreak \"q\" ü", "tq_version": "1"}
+    src, dst = str(tmp_path / "in.safetensors"), str(tmp_path / "out.safetensors")
+    save_file(tensors, src, metadata=md)
+    assert f"{len(tensors)} tensors" in _run("st_roundtrip", "copy", src, dst)
+    back = load_file(dst)                      # our writer, their reader
+    assert set(back) == set(tensors)
+    for k, v in tensors.items():
+        assert back[k].dtype == v.dtype and back[k].shape == v.shape, k
+        assert np.array_equal(back[k], v), k
+    assert _metadata(dst) == md
+    out = _run("st_roundtrip", "meta", dst)
+    assert "quantization_method=turboquant" in out and "tq_version=1" in out
+    # header is 8-byte aligned as the format recommends
+    n = int.from_bytes(open(dst, "rb").read(8), "little")
+    assert n % 8 == 0
+
+
+def test_reader_rejects_malformed_files(tmp_path):
+    bad = tmp_path / "bad.safetensors"
+    bad.write_bytes((100).to_bytes(8, "little") + b"{}")
+    p = subprocess.run([os.path.join(BIN, "st_roundtrip"), "copy", str(bad), str(tmp_path / "o")],
+                       capture_output=True, text=True)
+    assert p.returncode == 1 and "error" in p.stderr
+    hdr = json.dumps({"t": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]}}).encode()
+    bad.write_bytes(len(hdr).to_bytes(8, "little") + hdr + b"\0" * 8)       # data too short
+    p = subprocess.run([os.path.join(BIN, "st_roundtrip"), "copy", str(bad), str(tmp_path / "o")],
+                       capture_output=True, text=True)
+    assert p.returncode == 1
+    assert _run("st_roundtrip", "meta", str(tmp_path / "missing.safetensors")) == ""
+
+
+# --------------------------------------------------------------------------- GPU
+@pytest.mark.gpu
+@pytest.mark.parametrize("out_f,in_f,bs,batch", [(64, 512, 256, 3), (48, 384, 128, 1)])
+def test_cpp_api_against_oracle(tmp_path, oracle, out_f, in_f, bs, batch):
+    o = oracle
+    w = o.lcg_matrix(out_f, in_f, 42) * np.float32(0.05)
+    x = o.lcg_matrix(batch, in_f, 99)
+    src = str(tmp_path / "inputs.safetensors")
+    save_file({"w": w, "x": x}, src, metadata={"block_size": str(bs)})
+    assert "cpp api ok" in _run("test_cpp_api", src, str(tmp_path))
+    res = load_file(str(tmp_path / "results.safetensors"))
+
+    cb = o.generate_codebook(4)
+    for tag, shared in (("dual.", False), ("shared.", True)):
+        qw = o.quantize_weight(w, cb, cb, 4, 4, bs, shared)
+        assert np.array_equal(res[tag + "packed_primary"], qw.packed_primary)
+        assert np.array_equal(res[tag + "packed_residual"], qw.packed_residual)
+        assert np.array_equal(res[tag + "norms"], qw.norms)
+        assert np.array_equal(res[tag + "seeds"], qw.seeds)
+        w_ref = o.dequantize_weight_cpu(qw, cb, cb, bs)
+        assert np.array_equal(res[tag + "w"], w_ref)                       # bit-exact
+        y_ref = o.matmul_xwT(x, w_ref, acc_double=True)
+        rel = np.linalg.norm(res[tag + "y"] - y_ref) / np.linalg.norm(y_ref)
+        assert rel < 1e-3, rel                                              # fp32 activations
+        xb = o.bf16_bits_to_f32(o.f32_to_bf16_bits(x))
+        yb_ref = o.matmul_xwT(xb, w_ref, acc_double=True)
+        rel = np.linalg.norm(res[tag + "y_bf16_in"] - yb_ref) / np.linalg.norm(yb_ref)
+        assert rel < 1e-3, rel                                              # exact bf16 inputs, fp32 out
+        rel = np.linalg.norm(res[tag + "y_f16"].astype(np.float32) - y_ref) / np.linalg.norm(y_ref)
+        assert rel < 5e-3, rel                                              # half-precision in and out
+
+    rot = o.wht_forward(w, 0x1234, bs)
+    assert np.array_equal(res["rotated"], rot)
+    assert np.array_equal(res["unrotated"], o.wht_inverse(rot, 0x1234, bs))
+    idx = o.quantize(x.reshape(-1), cb)
+    assert np.array_equal(res["x_indices"], idx)
+    assert np.array_equal(res["x_centroids"], o.dequantize(idx, cb))
+    samples = rot.reshape(-1) * (np.float32(1.0) / w.reshape(-1)[0])
+    fit = o.generate_codebook_from_data(samples, 4)
+    assert np.array_equal(res["fit_centroids"], fit.centroids)
+
+    # The TQ8 file through a stock reader (reference tests/unit/test_serialization.cpp:120-160).
+    tq = load_file(str(tmp_path / "model.safetensors"))
+    md = _metadata(str(tmp_path / "model.safetensors"))
+    assert md == {"quantization_method": "turboquant", "tq_version": "1", "tq_primary_bits": "4",
+                  "tq_residual_bits": "4", "tq_total_bits": "8", "tq_per_layer_codebooks": "true"}
+    for layer, tag in (("model.dual_proj", "dual."), ("model.shared_proj", "shared.")):
+        assert tq[layer + ".packed_primary"].dtype == np.uint8
+        assert tq[layer + ".packed_primary"].shape == (out_f, in_f // 2)
+        assert np.array_equal(tq[layer + ".packed_residual"], res[tag + "packed_residual"])
+        assert tq[layer + ".norms"].dtype == np.float32 and tq[layer + ".norms"].shape == (out_f,)
+        assert tq[layer + ".seeds"].dtype == np.uint32 and tq[layer + ".seeds"].shape == (3,)
+    assert np.array_equal(tq["tq_codebook_primary"], cb.centroids)
+    assert np.array_equal(tq["tq_codebook_residual"], cb.centroids)
+    assert np.array_equal(tq["model.dual_proj.codebook_primary"], cb.centroids)
+    assert "model.shared_proj.codebook_primary" not in tq
+
+
+def _bf16_bits(a):
+    return a.view(np.uint16) if a.dtype != np.uint16 else a
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("passthrough_dtype", [None, np.float16])
+def test_tq_model_dequant_directory(tmp_path, oracle, passthrough_dtype):
+    """tq_model_dequant (reference src/turboquant_c_dequant.cpp:20-191) on a directory written
+    with the stock safetensors package: TQ8 shard with per-layer codebooks, passthrough shard,
+    a non-TQ shard, config.json carrying quantization_config."""
+    o = oracle
+    pkg = entry.load_package()
+    L = pkg.lib()
+    src, dst = tmp_path / "tq8", tmp_path / "out"
+    src.mkdir()
+    cb = o.generate_codebook(4)
+    tensors, expect = {}, {}
+    for i, (out_f, in_f, bs, shared) in enumerate([(32, 256, 128, True), (16, 512, 512, False)]):
+        w = o.lcg_matrix(out_f, in_f, 7 + i) * np.float32(0.03)
+        name = f"model.layers.{i}.mlp.up_proj"
+        cbp, cbr = (o.fit_layer_codebooks(w, bs) if i == 0 else (cb, cb))
+        qw = o.quantize_weight(w, cbp, cbr, 4, 4, bs, shared)
+        tensors[name + ".packed_primary"] = qw.packed_primary
+        tensors[name + ".packed_residual"] = qw.packed_residual
+        tensors[name + ".norms"] = qw.norms
+        tensors[name + ".seeds"] = qw.seeds
+        if i == 0:
+            tensors[name + ".codebook_primary"] = cbp.centroids
+            tensors[name + ".codebook_residual"] = cbr.centroids
+        expect[name + ".weight"] = o.dequantize_weight_cpu(qw, cbp, cbr, bs)
+    tensors["tq_codebook_primary"] = cb.centroids
+    tensors["tq_codebook_residual"] = cb.centroids
+    save_file(tensors, str(src / "model.safetensors"),
+              metadata={"quantization_method": "turboquant", "tq_version": "1", "tq_primary_bits": "4",
+                        "tq_residual_bits": "4", "tq_total_bits": "8", "tq_per_layer_codebooks": "true"})
+    if passthrough_dtype is not None:
+        save_file({"model.norm.weight": np.linspace(-1, 1, 8).astype(passthrough_dtype)},
+                  str(src / "model_passthrough.safetensors"))
+    plain = {"embed": np.arange(12, dtype=np.float32).reshape(3, 4)}
+    save_file(plain, str(src / "extra.safetensors"))
+    config = {"model_type": "test", "hidden_size": 64,
+              "quantization_config": {"quantization_method": "turboquant", "nested": {"a": 1}, "tq_total_bits": 8}}
+    (src / "config.json").write_text(json.dumps(config, indent=2))
+    (src / "tokenizer.json").write_text("{}")
+
+    L.tq_model_dequant.restype = ctypes.c_int
+    L.tq_model_dequant.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
+    assert L.tq_model_dequant(str(src).encode(), str(dst).encode()) == 0
+
+    cfg = json.loads((dst / "config.json").read_text())
+    assert cfg == {"model_type": "test", "hidden_size": 64}
+    assert (dst / "tokenizer.json").read_text() == "{}"
+    assert np.array_equal(load_file(str(dst / "extra.safetensors"))["embed"], plain["embed"])
+    assert not (dst / "model_passthrough.safetensors").exists()
+
+    with safe_open(str(dst / "model.safetensors"), framework="np") as f:
+        names = set(f.keys())
+    want = set(expect) | ({"model.norm.weight"} if passthrough_dtype is not None else set())
+    assert names == want
+    if passthrough_dtype is None:
+        # bf16 output: read the raw bits (numpy has no bf16) and compare with the oracle's
+        # fp32 weight rounded to nearest-even.
+        import torch
+        from safetensors.torch import load_file as load_torch
+        got = load_torch(str(dst / "model.safetensors"))
+        for k, w_ref in expect.items():
+            assert got[k].dtype == torch.bfloat16 and tuple(got[k].shape) == w_ref.shape
+            bits = got[k].view(torch.int16).numpy().view(np.uint16)
+            assert np.array_equal(bits, o.f32_to_bf16_bits(w_ref)), k
+    else:
+        got = load_file(str(dst / "model.safetensors"))
+        for k, w_ref in expect.items():
+            assert got[k].dtype == np.float16
+            assert np.array_equal(got[k], w_ref.astype(np.float16)), k
+        assert np.array_equal(got["model.norm.weight"], np.linspace(-1, 1, 8).astype(np.float16))

@@ -26,8 +26,8 @@ __device__ __forceinline__ void unpack_nibbles(const uint4& P, uint32_t (&idx)[k
         }
 }
 
-__global__ __launch_bounds__(kDqWaves* kWave) void tq_dequant_kernel(LayerView L, float* __restrict__ Wout,
-                                                                      int chunks, int slabs) {
+__global__ __launch_bounds__(kDqWaves* kWave) void tq_dequant_kernel(LayerView L, void* __restrict__ Wout,
+                                                                      int w_dtype, int chunks, int slabs) {
     __shared__ float tab[256];
     for (int i = threadIdx.x; i < 256; i += blockDim.x) tab[i] = L.tables[i];
     __syncthreads();
@@ -113,21 +113,38 @@ __global__ __launch_bounds__(kDqWaves* kWave) void tq_dequant_kernel(LayerView L
         }
     }
 
-    if (active) {
-        float4* dst = reinterpret_cast<float4*>(Wout + (size_t)row * in + (size_t)chunk * kChunk);
+    if (!active) return;
+    const size_t elem = (size_t)row * in + (size_t)chunk * kChunk;
+    if (w_dtype == kF32) {
+        float4* dst = reinterpret_cast<float4*>(static_cast<float*>(Wout) + elem);
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             dst[i] = make_float4(v[4 * i] * nrm, v[4 * i + 1] * nrm, v[4 * i + 2] * nrm, v[4 * i + 3] * nrm);
+    } else {
+        // The fp32 weight rounded to nearest-even, the cast src/turboquant_c_dequant.cpp:166 applies.
+        uint4* dst = reinterpret_cast<uint4*>(static_cast<uint16_t*>(Wout) + elem);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t h[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float f = v[8 * i + j] * nrm;
+                h[j] = (w_dtype == kBF16) ? (uint32_t)float_to_bf16_bits(f)
+                                          : (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+            }
+            dst[i] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+        }
     }
 }
 
-hipError_t launch_dequant(const LayerView& L, float* w, hipStream_t stream) {
+hipError_t launch_dequant(const LayerView& L, void* w, int w_dtype, hipStream_t stream) {
     const int chunks = L.in_features / kChunk;
     const int slabs = (chunks + kWave - 1) / kWave;
     const long long waves = (long long)L.out_features * slabs;
     const long long grid = (waves + kDqWaves - 1) / kDqWaves;
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(tq_dequant_kernel, dim3((unsigned)grid), dim3(kDqWaves * kWave), 0, stream, L, w, chunks, slabs);
+    hipLaunchKernelGGL(tq_dequant_kernel, dim3((unsigned)grid), dim3(kDqWaves * kWave), 0, stream, L, w, w_dtype, chunks,
+                       slabs);
     return hipGetLastError();
 }
 

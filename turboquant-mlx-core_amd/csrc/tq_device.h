@@ -42,7 +42,7 @@ struct LayerView {
 // Launchers (tq_gemv.hip, tq_dequant.hip).  All return hipError_t of the launch.
 hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch,
                        void* y, int y_dtype, int num_cus, hipStream_t stream);
-hipError_t launch_dequant(const LayerView& L, float* w, hipStream_t stream);
+hipError_t launch_dequant(const LayerView& L, void* w, int w_dtype, hipStream_t stream);
 // Prefill (tq_prefill.hip): rotate the activations to bf16 in `workspace`, then dequant + MFMA GEMM.
 bool prefill_supported(const LayerView& L, int x_dtype, int batch);
 size_t prefill_workspace_bytes(const LayerView& L, int batch);
@@ -76,6 +76,11 @@ hipError_t launch_finish_norms(const float* orig, const double* partial, float* 
 hipError_t launch_lloyd_pass(const float* data, size_t n, const float* bounds_dev, int nc, int subtract,
                              const float* gcent_dev, const float* gbounds_dev, int ngc,
                              double* part_sum, unsigned long long* part_cnt, int workgroups, hipStream_t stream);
+
+hipError_t launch_codebook_quantize(const float* values, size_t n, const float* bounds_dev, int nc, uint8_t* indices,
+                                    hipStream_t stream);
+hipError_t launch_codebook_lookup(const uint8_t* indices, size_t n, const float* centroids_dev, int nc, float* values,
+                                  hipStream_t stream);
 
 // True when the fast wave-per-slab kernels can handle this shape.
 inline bool shape_supported(int in_features, uint32_t block_size) {

@@ -279,24 +279,34 @@ int tq_linear_forward_host(tq_linear_t h, const void* x_host, int x_dtype, int b
     } catch (...) { set_error("tq_linear_forward_host: exception"); return 1; }
 }
 
-int tq_linear_dequantize(tq_linear_t h, float* w_dev, void* stream) {
+int tq_linear_dequantize_as(tq_linear_t h, void* w_dev, int w_dtype, void* stream) {
     try {
         if (!h || !w_dev) { set_error("tq_linear_dequantize: NULL argument"); return 1; }
-        return hip_ok(tq::launch_dequant(h->view, w_dev, static_cast<hipStream_t>(stream)), "tq_dequant launch") ? 0 : 1;
+        if (w_dtype < tq::kF32 || w_dtype > tq::kBF16) { set_error("tq_linear_dequantize: bad dtype"); return 1; }
+        return hip_ok(tq::launch_dequant(h->view, w_dev, w_dtype, static_cast<hipStream_t>(stream)),
+                      "tq_dequant launch") ? 0 : 1;
     } catch (...) { set_error("tq_linear_dequantize: exception"); return 1; }
 }
 
-int tq_linear_dequantize_host(tq_linear_t h, float* w_host) {
+int tq_linear_dequantize(tq_linear_t h, float* w_dev, void* stream) {
+    return tq_linear_dequantize_as(h, w_dev, tq::kF32, stream);
+}
+
+int tq_linear_dequantize_as_host(tq_linear_t h, void* w_host, int w_dtype) {
     try {
         if (!h || !w_host) { set_error("tq_linear_dequantize_host: NULL argument"); return 1; }
-        const size_t bytes = (size_t)h->view.out_features * h->view.in_features * sizeof(float);
-        float* d = nullptr;
-        if (!hip_ok(hipMalloc((void**)&d, bytes), "hipMalloc(weight)")) return 1;
-        bool ok = tq_linear_dequantize(h, d, nullptr) == 0 &&
+        const size_t bytes = (size_t)h->view.out_features * h->view.in_features * (w_dtype == tq::kF32 ? 4 : 2);
+        void* d = nullptr;
+        if (!hip_ok(hipMalloc(&d, bytes), "hipMalloc(weight)")) return 1;
+        bool ok = tq_linear_dequantize_as(h, d, w_dtype, nullptr) == 0 &&
                   hip_ok(hipMemcpy(w_host, d, bytes, hipMemcpyDeviceToHost), "copy weight");
         (void)hipFree(d);
         return ok ? 0 : 1;
     } catch (...) { set_error("tq_linear_dequantize_host: exception"); return 1; }
+}
+
+int tq_linear_dequantize_host(tq_linear_t h, float* w_host) {
+    return tq_linear_dequantize_as_host(h, w_host, tq::kF32);
 }
 
 void tq_linear_free(tq_linear_t h) {

@@ -289,8 +289,56 @@ __global__ __launch_bounds__(kFitThreads) void tq_lloyd_pass_kernel(const float*
 }
 
 // ---------------------------------------------------------------------------
+// Scalar codebook maps (reference src/codebook.cpp:284-321): value -> bin index, index -> centroid.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void tq_codebook_quantize_kernel(const float* __restrict__ values, size_t n,
+                                                                   const float* __restrict__ bounds, int nc,
+                                                                   uint8_t* __restrict__ indices) {
+    __shared__ float s_b[32];
+    if (threadIdx.x < 32) s_b[threadIdx.x] = (int)threadIdx.x < nc - 1 ? bounds[threadIdx.x] : 0.0f;
+    __syncthreads();
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        uint32_t idx = bin_of(values[i], s_b, nc - 1);
+        if (idx >= (uint32_t)nc) idx = nc - 1;
+        indices[i] = (uint8_t)idx;
+    }
+}
+
+__global__ __launch_bounds__(256) void tq_codebook_lookup_kernel(const uint8_t* __restrict__ indices, size_t n,
+                                                                 const float* __restrict__ centroids, int nc,
+                                                                 float* __restrict__ values) {
+    __shared__ float s_c[32];
+    if (threadIdx.x < 32) s_c[threadIdx.x] = (int)threadIdx.x < nc ? centroids[threadIdx.x] : 0.0f;
+    __syncthreads();
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        uint32_t idx = indices[i];
+        if (idx >= (uint32_t)nc) idx = nc - 1;                  // src/codebook.cpp:316
+        values[i] = s_c[idx];
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Launchers
 // ---------------------------------------------------------------------------
+static unsigned elementwise_grid(size_t n) {
+    const size_t g = (n + 255) / 256;
+    return (unsigned)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
+}
+
+hipError_t launch_codebook_quantize(const float* values, size_t n, const float* bounds_dev, int nc, uint8_t* indices,
+                                    hipStream_t stream) {
+    hipLaunchKernelGGL(tq_codebook_quantize_kernel, dim3(elementwise_grid(n)), dim3(256), 0, stream, values, n,
+                       bounds_dev, nc, indices);
+    return hipGetLastError();
+}
+
+hipError_t launch_codebook_lookup(const uint8_t* indices, size_t n, const float* centroids_dev, int nc, float* values,
+                                  hipStream_t stream) {
+    hipLaunchKernelGGL(tq_codebook_lookup_kernel, dim3(elementwise_grid(n)), dim3(256), 0, stream, indices, n,
+                       centroids_dev, nc, values);
+    return hipGetLastError();
+}
+
 hipError_t launch_row_norms(const float* w, float* norms, int out, int in, hipStream_t stream) {
     hipLaunchKernelGGL(tq_row_norm_kernel, dim3((out + 3) / 4), dim3(256), 0, stream, w, norms, out, in);
     return hipGetLastError();

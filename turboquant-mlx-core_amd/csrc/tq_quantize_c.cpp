@@ -272,4 +272,64 @@ int tq_fit_layer_codebooks_host(const float* weight_host, int out, int in, uint3
     } catch (...) { set_error("tq_fit_layer_codebooks_host: exception"); return 1; }
 }
 
+int tq_generate_codebook_from_data_host(const float* data_host, size_t n, int bits, int iterations,
+                                        float* centroids_out, float* boundaries_out) {
+    try {
+        if (!centroids_out || (n > 0 && !data_host)) { set_error("tq_generate_codebook_from_data: NULL argument"); return -1; }
+        if (n == 0) return tq_generate_codebook(bits, centroids_out, boundaries_out);   // src/codebook.cpp:101-103
+        if (bits < 1 || bits > 5) { set_error("Unsupported bit width; must be 1-5"); return -1; }
+        DevBuf d;
+        if (!d.alloc(n * sizeof(float), "hipMalloc(samples)") ||
+            !hip_ok(hipMemcpy(d.p, data_host, n * sizeof(float), hipMemcpyHostToDevice), "copy samples") ||
+            !lloyd_max(d.as<float>(), n, bits, iterations, false, nullptr, nullptr, 0, centroids_out))
+            return -1;
+        if (boundaries_out) midpoints(centroids_out, 1 << bits, boundaries_out);
+        return 1 << bits;
+    } catch (...) { set_error("tq_generate_codebook_from_data: exception"); return -1; }
+}
+
+int tq_codebook_quantize_host(const float* values_host, size_t n, const float* boundaries_host, int n_centroids,
+                              uint8_t* indices_host) {
+    try {
+        if (n == 0) return 0;
+        if (!values_host || !boundaries_host || !indices_host || n_centroids < 2 || n_centroids > 32) {
+            set_error("tq_codebook_quantize: bad argument"); return 1;
+        }
+        DevBuf v, b, o;
+        float bounds[32] = {0};
+        std::memcpy(bounds, boundaries_host, (n_centroids - 1) * sizeof(float));
+        if (!v.alloc(n * sizeof(float), "hipMalloc(values)") || !b.alloc(sizeof(bounds), "hipMalloc(bounds)") ||
+            !o.alloc(n, "hipMalloc(indices)") ||
+            !hip_ok(hipMemcpy(v.p, values_host, n * sizeof(float), hipMemcpyHostToDevice), "copy values") ||
+            !hip_ok(hipMemcpy(b.p, bounds, sizeof(bounds), hipMemcpyHostToDevice), "copy bounds") ||
+            !hip_ok(tq::launch_codebook_quantize(v.as<float>(), n, b.as<float>(), n_centroids, o.as<uint8_t>(), nullptr),
+                    "codebook quantize") ||
+            !hip_ok(hipMemcpy(indices_host, o.p, n, hipMemcpyDeviceToHost), "copy indices"))
+            return 1;
+        return 0;
+    } catch (...) { set_error("tq_codebook_quantize: exception"); return 1; }
+}
+
+int tq_codebook_dequantize_host(const uint8_t* indices_host, size_t n, const float* centroids_host, int n_centroids,
+                                float* values_host) {
+    try {
+        if (n == 0) return 0;
+        if (!indices_host || !centroids_host || !values_host || n_centroids < 1 || n_centroids > 32) {
+            set_error("tq_codebook_dequantize: bad argument"); return 1;
+        }
+        DevBuf i, c, o;
+        float cent[32] = {0};
+        std::memcpy(cent, centroids_host, n_centroids * sizeof(float));
+        if (!i.alloc(n, "hipMalloc(indices)") || !c.alloc(sizeof(cent), "hipMalloc(centroids)") ||
+            !o.alloc(n * sizeof(float), "hipMalloc(values)") ||
+            !hip_ok(hipMemcpy(i.p, indices_host, n, hipMemcpyHostToDevice), "copy indices") ||
+            !hip_ok(hipMemcpy(c.p, cent, sizeof(cent), hipMemcpyHostToDevice), "copy centroids") ||
+            !hip_ok(tq::launch_codebook_lookup(i.as<uint8_t>(), n, c.as<float>(), n_centroids, o.as<float>(), nullptr),
+                    "codebook lookup") ||
+            !hip_ok(hipMemcpy(values_host, o.p, n * sizeof(float), hipMemcpyDeviceToHost), "copy values"))
+            return 1;
+        return 0;
+    } catch (...) { set_error("tq_codebook_dequantize: exception"); return 1; }
+}
+
 }  // extern "C"
