@@ -155,7 +155,10 @@ def test_error_conventions(tq, oracle):
 # ------------------------------------------------------------------ prefill
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("out,inf,bs,batch", [(64, 128, 128, 16), (300, 512, 256, 37), (513, 2048, 512, 64),
-                                              (256, 5120, 512, 300), (1000, 896 * 2, 128, 17)])
+                                              (256, 5120, 512, 300), (1000, 896 * 2, 128, 17),
+                                              # K = 64, 192, 256, 384: 2, 6, 8, 12 steps of the 6-step pipeline
+                                              (70, 64, 64, 16), (40, 192, 64, 20), (33, 256, 256, 300),
+                                              (257, 384, 128, 513)])
 def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, batch):
     """batch >= 16 with 16-bit activations takes the MFMA path (bf16 weight tiles, bf16 rotated
     activations, fp32 accumulation): 5e-3 relative L2 against dequantise + fp32 matmul."""

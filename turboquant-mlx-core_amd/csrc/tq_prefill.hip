@@ -7,11 +7,14 @@
 //
 //   Y[m, n] = norm[n] / sqrt(in * bs) * sum_k X~[m, k] * L[n, k],   L = centroid (sum) of the indices
 //
-// Workgroup tile 256 (M) x 256 (N) x 64 (K), 8 waves as 2 (M) x 4 (N), each wave 128 x 64 built
-// from v_mfma_f32_32x32x16_bf16.  Per K step every thread fetches 64 B of X~ and 32 index bytes
-// (32 weights), turns the indices into bf16 through the lane-private LDS table, and parks both in
-// registers while the MFMAs of the current step run; the tiles are then written to LDS in the
-// k-contiguous layout both MFMA operands want (row pitch 144 B: conflict-free 128-bit reads).
+// Workgroup tile 256 (M) x 256 (N), 8 waves as 2 (M) x 4 (N), each wave 128 x 64 built from
+// v_mfma_f32_32x32x16_bf16.  K advances in 32-column steps.  Activation tiles are copied from
+// global memory straight into LDS (three tiles in rotation, requested two steps ahead; the
+// rotate kernel stores X~ as ready-made tile images).  Index bytes travel through registers
+// (64-column stages, requested four steps ahead), are turned into bf16 through the lane-private
+// LDS table and written to one of two weight tiles.  One barrier per step; the two waves of a
+// SIMD run the decode and the multiply half of a step in opposite order, which keeps the matrix
+// pipe fed during the decodes.
 #include "tq_device.h"
 
 namespace tq {
@@ -20,14 +23,22 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 
-constexpr int kBM = 256, kBN = 256, kBK = 64;
-constexpr int kPitch = (kBK + 8) * 2;                 // bytes per LDS tile row (bf16), padded
-constexpr int kTileBytes = 256 * kPitch;              // 36864
+typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
+
+constexpr int kBM = 256, kBN = 256;
+constexpr int kBK = 32;                               // K extent of one LDS tile (one step)
+constexpr int kKLoad = 64;                            // K extent of one register stage of index bytes (two steps)
+constexpr int kBPitch = (kBK + 8) * 2;                // weight tile: bytes per row (bf16), padded -> 80
+constexpr int kBTile = 256 * kBPitch;                 // 20480
+constexpr int kATile = 256 * kBK * 2;                 // activation tile image: 256 rows x 64 B, swizzled -> 16384
 constexpr int kGemmThreads = 512;
 constexpr int kGemmLutBytes = 256 * 256;
+constexpr int kBOff = kGemmLutBytes;                  // two weight tiles
+constexpr int kAOff = kBOff + 2 * kBTile;             // three activation tiles
+constexpr int kGemmSmem = kAOff + 3 * kATile;         // 155648 of the CU's 163840 bytes
 
 struct PrefillArgs {
-    const uint16_t* xt;        // rotated activations bf16 [planes][M, K]
+    const uint16_t* xt;        // rotated activations, bf16 tile images [planes][m_tiles][K/32][16 KB]
     const uint8_t* plane0;     // combined bytes [N, K] (shared) or primary nibbles [N, K/2]
     const uint8_t* plane1;     // residual nibbles [N, K/2] (dual) or NULL
     const float* tables;       // 256 floats (see build_tables in tq_linear_c.cpp)
@@ -55,11 +66,23 @@ __device__ __forceinline__ uint32_t pack_bf16x2(uint32_t lo_val, uint32_t hi_val
     return __builtin_amdgcn_perm(hi_val, lo_val, 0x07060302u);   // {lo.b2, lo.b3, hi.b2, hi.b3}
 }
 
+// Position of the 16-byte slot that holds columns [8c, 8c+8) of row r inside a 64-byte tile row.
+// The XOR spreads the 16 rows a 128-bit LDS read touches at once over all 16 slot phases
+// (row & 3 picks the 64-byte quarter of the 256-byte bank line, (row >> 2) & 3 the slot in it).
+__device__ __forceinline__ int a_slot(int row, int c) { return c ^ ((row >> 2) & 3); }
+
+// Index bytes of one thread for a 64-column stage: two pieces, one per 32-column step.
+template <bool COMBINED> struct PrefillStage { u32x4v b[2]; };
+template <> struct PrefillStage<false> { u32x2v b[2]; };
+
+// The global->LDS copies and the index loads below are issued from inline assembly and waited
+// for by hand: the memory counter retires in order, every request in the loop is unconditional,
+// and the wait before each barrier (at most 4 younger requests outstanding) is therefore exact.
+// Letting the compiler place these waits makes every LDS read after a global->LDS copy wait for
+// that copy, which serialises the pipeline.
 template <int MODE>
 __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillArgs a) {
-    __shared__ __align__(16) char smem[kGemmLutBytes + 2 * kTileBytes];
-    char* As = smem + kGemmLutBytes;
-    char* Bs = As + kTileBytes;
+    __shared__ __align__(16) char smem[kGemmSmem];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -75,17 +98,26 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
     if (n_tile >= a.n_tiles) return;                       // whole workgroup leaves together
     const int m0 = m_tile * kBM, n0 = n_tile * kBN;
 
-    // Loader mapping: thread -> (tile row, 32-column half).
-    const int lrow = tid >> 1, lhalf = tid & 1;
-    const int a_row = (m0 + lrow < a.M) ? m0 + lrow : a.M - 1;
-    const int b_row = (n0 + lrow < a.N) ? n0 + lrow : a.N - 1;
-
     constexpr bool combined = (MODE == kSharedLut);
     constexpr int kPlanes = (MODE == kDual) ? 2 : 1;
-    const int ksteps = a.K / kBK;
+    const int T = a.K / kBK;                               // 32-column steps (even)
+    const int G = a.K / kKLoad;                            // 64-column index stages
 
-    // MFMA mapping: 2 x 4 waves, each 128 x 64.
+    // Weight loader mapping: thread -> (tile row, 16-column half of a 32-column tile).
+    const int lrow = tid >> 1, lh = tid & 1;
+    const int b_row = (n0 + lrow < a.N) ? n0 + lrow : a.N - 1;
+    const uint32_t b_voff = combined ? (uint32_t)b_row * (uint32_t)a.K + lh * 16
+                                     : (uint32_t)b_row * (uint32_t)(a.K >> 1) + lh * 8;
+    // Activation copy: wave w moves bytes [2048 w, 2048 w + 2048) of every 16 KB tile image.
+    const uint32_t dma_voff = (uint32_t)wave * 2048 + (uint32_t)lane * 16;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)smem;
+
+    // MFMA mapping: 2 x 4 waves, each 128 x 64; waves w and w+4 share a SIMD.
     const int wm = wave >> 2, wn = wave & 3;
+    const int a_frag0 = (wm * 128 + (lane & 31)) * 64 + (a_slot(lane & 31, lane >> 5) << 4);        // s = 0
+    const int a_frag1 = (wm * 128 + (lane & 31)) * 64 + (a_slot(lane & 31, 2 + (lane >> 5)) << 4);  // s = 1
+    const int b_frag = (wn * 64 + (lane & 31)) * kBPitch + (lane >> 5) * 16;
+
     f32x16 acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -94,8 +126,11 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
+    using Stage = PrefillStage<combined>;
+
     for (int plane = 0; plane < kPlanes; ++plane) {
         // Decode table of this plane -> LDS, one private column per lane, values rounded to bf16.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         {
             const int entries = combined ? 256 : 16;
@@ -106,37 +141,54 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
                 dst[i] = make_uint4(v, v, v, v);
             }
         }
-        __syncthreads();
 
-        const uint16_t* xa = a.xt + (size_t)plane * a.M * a.K + (size_t)a_row * a.K + lhalf * 32;
-        const uint8_t* wb = combined ? a.plane0 + (size_t)b_row * a.K + lhalf * 32
-                                     : (plane == 0 ? a.plane0 : a.plane1) + (size_t)b_row * (a.K >> 1) + lhalf * 16;
+        const char* a_tiles = reinterpret_cast<const char*>(a.xt) +
+                              ((size_t)plane * a.m_tiles + m_tile) * (size_t)T * kATile;
+        const uint8_t* w_plane = combined ? a.plane0 : (plane == 0 ? a.plane0 : a.plane1);
 
-        u32x4v ra[4];         // 32 bf16 of X~
-        uint32_t rb[16];      // 32 decoded bf16 weights
-        auto fetch_decode = [&](int ks) {
-            const u32x4v* pa = reinterpret_cast<const u32x4v*>(xa + (size_t)ks * kBK);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ra[i] = pa[i];
+        // Activation tile t -> LDS tile `buf`, straight from global memory.
+        auto copy_a = [&](int t, int buf) {
+            const char* src = a_tiles + (size_t)(t < T ? t : T - 1) * kATile;
+            const uint32_t dst = lds_base + kAOff + buf * kATile + wave * 2048;
+            asm volatile("s_mov_b32 m0, %0\n\t"
+                         "global_load_lds_dwordx4 %1, %2\n\t"
+                         "global_load_lds_dwordx4 %1, %2 offset:1024"
+                         :: "s"(dst), "v"(dma_voff), "s"(src));
+        };
+        // Index bytes of stage g -> registers.
+        auto load_b = [&](Stage& st, int g) {
+            const uint32_t off = b_voff + (uint32_t)(g < G ? g : G - 1) * (combined ? kKLoad : kKLoad / 2);
+            if constexpr (combined)
+                asm volatile("global_load_dwordx4 %0, %2, %3\n\t"
+                             "global_load_dwordx4 %1, %2, %3 offset:32"
+                             : "=&v"(st.b[0]), "=&v"(st.b[1]) : "v"(off), "s"(w_plane));
+            else
+                asm volatile("global_load_dwordx2 %0, %2, %3\n\t"
+                             "global_load_dwordx2 %1, %2, %3 offset:16"
+                             : "=&v"(st.b[0]), "=&v"(st.b[1]) : "v"(off), "s"(w_plane));
+        };
+
+        // Decode half u of a stage into weight tile `buf`.
+        auto fill = [&](const Stage& st, int u, int buf) {
+            uint32_t rb[8];
             if constexpr (combined) {
-                const uint4* pb = reinterpret_cast<const uint4*>(wb + (size_t)ks * kBK);
-                const uint4 b0 = pb[0], b1 = pb[1];
-                const uint32_t w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+                const uint32_t w4[4] = {st.b[u].x, st.b[u].y, st.b[u].z, st.b[u].w};
 #pragma unroll
-                for (int d = 0; d < 8; ++d) {
-                    const uint32_t v0 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w[d], laneoff, 0));
-                    const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w[d], laneoff, 1));
-                    const uint32_t v2 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w[d], laneoff, 2));
-                    const uint32_t v3 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w[d], laneoff, 3));
+                for (int d = 0; d < 4; ++d) {
+                    const uint32_t w = w4[d];
+                    const uint32_t v0 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w, laneoff, 0));
+                    const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w, laneoff, 1));
+                    const uint32_t v2 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w, laneoff, 2));
+                    const uint32_t v3 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w, laneoff, 3));
                     rb[2 * d] = pack_bf16x2(v0, v1);
                     rb[2 * d + 1] = pack_bf16x2(v2, v3);
                 }
             } else {
-                const uint4 b0 = *reinterpret_cast<const uint4*>(wb + (size_t)ks * (kBK >> 1));
-                const uint32_t w[4] = {b0.x, b0.y, b0.z, b0.w};
+                const uint32_t w2[2] = {st.b[u].x, st.b[u].y};
 #pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    const uint32_t ce = w[d] & 0x0F0F0F0Fu, co = (w[d] >> 4) & 0x0F0F0F0Fu;
+                for (int d = 0; d < 2; ++d) {
+                    const uint32_t w = w2[d];
+                    const uint32_t ce = w & 0x0F0F0F0Fu, co = (w >> 4) & 0x0F0F0F0Fu;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const uint32_t ve = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(ce, laneoff, j));
@@ -145,46 +197,135 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
                     }
                 }
             }
-        };
-        auto park = [&]() {
-            u32x4v* da = reinterpret_cast<u32x4v*>(As + lrow * kPitch + lhalf * 64);
-            u32x4v* db = reinterpret_cast<u32x4v*>(Bs + lrow * kPitch + lhalf * 64);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                da[i] = ra[i];
-                u32x4v t = {rb[4 * i], rb[4 * i + 1], rb[4 * i + 2], rb[4 * i + 3]};
-                db[i] = t;
-            }
+            u32x4v* db = reinterpret_cast<u32x4v*>(smem + kBOff + buf * kBTile + lrow * kBPitch + lh * 32);
+            const u32x4v t0 = {rb[0], rb[1], rb[2], rb[3]}, t1 = {rb[4], rb[5], rb[6], rb[7]};
+            db[0] = t0;
+            db[1] = t1;
         };
 
-        fetch_decode(0);
-        park();
-        __syncthreads();
-
-        for (int ks = 0; ks < ksteps; ++ks) {
-            if (ks + 1 < ksteps) fetch_decode(ks + 1);       // loads + lookups fly under the MFMAs
-
+        Stage S0, S1, S2;
+        // Everything requested so far except the 4 youngest requests has arrived.  The stage
+        // registers are tied to the statement so no use of them can be scheduled above it.
+        auto wait_all_but_4 = [&]() {
+            asm volatile("s_waitcnt vmcnt(4)"
+                         : "+v"(S0.b[0]), "+v"(S0.b[1]), "+v"(S1.b[0]), "+v"(S1.b[1]), "+v"(S2.b[0]), "+v"(S2.b[1])
+                         :: "memory");
+        };
+        // Step t = 6q + R: multiply activation tile R % 3 with weight tile R % 2, decode step t+1
+        // into the other weight tile, request activation tile t+2 and (odd steps) the index stage
+        // three ahead of the one whose second half was just decoded.
+        // The 8 table reads of decode half h (0/1) of stage half u, and their packing into 4
+        // registers of bf16 pairs.
+        auto lookup_half = [&](const Stage& st, int u, int h, uint32_t (&lv)[8]) {
+            if constexpr (combined) {
+                const uint32_t w2[2] = {h == 0 ? st.b[u].x : st.b[u].z, h == 0 ? st.b[u].y : st.b[u].w};
 #pragma unroll
-            for (int s = 0; s < kBK / 16; ++s) {
-                bf16x8 fa[4], fb[2];
-                const int koff = s * 32 + (lane >> 5) * 16;          // bytes
+                for (int d = 0; d < 2; ++d)
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    fa[i] = *reinterpret_cast<const bf16x8*>(As + (wm * 128 + i * 32 + (lane & 31)) * kPitch + koff);
+                    for (int j = 0; j < 4; ++j)
+                        lv[4 * d + j] = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w2[d], laneoff, j));
+            } else {
+                const uint32_t w = h == 0 ? st.b[u].x : st.b[u].y;
+                const uint32_t ce = w & 0x0F0F0F0Fu, co = (w >> 4) & 0x0F0F0F0Fu;
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    fb[j] = *reinterpret_cast<const bf16x8*>(Bs + (wn * 64 + j * 32 + (lane & 31)) * kPitch + koff);
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int j = 0; j < 2; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < 4; ++j) {
+                    lv[2 * j] = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(ce, laneoff, j));
+                    lv[2 * j + 1] = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(co, laneoff, j));
+                }
             }
-            __syncthreads();                                  // every wave is done reading the tiles
-            if (ks + 1 < ksteps) park();
+        };
+        auto pack_half = [&](const uint32_t (&lv)[8], uint32_t* rb) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) rb[q] = pack_bf16x2(lv[2 * q], lv[2 * q + 1]);
+        };
+
+        // Step t = 6q + R: multiply activation tile R % 3 with weight tile R % 2, decode step t+1
+        // into the other weight tile, request activation tile t+2 and (odd steps) the index stage
+        // three ahead of the one whose second half was just decoded.  The order below is a hand
+        // made software pipeline: every LDS read and every memory request is issued with matrix
+        // instructions of the same wave in flight behind it, and the scheduling fences keep the
+        // compiler from regrouping it.
+        auto step = [&](int t, int abuf, int bbuf, const Stage& st, int u, Stage* reload) {
+            const char* As = smem + kAOff + abuf * kATile;
+            const char* Bs = smem + kBOff + bbuf * kBTile + b_frag;
+            const bool do_fill = t + 1 < T;
+            bf16x8 fa0[4], fb0[2], fa1[4], fb1[2];
+            uint32_t lv[8], rb[8];
+            auto mm = [&](int i, const bf16x8 (&fa)[4], const bf16x8 (&fb)[2]) {
+                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[0], acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[1], acc[i][1], 0, 0, 0);
+            };
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb0[j] = *reinterpret_cast<const bf16x8*>(Bs + j * 32 * kBPitch);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fa0[i] = *reinterpret_cast<const bf16x8*>(As + a_frag0 + i * 32 * 64);
+            if (do_fill) lookup_half(st, u, 0, lv);
+            __builtin_amdgcn_sched_barrier(0);
+            mm(0, fa0, fb0);
+            copy_a(t + 2, (abuf + 2) % 3);
+            mm(1, fa0, fb0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb1[j] = *reinterpret_cast<const bf16x8*>(Bs + j * 32 * kBPitch + 32);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fa1[i] = *reinterpret_cast<const bf16x8*>(As + a_frag1 + i * 32 * 64);
+            if (do_fill) {
+                pack_half(lv, rb);
+                lookup_half(st, u, 1, lv);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mm(2, fa0, fb0);
+            if (reload) load_b(*reload, (t >> 1) + 3);
+            mm(3, fa0, fb0);
+            __builtin_amdgcn_sched_barrier(0);
+            mm(0, fa1, fb1);
+            mm(1, fa1, fb1);
+            if (do_fill) {
+                pack_half(lv, rb + 4);
+                u32x4v* db = reinterpret_cast<u32x4v*>(smem + kBOff + (bbuf ^ 1) * kBTile + lrow * kBPitch + lh * 32);
+                const u32x4v t0 = {rb[0], rb[1], rb[2], rb[3]}, t1 = {rb[4], rb[5], rb[6], rb[7]};
+                db[0] = t0;
+                db[1] = t1;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mm(2, fa1, fb1);
+            mm(3, fa1, fb1);
+            wait_all_but_4();
             __syncthreads();
+        };
+
+        copy_a(0, 0);
+        copy_a(1, 1);
+        load_b(S0, 0);
+        load_b(S1, 1);
+        load_b(S2, 2);
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(S0.b[0]), "+v"(S0.b[1]), "+v"(S1.b[0]), "+v"(S1.b[1]), "+v"(S2.b[0]), "+v"(S2.b[1])
+                     :: "memory");
+        __syncthreads();                                   // table and first activation tiles visible
+        fill(S0, 0, 0);
+        __syncthreads();
+        // Whole groups of six steps in the loop (one exit only, so the accumulators stay in place),
+        // then the two or four steps that remain.
+        int t = 0;
+        for (; t + 6 <= T; t += 6) {
+            step(t, 0, 0, S0, 1, nullptr);
+            step(t + 1, 1, 1, S1, 0, &S0);
+            step(t + 2, 2, 0, S1, 1, nullptr);
+            step(t + 3, 0, 1, S2, 0, &S1);
+            step(t + 4, 1, 0, S2, 1, nullptr);
+            step(t + 5, 2, 1, S0, 0, &S2);
+        }
+        if (t < T) {
+            step(t, 0, 0, S0, 1, nullptr);
+            step(t + 1, 1, 1, S1, 0, &S0);
+        }
+        if (t + 2 < T) {
+            step(t + 2, 2, 0, S1, 1, nullptr);
+            step(t + 3, 0, 1, S2, 0, &S1);
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // no copy into LDS may outlive the workgroup
 
     // Epilogue: * norm[n] / sqrt(in * bs), convert, store.
 #pragma unroll
@@ -204,7 +345,9 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 }
 
 // ---------------------------------------------------------------------------
-// Rotate activations [M, K] (f32 / f16 / bf16) -> bf16 [M, K]: X~ = H (s (.) X) per block.
+// Rotate activations [M, K] (f32 / f16 / bf16) -> bf16 tile images: X~ = H (s (.) X) per block,
+// stored as [M/256][K/32] images of 256 rows x 64 bytes in the exact byte order the GEMM keeps
+// them in LDS (16-byte slots permuted by a_slot), so a tile is one contiguous 16 KB copy.
 // One wave per (row, 2048-column slab), 32 consecutive columns per lane, fp32 butterfly.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void tq_rotate_bf16_kernel(const void* __restrict__ x, int x_dtype,
@@ -229,27 +372,29 @@ __global__ __launch_bounds__(256) void tq_rotate_bf16_kernel(const void* __restr
     }
     fwht_lane32(v, bs, lane);
     if (active) {
-        uint4* dst = reinterpret_cast<uint4*>(out + (size_t)row * cols + (size_t)chunk * kChunk);
+        const int m_tile = row >> 8, r = row & 255;
+        uint4* dst = reinterpret_cast<uint4*>(out + (((size_t)m_tile * chunks + chunk) * 256 + r) * kBK);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t w[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 w[j] = (uint32_t)float_to_bf16_bits(v[8 * i + 2 * j]) | ((uint32_t)float_to_bf16_bits(v[8 * i + 2 * j + 1]) << 16);
-            dst[i] = make_uint4(w[0], w[1], w[2], w[3]);
+            dst[a_slot(r, i)] = make_uint4(w[0], w[1], w[2], w[3]);
         }
     }
 }
 
 size_t prefill_workspace_bytes(const LayerView& L, int batch) {
     const size_t planes = (L.mode == kDual) ? 2 : 1;
-    return planes * (size_t)batch * L.in_features * sizeof(uint16_t);
+    const size_t m_tiles = ((size_t)batch + kBM - 1) / kBM;            // whole tile images
+    return planes * m_tiles * kBM * L.in_features * sizeof(uint16_t);
 }
 
 bool prefill_supported(const LayerView& L, int x_dtype, int batch) {
     if (x_dtype == kF32 || batch < 16) return false;          // fp32 activations keep the exact fp32 GEMV path
     if (L.mode != kSharedLut && L.mode != kDual && L.mode != kPrimaryOnly) return false;
-    return L.in_features % kBK == 0;
+    return L.in_features % kKLoad == 0;
 }
 
 hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
@@ -263,8 +408,9 @@ hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int ba
     hipLaunchKernelGGL(tq_rotate_bf16_kernel, dim3(rgrid), dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
                        L.seed_primary, L.block_size);
     if (L.mode == kDual)
-        hipLaunchKernelGGL(tq_rotate_bf16_kernel, dim3(rgrid), dim3(256), 0, stream, x, x_dtype, xt + (size_t)M * K,
-                           M, K, chunks, slabs, L.seed_residual, L.block_size);
+        hipLaunchKernelGGL(tq_rotate_bf16_kernel, dim3(rgrid), dim3(256), 0, stream, x, x_dtype,
+                           xt + (size_t)((M + kBM - 1) / kBM) * kBM * K, M, K, chunks, slabs, L.seed_residual,
+                           L.block_size);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
 
