@@ -325,21 +325,74 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
             step(t + 3, 0, 1, S2, 0, &S1);
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // no copy into LDS may outlive the workgroup
+    // No copy into LDS may outlive the loop: after this barrier LDS is free for the epilogue.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
 
-    // Epilogue: * norm[n] / sqrt(in * bs), convert, store.
+    // Epilogue: * norm[n] / sqrt(in * bs), convert, store.  Each wave transposes its 128 x 64 tile
+    // through a private LDS region so that every store instruction writes whole 128-byte rows;
+    // row counts that break the 16-byte alignment of those stores take the element-wise path.
+    float scale[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int col = n0 + wn * 64 + j * 32 + (lane & 31);
-        const bool col_ok = col < a.N;
-        const float s = col_ok ? a.out_scale * a.norms[col] : 0.0f;
+        scale[j] = col < a.N ? a.out_scale * a.norms[col] : 0.0f;
+    }
+    constexpr int kEpiPitch = 144;                                   // 128 data bytes + 16: conflict-light, 16-byte aligned
+    char* const stage = smem + wave * (128 * kEpiPitch);
+    const int row_base = m0 + wm * 128, col_base = n0 + wn * 64;
+    if (a.y_dtype != kF32 && (a.N & 7) == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * 128 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-                if (col_ok && row < a.M) store_scalar(a.y, a.y_dtype, (size_t)row * a.N + col, acc[i][j][r] * s);
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                    const float v = acc[i][j][r] * scale[j];
+                    const uint16_t h = a.y_dtype == kBF16 ? float_to_bf16_bits(v)
+                                                          : __builtin_bit_cast(uint16_t, (_Float16)v);
+                    *reinterpret_cast<uint16_t*>(stage + row * kEpiPitch + (j * 32 + (lane & 31)) * 2) = h;
+                }
+        uint16_t* y = static_cast<uint16_t*>(a.y);
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+            const int row = it * 8 + (lane >> 3), piece = lane & 7;
+            const u32x4v v = *reinterpret_cast<const u32x4v*>(stage + row * kEpiPitch + piece * 16);
+            const int grow = row_base + row, gcol = col_base + piece * 8;
+            if (grow < a.M && gcol < a.N) *reinterpret_cast<u32x4v*>(y + (size_t)grow * a.N + gcol) = v;
+        }
+    } else if (a.y_dtype == kF32 && (a.N & 3) == 0) {
+        float* y = static_cast<float*>(a.y);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                    *reinterpret_cast<float*>(stage + row * kEpiPitch + (lane & 31) * 4) = acc[i][j][r] * scale[j];
+                }
+#pragma unroll
+            for (int it = 0; it < 16; ++it) {
+                const int row = it * 8 + (lane >> 3), piece = lane & 7;
+                const u32x4v v = *reinterpret_cast<const u32x4v*>(stage + row * kEpiPitch + piece * 16);
+                const int grow = row_base + row, gcol = col_base + j * 32 + piece * 4;
+                if (grow < a.M && gcol < a.N) *reinterpret_cast<u32x4v*>(y + (size_t)grow * a.N + gcol) = v;
             }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = col_base + j * 32 + (lane & 31);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = row_base + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                    if (col < a.N && row < a.M)
+                        store_scalar(a.y, a.y_dtype, (size_t)row * a.N + col, acc[i][j][r] * scale[j]);
+                }
         }
     }
 }
