@@ -145,10 +145,10 @@ def test_error_conventions(tq, oracle):
         tq.TurboQuantLinear(256, 8, qw, cbp, cbr, 128)       # shape mismatch
     with pytest.raises(ValueError):
         tq.TurboQuantLinear(128, 8, qw, cbp, cbr, 96)        # block size does not divide
-    q5, c5, c3 = _make(oracle, 8, 128, 128, "5+3shared")
+    q5, c5, c3 = _make(oracle, 8, 128, 128, "5+3dual")
     layer = tq.TurboQuantLinear(128, 8, q5, c5, c3, 128)
     with pytest.raises(RuntimeError):
-        layer.forward(np.zeros((1, 128), np.float32))        # 5-bit: dequantise only
+        layer.forward(np.zeros((1, 128), np.float32))        # 5-bit with its own residual rotation: dequantise only
     layer.close()
 
 

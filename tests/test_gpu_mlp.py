@@ -1,0 +1,149 @@
+"""Gated MLP block (tq_mlp_*) and the 5-bit primary layers on the fused kernels, against the
+CPU oracle: dequantise each layer, fp32 matmul, SiLU gate in fp32 between the linears."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tq():
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    pkg.lib()
+    return pkg
+
+
+class _Hip:
+    """Device buffers through the HIP runtime the library already loaded (ctypes, no torch: a second
+    HIP runtime in the process would not find the GPU)."""
+
+    def __init__(self):
+        import ctypes
+        self.c = ctypes
+        self.rt = ctypes.CDLL("libamdhip64.so")
+        self.rt.hipMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
+        self.rt.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        self.rt.hipFree.argtypes = [ctypes.c_void_p]
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a)
+        p = self.c.c_void_p()
+        assert self.rt.hipMalloc(self.c.byref(p), max(a.nbytes, 4)) == 0
+        assert self.rt.hipMemcpy(p, a.ctypes.data_as(self.c.c_void_p), a.nbytes, 1) == 0
+        return p
+
+    def alloc(self, nbytes):
+        p = self.c.c_void_p()
+        assert self.rt.hipMalloc(self.c.byref(p), nbytes) == 0
+        return p
+
+    def download(self, p, shape, dtype):
+        out = np.empty(shape, dtype)
+        assert self.rt.hipDeviceSynchronize() == 0
+        assert self.rt.hipMemcpy(out.ctypes.data_as(self.c.c_void_p), p, out.nbytes, 2) == 0
+        return out
+
+    def free(self, *ptrs):
+        for p in ptrs:
+            self.rt.hipFree(p)
+
+
+def _rel(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / np.linalg.norm(b.astype(np.float64)))
+
+
+def _layer(tq, o, out_f, in_f, bs, shared, seed, scale=0.05):
+    w = (np.random.default_rng(seed).standard_normal((out_f, in_f)) * scale).astype(np.float32)
+    cbp, cbr = o.fit_layer_codebooks(w, bs)
+    qw = o.quantize_weight(w, cbp, cbr, 4, 4, bs, shared)
+    return tq.TurboQuantLinear(in_f, out_f, qw, cbp, cbr, bs), o.dequantize_weight_cpu(qw, cbp, cbr, bs)
+
+
+def _silu(g):
+    g = g.astype(np.float32)
+    return g / (np.float32(1.0) + np.exp(-g))
+
+
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("hidden,inter,bs,batch,x_dt", [(512, 1536, 256, 1, "bf16"), (512, 1536, 256, 4, "bf16"),
+                                                         (256, 640, 128, 3, "f32"), (512, 1024, 512, 40, "bf16")])
+def test_mlp_block_matches_oracle(tq, oracle, shared, hidden, inter, bs, batch, x_dt):
+    hip = _Hip()
+    o = oracle
+    gate, wg = _layer(tq, o, inter, hidden, bs, shared, 1)
+    up, wu = _layer(tq, o, inter, hidden, bs, shared, 2)
+    down, wd = _layer(tq, o, hidden, inter, bs, shared, 3)
+    mlp = tq.TurboQuantMLP(gate, up, down, max_batch=batch)
+
+    x32 = np.random.default_rng(batch).standard_normal((batch, hidden)).astype(np.float32)
+    if x_dt == "bf16":
+        xbits = o.f32_to_bf16_bits(x32)
+        x_ref = o.bf16_bits_to_f32(xbits)
+        x_dev = hip.upload(xbits)
+        code = tq.BF16
+    else:
+        x_ref = x32
+        x_dev = hip.upload(x32)
+        code = tq.F32
+    y_dev = hip.alloc(batch * hidden * 4)
+    for _ in range(2):                                   # the block reuses its intermediates
+        mlp.forward_device(x_dev, code, batch, y_dev, tq.F32)
+        y = hip.download(y_dev, (batch, hidden), np.float32)
+
+    act = _silu(o.matmul_xwT(x_ref, wg, acc_double=True)) * o.matmul_xwT(x_ref, wu, acc_double=True)
+    if batch >= 16 and x_dt == "bf16":
+        act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))   # handed to the MFMA path as bf16
+    want = o.matmul_xwT(act.astype(np.float32), wd, acc_double=True)
+    tol = 1e-3 if (x_dt == "f32" or batch < 16) else 8e-3   # three bf16 MFMA layers in a row
+    assert _rel(y, want) < tol
+    with pytest.raises(RuntimeError):
+        mlp.forward_device(x_dev, code, batch + 1, y_dev, tq.F32)
+    mlp.close()
+    hip.free(x_dev, y_dev)
+    for l in (gate, up, down):
+        l.close()
+
+
+def test_mlp_create_rejects_mismatched_layers(tq, oracle):
+    a, _ = _layer(tq, oracle, 256, 128, 128, True, 1)
+    b, _ = _layer(tq, oracle, 128, 128, 128, True, 2)
+    with pytest.raises(ValueError):
+        tq.TurboQuantMLP(a, b, a)
+    for l in (a, b):
+        l.close()
+
+
+@pytest.mark.parametrize("rbits,shared", [(3, True), (0, True)])
+@pytest.mark.parametrize("out_f,in_f,bs,batch", [(96, 512, 256, 1), (64, 2048, 512, 3), (80, 512, 128, 32)])
+def test_five_bit_primary_fused_forward(tq, oracle, rbits, shared, out_f, in_f, bs, batch):
+    """5-bit primary + 3-bit shared-rotation residual (and 5-bit alone) run on the fused kernels
+    through a one-byte-per-weight plane; the dequantised weight stays bit-exact."""
+    o = oracle
+    w = (np.random.default_rng(5).standard_normal((out_f, in_f)) * 0.03).astype(np.float32)
+    cbp, cbr = o.generate_codebook(5), o.generate_codebook(rbits if rbits else 3)
+    qw = o.quantize_weight(w, cbp, cbr, 5, rbits, bs, shared)
+    w_ref = o.dequantize_weight_cpu(qw, cbp, cbr, bs)
+    layer = tq.TurboQuantLinear(in_f, out_f, qw, cbp, cbr, bs)
+    assert layer.mode() == ("shared_5bit" if rbits else "primary_only_5bit")
+    assert np.array_equal(layer.dequantize(), w_ref)
+    x = np.random.default_rng(batch).standard_normal((batch, in_f)).astype(np.float32)
+    y = layer.forward(x)
+    assert _rel(y, o.matmul_xwT(x, w_ref, acc_double=True)) < 1e-3
+    xb = o.f32_to_bf16_bits(x)
+    yb = layer.forward(xb, tq.BF16, tq.F32)
+    assert _rel(yb, o.matmul_xwT(o.bf16_bits_to_f32(xb), w_ref, acc_double=True)) < 5e-3
+    layer.close()
+
+
+def test_five_bit_dual_rotation_still_dequantise_only(tq, oracle):
+    o = oracle
+    w = o.lcg_matrix(16, 128, 3)
+    cbp, cbr = o.generate_codebook(5), o.generate_codebook(3)
+    qw = o.quantize_weight(w, cbp, cbr, 5, 3, 64, False)
+    layer = tq.TurboQuantLinear(128, 16, qw, cbp, cbr, 64)
+    assert layer.mode() == "dual_5bit"
+    assert np.array_equal(layer.dequantize(), o.dequantize_weight_cpu(qw, cbp, cbr, 64))
+    with pytest.raises(RuntimeError):
+        layer.forward(np.zeros((1, 128), np.float32))
+    layer.close()

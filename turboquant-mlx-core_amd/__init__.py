@@ -70,6 +70,11 @@ def lib():
                                              C.c_int, _f32p, _f32p]
         L.tq_fit_layer_codebooks_host.argtypes = [_f32p, C.c_int, C.c_int, C.c_uint32, C.c_int, C.c_int, _f32p, C.c_int,
                                                   C.c_int, _f32p, _f32p]
+        L.tq_mlp_create.restype = C.c_void_p
+        L.tq_mlp_create.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        L.tq_mlp_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
+        L.tq_mlp_free.argtypes = [C.c_void_p]
+        L.tq_mlp_free.restype = None
         _lib = L
     return _lib
 
@@ -148,6 +153,33 @@ class TurboQuantLinear:
     def close(self):
         if getattr(self, "_h", None):
             lib().tq_linear_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class TurboQuantMLP:
+    """Gated MLP block y = down(silu(gate(x)) * up(x)) over three TurboQuantLinear layers
+    (tq_mlp_* in include/turboquant_c/tq_mlp.h).  Device pointers in, device pointers out;
+    the layers must stay alive as long as the block."""
+
+    def __init__(self, gate, up, down, max_batch=1):
+        self._layers = (gate, up, down)
+        self._h = lib().tq_mlp_create(gate._h, up._h, down._h, max_batch)
+        if not self._h:
+            raise ValueError(last_error())
+
+    def forward_device(self, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream=None):
+        if lib().tq_mlp_forward(self._h, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream) != 0:
+            raise RuntimeError(last_error())
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().tq_mlp_free(self._h)
             self._h = None
 
     def __del__(self):

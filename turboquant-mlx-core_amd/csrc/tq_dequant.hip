@@ -60,6 +60,20 @@ __global__ __launch_bounds__(kDqWaves* kWave) void tq_dequant_kernel(LayerView L
                 pi[4 * d + j] = c & 0x0fu;
                 ri[4 * d + j] = c >> 4;
             }
+    } else if (active && five && L.packed_combined) {
+        // 5-bit primary with a residual of at most 3 bits: one byte per weight, residual index in
+        // the top 3 bits (both already clamped to their codebooks when the plane was built)
+        const uint4* p = reinterpret_cast<const uint4*>(L.packed_combined + (size_t)row * in + (size_t)chunk * 32);
+        const uint4 a = p[0], b = p[1];
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t c = (w[d] >> (8 * j)) & 0xffu;
+                pi[4 * d + j] = c & 0x1fu;
+                ri[4 * d + j] = c >> 5;
+            }
     } else if (active) {
         if (five) {
             const uint4* p = reinterpret_cast<const uint4*>(L.packed_primary + (size_t)row * in + (size_t)chunk * 32);
@@ -236,6 +250,44 @@ hipError_t launch_combine_planes(const uint8_t* primary, const uint8_t* residual
                                  size_t plane_bytes, hipStream_t stream) {
     hipLaunchKernelGGL(tq_combine_planes_kernel, dim3(2048), dim3(256), 0, stream, primary, residual,
                        reinterpret_cast<uint16_t*>(combined), plane_bytes);
+    return hipGetLastError();
+}
+
+// 5-bit primary (one index per byte) + residual nibbles of at most 3 significant bits -> one byte
+// per weight: min(r, n_residual - 1) << 5 | min(p, n_primary - 1)  (clamps of src/dequantizer.cpp:94,103).
+__global__ void tq_combine_planes5_kernel(const uint8_t* __restrict__ primary, const uint8_t* __restrict__ residual,
+                                          uint16_t* __restrict__ combined, size_t residual_bytes, uint32_t pmax,
+                                          uint32_t rmax) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < residual_bytes; i += stride) {
+        const uint32_t rb = residual[i];
+        const uint32_t p0 = min((uint32_t)primary[2 * i], pmax), p1 = min((uint32_t)primary[2 * i + 1], pmax);
+        const uint32_t r0 = min(rb & 0x0fu, rmax), r1 = min(rb >> 4, rmax);
+        combined[i] = (uint16_t)((r0 << 5) | p0 | (((r1 << 5) | p1) << 8));
+    }
+}
+
+hipError_t launch_combine_planes5(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,
+                                  size_t residual_bytes, int n_primary, int n_residual, hipStream_t stream) {
+    hipLaunchKernelGGL(tq_combine_planes5_kernel, dim3(2048), dim3(256), 0, stream, primary, residual,
+                       reinterpret_cast<uint16_t*>(combined), residual_bytes, (uint32_t)(n_primary - 1),
+                       (uint32_t)(n_residual - 1));
+    return hipGetLastError();
+}
+
+__global__ void tq_silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up, void* __restrict__ out,
+                                   int out_dtype, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const float g = gate[i];
+        store_scalar(out, out_dtype, i, g / (1.0f + expf(-g)) * up[i]);
+    }
+}
+
+hipError_t launch_silu_mul(const float* gate, const float* up, void* out, int out_dtype, size_t n, hipStream_t stream) {
+    const size_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(tq_silu_mul_kernel, dim3((unsigned)(blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks))), dim3(256), 0,
+                       stream, gate, up, out, out_dtype, n);
     return hipGetLastError();
 }
 

@@ -40,8 +40,13 @@ struct LayerView {
 };
 
 // Launchers (tq_gemv.hip, tq_dequant.hip).  All return hipError_t of the launch.
+// gate (optional, fp32 [batch, out]): store silu(gate) * y instead of y.
 hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch,
-                       void* y, int y_dtype, int num_cus, hipStream_t stream);
+                       void* y, int y_dtype, int num_cus, hipStream_t stream, const float* gate = nullptr);
+// out[i] = silu(gate[i]) * up[i] over n fp32 values, written as out_dtype (gated MLP, batched path).
+hipError_t launch_silu_mul(const float* gate, const float* up, void* out, int out_dtype, size_t n, hipStream_t stream);
+hipError_t launch_combine_planes5(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,
+                                  size_t residual_bytes, int n_primary, int n_residual, hipStream_t stream);
 hipError_t launch_dequant(const LayerView& L, void* w, int w_dtype, hipStream_t stream);
 // Prefill (tq_prefill.hip): rotate the activations to bf16 in `workspace`, then dequant + MFMA GEMM.
 bool prefill_supported(const LayerView& L, int x_dtype, int batch);

@@ -30,9 +30,18 @@ struct GemvArgs {
     int W, S;        // slabs per row, row streams per workgroup
     int iters;       // uniform trip count: ceil(longest row range / R)
     float out_scale; // inv_scale * inv_sqrt_bs
+    const float* gate;   // optional [batch, out] fp32: the stored value becomes silu(gate) * y (gated MLP)
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// y, or silu(g) * y = g / (1 + exp(-g)) * y when a gate vector is given (fp32, as between the
+// linears of a gated MLP block).
+__device__ __forceinline__ float apply_gate(const float* gate, size_t idx, float y) {
+    if (!gate) return y;
+    const float g = gate[idx];
+    return g / (1.0f + expf(-g)) * y;
+}
 
 // 128-bit streaming load (weights are read exactly once).
 __device__ __forceinline__ uint4 load_stream16(const uint8_t* p) {
@@ -462,7 +471,8 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
         const bool owner = lane < V && r < r_end;
 
         if (a.W == 1) {
-            if (owner) store_scalar(a.y, a.y_dtype, (size_t)b * out + r, total * row_scale);
+            if (owner) store_scalar(a.y, a.y_dtype, (size_t)b * out + r,
+                                    apply_gate(a.gate, (size_t)b * out + r, total * row_scale));
         } else {
             float* buf_base = partial + (it & 1) * (16 * 16);
             if (lane < V) buf_base[wave * V + lane] = total;
@@ -470,7 +480,7 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
             if (slab == 0 && owner) {
                 float t = 0.0f;
                 for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * V + lane];
-                store_scalar(a.y, a.y_dtype, (size_t)b * out + r, t * row_scale);
+                store_scalar(a.y, a.y_dtype, (size_t)b * out + r, apply_gate(a.gate, (size_t)b * out + r, t * row_scale));
             }
         }
     };
@@ -540,6 +550,7 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
         GemvArgs a = base;
         a.x = static_cast<const char*>(base.x) + (size_t)done * in * xe;
         a.y = static_cast<char*>(base.y) + (size_t)done * out * ye;
+        a.gate = base.gate ? base.gate + (size_t)done * out : nullptr;
         const int left = batch - done;
         hipError_t e;
         int step = 1;
@@ -557,9 +568,10 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
 }
 
 hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch,
-                       void* y, int y_dtype, int num_cus, hipStream_t stream) {
+                       void* y, int y_dtype, int num_cus, hipStream_t stream, const float* gate) {
     GemvArgs a{};
     a.L = L;
+    a.gate = gate;
     a.x = x; a.y = y; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
     a.out_scale = L.inv_scale * L.inv_sqrt_bs;
     switch (L.mode) {

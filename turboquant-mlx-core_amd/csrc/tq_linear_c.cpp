@@ -4,6 +4,7 @@
 // device buffer ownership and kernel dispatch.  Nothing here computes on the CPU:
 // a missing GPU or a failed HIP call is reported as an error.
 #include "turboquant_c/tq_linear.h"
+#include "turboquant_c/tq_mlp.h"
 
 #include <cmath>
 #include <cstdio>
@@ -56,6 +57,11 @@ struct tq_linear_s {
     uint8_t* d_combined = nullptr;
     float* d_norms = nullptr;
     float* d_tables = nullptr;
+    // 5-bit primary with a residual of at most 3 bits (or none): the fused kernels run it as a
+    // shared-rotation layer over a one-byte-per-weight plane (r << 5 | p) and its 256-entry table.
+    float* d_tables_fwd = nullptr;
+    tq::LayerView fwd_view{};
+    bool has_fwd_view = false;
     int primary_cols = 0;
     int residual_cols = 0;
     // Staging for the *_host entry points, grown on demand.
@@ -70,6 +76,7 @@ struct tq_linear_s {
         if (d_combined) (void)hipFree(d_combined);
         if (d_norms) (void)hipFree(d_norms);
         if (d_tables) (void)hipFree(d_tables);
+        if (d_tables_fwd) (void)hipFree(d_tables_fwd);
         if (d_stage_x) (void)hipFree(d_stage_x);
         if (d_stage_y) (void)hipFree(d_stage_y);
         if (d_work) (void)hipFree(d_work);
@@ -182,6 +189,27 @@ tq_linear_t create_impl(int in_features, int out_features,
         (void)hipFree(h->d_residual); h->d_residual = nullptr;
     }
 
+    const bool fused5 = (mode == tq::kShared5 || mode == tq::kPrimaryOnly5) && nr <= 8;
+    if (fused5) {
+        const size_t cbytes = (size_t)out_features * in_features;
+        float lut[256];
+        std::memset(lut, 0, sizeof(lut));
+        for (int r = 0; r < 8; ++r)
+            for (int p5 = 0; p5 < 32; ++p5) {
+                const float c = cbp[p5 < np ? p5 : np - 1];
+                lut[(r << 5) | p5] = mode == tq::kShared5 ? c + cbr[r < nr ? r : nr - 1] : c;   // src/dequantizer.cpp:186-212
+            }
+        ok = hip_ok(hipMalloc((void**)&h->d_combined, cbytes), "hipMalloc(packed_combined)") &&
+             hip_ok(hipMalloc((void**)&h->d_tables_fwd, sizeof(lut)), "hipMalloc(tables)") &&
+             hip_ok(hipMemcpy(h->d_tables_fwd, lut, sizeof(lut), hipMemcpyHostToDevice), "copy tables") &&
+             hip_ok(tq::launch_combine_planes5(h->d_primary, h->d_residual, h->d_combined, rbytes, np < 32 ? np : 32, nr,
+                                               nullptr), "combine_planes5") &&
+             hip_ok(hipDeviceSynchronize(), "combine_planes5 sync");
+        if (!ok) { delete h; return nullptr; }
+        (void)hipFree(h->d_primary); h->d_primary = nullptr;
+        (void)hipFree(h->d_residual); h->d_residual = nullptr;
+    }
+
     h->primary_cols = primary_cols;
     h->residual_cols = residual_cols;
     tq::LayerView& v = h->view;
@@ -198,10 +226,37 @@ tq_linear_t create_impl(int in_features, int out_features,
     v.mode = mode;
     v.inv_scale = 1.0f / std::sqrt(static_cast<float>(in_features));      // src/dequantizer.cpp:76
     v.inv_sqrt_bs = 1.0f / std::sqrt(static_cast<float>(block_size));     // src/rotation.cpp:333
+    if (fused5) {
+        h->fwd_view = v;
+        h->fwd_view.mode = tq::kSharedLut;
+        h->fwd_view.tables = h->d_tables_fwd;
+        h->has_fwd_view = true;
+    }
     return h;
 }
 
 }  // namespace
+
+// Shared by tq_linear_forward and the MLP block (tq_mlp_c.cpp).  gate: optional fp32 [batch, out];
+// the batch-1..15 kernel then stores silu(gate) * y.  Returns 0 on success.
+int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void* y_dev, int y_dtype,
+                 hipStream_t stream, const float* gate) {
+    if (h->view.mode >= tq::kShared5 && !h->has_fwd_view) {
+        set_error("tq_linear_forward: 5-bit primary with its own residual rotation or a 4-bit residual is not "
+                  "supported by the fused kernels"); return 1;
+    }
+    const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
+    if (tq::prefill_supported(V, x_dtype, batch)) {
+        if (gate) { set_error("tq_linear_forward: gated store is a batch < 16 feature"); return 1; }
+        // Dense contraction: rotate once, dequantise tiles to bf16 in LDS, MFMA.  The first call
+        // with a larger batch allocates the rotated-activation workspace (not capturable in a graph).
+        if (!ensure_stage(&h->d_work, &h->work_bytes, tq::prefill_workspace_bytes(V, batch))) return 1;
+        return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, h->d_work, stream),
+                      "tq_prefill launch") ? 0 : 1;
+    }
+    return hip_ok(tq::launch_gemv(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream, gate),
+                  "tq_gemv launch") ? 0 : 1;
+}
 
 extern "C" {
 
@@ -246,18 +301,7 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
         if (batch <= 0 || !dtype_valid(x_dtype) || !dtype_valid(y_dtype)) {
             set_error("tq_linear_forward: bad batch or dtype"); return 1;
         }
-        if (h->view.mode >= tq::kShared5) {
-            set_error("tq_linear_forward: 5-bit primary is not supported by the fused kernels"); return 1;
-        }
-        if (tq::prefill_supported(h->view, x_dtype, batch)) {
-            // Dense contraction: rotate once, dequantise tiles to bf16 in LDS, MFMA.  The first call
-            // with a larger batch allocates the rotated-activation workspace (not capturable in a graph).
-            if (!ensure_stage(&h->d_work, &h->work_bytes, tq::prefill_workspace_bytes(h->view, batch))) return 1;
-            return hip_ok(tq::launch_prefill(h->view, x_dev, x_dtype, batch, y_dev, y_dtype, h->d_work,
-                                             static_cast<hipStream_t>(stream)), "tq_prefill launch") ? 0 : 1;
-        }
-        return hip_ok(tq::launch_gemv(h->view, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(),
-                                      static_cast<hipStream_t>(stream)), "tq_gemv launch") ? 0 : 1;
+        return forward_impl(h, x_dev, x_dtype, batch, y_dev, y_dtype, static_cast<hipStream_t>(stream), nullptr);
     } catch (...) { set_error("tq_linear_forward: exception"); return 1; }
 }
 
@@ -341,6 +385,76 @@ int tq_wht_rotate_host(const float* in_host, float* out_host, int rows, int cols
         (void)hipFree(d);
         return ok ? 0 : 1;
     } catch (...) { set_error("tq_wht_rotate_host: exception"); return 1; }
+}
+
+// ---------------------------------------------------------------------------
+// Gated MLP block: y = down( silu(gate(x)) * up(x) ), fp32 between the linears.
+// ---------------------------------------------------------------------------
+struct tq_mlp_s {
+    tq_linear_t gate, up, down;
+    int max_batch;
+    float* d_gate = nullptr;    // [max_batch, intermediate] fp32
+    float* d_up = nullptr;      // [max_batch, intermediate] fp32 (batched path only)
+    void* d_act = nullptr;      // [max_batch, intermediate] fp32 (decode) or bf16 (batched path)
+    ~tq_mlp_s() {
+        if (d_gate) (void)hipFree(d_gate);
+        if (d_up) (void)hipFree(d_up);
+        if (d_act) (void)hipFree(d_act);
+    }
+};
+
+tq_mlp_t tq_mlp_create(tq_linear_t gate, tq_linear_t up, tq_linear_t down, int max_batch) {
+    try {
+        if (!gate || !up || !down) { set_error("tq_mlp_create: NULL layer"); return nullptr; }
+        if (max_batch <= 0) { set_error("tq_mlp_create: max_batch must be positive"); return nullptr; }
+        const int hidden = gate->view.in_features, inter = gate->view.out_features;
+        if (up->view.in_features != hidden || up->view.out_features != inter || down->view.in_features != inter) {
+            set_error("tq_mlp_create: layer shapes do not form gate/up [I, H], down [O, I]"); return nullptr;
+        }
+        tq_mlp_s* m = new (std::nothrow) tq_mlp_s{gate, up, down, max_batch};
+        if (!m) { set_error("tq_mlp_create: out of host memory"); return nullptr; }
+        const size_t n = (size_t)max_batch * inter;
+        bool ok = hip_ok(hipMalloc((void**)&m->d_gate, n * sizeof(float)), "hipMalloc(gate)") &&
+                  hip_ok(hipMalloc((void**)&m->d_up, n * sizeof(float)), "hipMalloc(up)") &&
+                  hip_ok(hipMalloc(&m->d_act, n * sizeof(float)), "hipMalloc(act)");
+        // The batched path of the three layers needs rotated-activation workspaces: size them now so
+        // that tq_mlp_forward never allocates.
+        for (tq_linear_t l : {gate, up, down}) {
+            const tq::LayerView& V = l->has_fwd_view ? l->fwd_view : l->view;
+            if (ok && max_batch >= 16)
+                ok = ensure_stage(&l->d_work, &l->work_bytes, tq::prefill_workspace_bytes(V, max_batch));
+        }
+        if (!ok) { delete m; return nullptr; }
+        return m;
+    } catch (...) { set_error("tq_mlp_create: exception"); return nullptr; }
+}
+
+int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* y_dev, int y_dtype, void* stream) {
+    try {
+        if (!m || !x_dev || !y_dev) { set_error("tq_mlp_forward: NULL argument"); return 1; }
+        if (batch <= 0 || batch > m->max_batch || !dtype_valid(x_dtype) || !dtype_valid(y_dtype)) {
+            set_error("tq_mlp_forward: bad batch (larger than max_batch?) or dtype"); return 1;
+        }
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        const size_t n = (size_t)batch * m->gate->view.out_features;
+        const tq::LayerView& VG = m->gate->has_fwd_view ? m->gate->fwd_view : m->gate->view;
+        if (!tq::prefill_supported(VG, x_dtype, batch)) {
+            // decode: three launches, the SiLU gate folded into the store of the up projection
+            if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
+            if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_act, tq::kF32, st, m->d_gate) != 0) return 1;
+            return forward_impl(m->down, m->d_act, tq::kF32, batch, y_dev, y_dtype, st, nullptr);
+        }
+        // batched: MFMA path for all three, activation handed to the down projection as bf16
+        if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
+        if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_up, tq::kF32, st, nullptr) != 0) return 1;
+        if (!hip_ok(tq::launch_silu_mul(m->d_gate, m->d_up, m->d_act, tq::kBF16, n, st), "silu_mul launch")) return 1;
+        return forward_impl(m->down, m->d_act, tq::kBF16, batch, y_dev, y_dtype, st, nullptr);
+    } catch (...) { set_error("tq_mlp_forward: exception"); return 1; }
+}
+
+void tq_mlp_free(tq_mlp_t m) {
+    if (!m) return;
+    delete m;
 }
 
 }  // extern "C"
