@@ -107,6 +107,29 @@ def time_graph(tq, torch, handles, x, y, xcode, batch, steps, warmup):
     return start.elapsed_time(end) * 1e-3
 
 
+def time_graph_fn(torch, enqueue_step, steps, warmup):
+    """Capture `steps` calls of enqueue_step(stream_handle) in one HIP graph; return seconds per step."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(max(warmup, 1)):
+            enqueue_step(stream.cuda_stream)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for _ in range(steps):
+            enqueue_step(stream.cuda_stream)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        graph.replay()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        start.record(stream)
+        graph.replay()
+        end.record(stream)
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) * 1e-3 / steps
+
+
 def cpu_baseline(torch, tensors, out, inf, bs, x_f32):
     """Reference CPU path (dequantize_weight_cpu + fp32 matmul, restated in oracle/) on the
     host cores of this box, whole layer, single thread as the reference's serial loops."""
@@ -263,6 +286,62 @@ def main():
                                                   "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
                                                   "includes": "activation rotation kernel + dequant/MFMA GEMM kernel"}
     tq.lib().tq_linear_free(hp)
+    torch.cuda.empty_cache()
+
+    # ---- decode MLP block, Qwen2.5-7B shape: gate/up 18944 x 3584, down 3584 x 18944, batch 1 ----
+    L = tq.lib()
+    hid, inter = 3584, 18944
+    for shared in (False, True):
+        blocks, keep = [], []
+        for c in range(2):                       # two blocks of 204 MB cycled: HBM-resident weights
+            hs = [make_layer(tq, torch, o_, i_, bs, seed=700 + 10 * c + k, sigma=0.015, shared=shared,
+                             per_layer_codebooks=True)[0]
+                  for k, (o_, i_) in enumerate([(inter, hid), (inter, hid), (hid, inter)])]
+            m = L.tq_mlp_create(hs[0], hs[1], hs[2], 1)
+            if not m:
+                raise RuntimeError(tq.last_error())
+            blocks.append(m); keep.append(hs)
+        xm = torch.randn(1, hid, device="cuda", generator=g).to(torch.bfloat16)
+        ym = torch.empty(1, hid, device="cuda", dtype=torch.float32)
+        turn = [0]
+
+        def mlp_step(s):
+            if L.tq_mlp_forward(blocks[turn[0] % 2], xm.data_ptr(), tq.BF16, 1, ym.data_ptr(), tq.F32, s) != 0:
+                raise RuntimeError(tq.last_error())
+            turn[0] += 1
+        steps_m = max(2, args.steps // 2 * 2)
+        us_m = time_graph_fn(torch, mlp_step, steps_m, 2) * 1e6
+        Bm = 2 * algorithmic_bytes(inter, hid, 1, 2, 4) + algorithmic_bytes(hid, inter, 1, 4, 4)
+        extra["mlp_block_7b_bs1_" + ("shared_rotation" if shared else "dual_rotation")] = {
+            "us_per_block": us_m, "algorithmic_bytes": Bm, "hbm_frac": Bm / (us_m * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "kernels_per_block": 3}
+        for m in blocks:
+            L.tq_mlp_free(m)
+        for hs in keep:
+            for h in hs:
+                L.tq_linear_free(h)
+        torch.cuda.empty_cache()
+
+    # ---- decoder-layer projections, Qwen2.5-32B shape, batch 1 / 4 / 8, bf16 activations ----
+    shapes = [("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120, 5120),
+              ("gate", 27648, 5120), ("up", 27648, 5120), ("down", 5120, 27648)]
+    layers = [(n_, o_, i_, make_layer(tq, torch, o_, i_, bs, seed=900 + k, sigma=0.01, shared=True,
+                                      per_layer_codebooks=True)[0]) for k, (n_, o_, i_) in enumerate(shapes)]
+    for batch in (1, 4, 8):
+        xs = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
+        ys = {o_: torch.empty(batch, o_, device="cuda", dtype=torch.float32) for o_ in (5120, 1024, 27648)}
+
+        def layer_step(s):
+            for n_, o_, i_, h in layers:
+                if L.tq_linear_forward(h, xs[i_].data_ptr(), tq.BF16, batch, ys[o_].data_ptr(), tq.F32, s) != 0:
+                    raise RuntimeError(tq.last_error())
+        us_l = time_graph_fn(torch, layer_step, max(args.steps // 10, 10), 2) * 1e6
+        Bl = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
+        extra[f"decoder_layer_projections_32b_bs{batch}"] = {
+            "us_per_layer_all_7_projections": us_l, "algorithmic_bytes": Bl,
+            "hbm_frac": Bl / (us_l * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    for _, _, _, h in layers:
+        L.tq_linear_free(h)
     finish(args, torch, extra, result)
 
 
