@@ -23,8 +23,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152403.7 KiB + 632.3 KiB.
-MEASURED_TRAFFIC_BYTES = 312770253
+# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152437.9 KiB + 647.2 KiB.
+MEASURED_TRAFFIC_BYTES = 312855552
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
 
@@ -233,8 +233,22 @@ def main():
     del tensors
     torch.cuda.empty_cache()
 
-    # ---- secondary configuration of the metric: 4096 x 4096 fp32, batch 1 ------------
+    # ---- what this machine sustains: streaming read and bf16 MFMA loop (roofline denominators) ----
     extra = {}
+    import ctypes as C
+    Lp = tq.lib()
+    Lp.tq_probe_hbm_read.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
+    Lp.tq_probe_mfma_bf16.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+    val = C.c_double()
+    probes = {}
+    if Lp.tq_probe_hbm_read(1 << 30, 10, C.byref(val)) == 0:
+        probes["hbm_stream_read_gbs"] = val.value
+    for name, rnd in (("mfma_bf16_tflops_ones", 0), ("mfma_bf16_tflops_random_operands", 1)):
+        if Lp.tq_probe_mfma_bf16(rnd, 20000, C.byref(val)) == 0:
+            probes[name] = val.value
+    extra["machine_probes"] = probes
+    if "hbm_stream_read_gbs" in probes:
+        result["roofline"]["frac_of_measured_stream_read"] = achieved / probes["hbm_stream_read_gbs"]
     if args.skip_extra:
         finish(args, torch, extra, result)
         return
@@ -284,6 +298,9 @@ def main():
         flops = 2.0 * M * outp * inp
         extra[f"prefill_27648x5120_M{M}_bf16"] = {"us_per_layer": usp, "tflops": flops / usp / 1e6,
                                                   "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
+                                                  "frac_of_measured_mfma_loop_random_operands":
+                                                      flops / usp / 1e6 / probes.get("mfma_bf16_tflops_random_operands",
+                                                                                     float("nan")),
                                                   "includes": "activation rotation kernel + dequant/MFMA GEMM kernel"}
     tq.lib().tq_linear_free(hp)
     torch.cuda.empty_cache()
