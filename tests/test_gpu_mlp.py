@@ -15,13 +15,16 @@ def tq():
 
 
 class _Hip:
-    """Device buffers through the HIP runtime the library already loaded (ctypes, no torch: a second
-    HIP runtime in the process would not find the GPU)."""
+    """Device buffers through the HIP runtime the library itself is linked against (ctypes, no torch:
+    another copy of the runtime in the process, such as the one torch bundles, does not see the
+    device this library initialised)."""
 
     def __init__(self):
         import ctypes
+        import os
         self.c = ctypes
-        self.rt = ctypes.CDLL("libamdhip64.so")
+        path = "/opt/rocm/lib/libamdhip64.so"
+        self.rt = ctypes.CDLL(path if os.path.exists(path) else "libamdhip64.so")
         self.rt.hipMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
         self.rt.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
         self.rt.hipFree.argtypes = [ctypes.c_void_p]
