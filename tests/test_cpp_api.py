@@ -113,7 +113,8 @@ def test_cpp_api_against_oracle(tmp_path, oracle, out_f, in_f, bs, batch):
         xb = o.bf16_bits_to_f32(o.f32_to_bf16_bits(x))
         yb_ref = o.matmul_xwT(xb, w_ref, acc_double=True)
         rel = np.linalg.norm(res[tag + "y_bf16_in"] - yb_ref) / np.linalg.norm(yb_ref)
-        assert rel < 1e-3, rel                                              # exact bf16 inputs, fp32 out
+        assert rel < (1e-3 if batch == 1 else 5e-3), rel                    # bf16 activations: batch 1 exact fp32 kernel,
+                                                                            # more rows the bf16-weight MFMA kernel
         rel = np.linalg.norm(res[tag + "y_f16"].astype(np.float32) - y_ref) / np.linalg.norm(y_ref)
         assert rel < 5e-3, rel                                              # half-precision in and out
 

@@ -180,3 +180,33 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
     y1 = layer.forward(xbits[3:4], tq.BF16, tq.F32)
     layer.close()
     assert _rel(y[3:4], y1) < 5e-3
+
+
+# ------------------------------------------------------------------ small batches on the matrix cores
+@pytest.mark.parametrize("out,inf,bs,batch", [(64, 512, 512, 2), (300, 1024, 256, 5), (513, 2048, 512, 15),
+                                              (1000, 5120, 512, 8), (16, 512, 64, 3), (47, 1536, 128, 9)])
+def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, out, inf, bs, batch):
+    """2..15 rows of 16-bit activations on a shared-rotation layer whose width is a multiple of 512
+    take the small-batch MFMA kernel (bf16 weights and rotated activations, fp32 accumulation over
+    512-column chunks): 5e-3 relative L2, ragged row counts, every row equal to its batch-1 result."""
+    qw, cbp, cbr = _make(oracle, out, inf, bs, "shared")
+    x32 = np.random.default_rng(100 + batch).standard_normal((batch, inf)).astype(np.float32)
+    xbits = oracle.f32_to_bf16_bits(x32)
+    want = oracle.linear_forward(qw, cbp, cbr, bs, oracle.bf16_bits_to_f32(xbits))
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    y = layer.forward(xbits, tq.BF16, tq.F32)
+    assert y.shape == (batch, out)
+    assert _rel(y, want) < 5e-3
+    for b in range(batch):                                   # no row leaks into another
+        assert _rel(y[b:b + 1], want[b:b + 1]) < 8e-3
+    yb = oracle.bf16_bits_to_f32(layer.forward(xbits, tq.BF16, tq.BF16))
+    assert _rel(yb, want) < 7e-3
+    x16 = x32.astype(np.float16)
+    y16 = layer.forward(x16, tq.F16, tq.F32)
+    assert _rel(y16, oracle.linear_forward(qw, cbp, cbr, bs, x16.astype(np.float32))) < 5e-3
+    y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)      # exact fp32 batch-1 kernel
+    assert _rel(y[batch - 1:batch], y1) < 5e-3
+    # fp32 activations keep the exact path at any batch
+    yf = layer.forward(x32)
+    assert _rel(yf, oracle.linear_forward(qw, cbp, cbr, bs, x32)) < 1e-3
+    layer.close()

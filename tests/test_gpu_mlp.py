@@ -95,10 +95,10 @@ def test_mlp_block_matches_oracle(tq, oracle, shared, hidden, inter, bs, batch, 
         y = hip.download(y_dev, (batch, hidden), np.float32)
 
     act = _silu(o.matmul_xwT(x_ref, wg, acc_double=True)) * o.matmul_xwT(x_ref, wu, acc_double=True)
-    if batch >= 16 and x_dt == "bf16":
-        act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))   # handed to the MFMA path as bf16
+    if batch >= 2 and x_dt == "bf16":
+        act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))   # handed to the matrix-core paths as bf16
     want = o.matmul_xwT(act.astype(np.float32), wd, acc_double=True)
-    tol = 1e-3 if (x_dt == "f32" or batch < 16) else 8e-3   # three bf16 MFMA layers in a row
+    tol = 1e-3 if (x_dt == "f32" or batch == 1) else 8e-3   # three bf16-weight layers in a row
     assert _rel(y, want) < tol
     with pytest.raises(RuntimeError):
         mlp.forward_device(x_dev, code, batch + 1, y_dev, tq.F32)

@@ -53,6 +53,14 @@ bool prefill_supported(const LayerView& L, int x_dtype, int batch);
 size_t prefill_workspace_bytes(const LayerView& L, int batch);
 hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                           void* workspace, hipStream_t stream);
+hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
+                               hipStream_t stream);
+// Small batches (tq_skinny.hip): 2..15 rows of 16-bit activations on shared-rotation layers, batch rows as
+// the M side of 16x16x32 MFMAs.  xt_workspace as for launch_prefill; partial: skinny_partial_bytes().
+bool skinny_supported(const LayerView& L, int x_dtype, int batch);
+size_t skinny_partial_bytes(const LayerView& L);
+hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
+                         void* xt_workspace, float* partial, int num_cus, hipStream_t stream);
 hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t seed,
                       uint32_t block_size, float inv_sqrt_bs, int inverse, hipStream_t stream);
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream);

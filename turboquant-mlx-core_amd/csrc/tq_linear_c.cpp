@@ -69,6 +69,8 @@ struct tq_linear_s {
     void* d_stage_y = nullptr; size_t stage_y_bytes = 0;
     // Rotated-activation workspace of the prefill path, grown on demand.
     void* d_work = nullptr; size_t work_bytes = 0;
+    // Per-chunk partial products of the small-batch path.
+    void* d_partial = nullptr; size_t partial_bytes = 0;
 
     ~tq_linear_s() {
         if (d_primary) (void)hipFree(d_primary);
@@ -80,6 +82,7 @@ struct tq_linear_s {
         if (d_stage_x) (void)hipFree(d_stage_x);
         if (d_stage_y) (void)hipFree(d_stage_y);
         if (d_work) (void)hipFree(d_work);
+        if (d_partial) (void)hipFree(d_partial);
     }
 };
 
@@ -254,6 +257,15 @@ int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void
         return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, h->d_work, stream),
                       "tq_prefill launch") ? 0 : 1;
     }
+    if (!gate && tq::skinny_supported(V, x_dtype, batch)) {
+        // 2..15 rows of 16-bit activations: batch rows on the matrix cores, bf16 weights.  Workspaces are
+        // allocated on the first such call (not capturable in a graph), then reused.
+        if (!ensure_stage(&h->d_work, &h->work_bytes, tq::prefill_workspace_bytes(V, batch)) ||
+            !ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V))) return 1;
+        return hip_ok(tq::launch_skinny(V, x_dev, x_dtype, batch, y_dev, y_dtype, h->d_work,
+                                        static_cast<float*>(h->d_partial), device_cu_count(), stream),
+                      "tq_skinny launch") ? 0 : 1;
+    }
     return hip_ok(tq::launch_gemv(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream, gate),
                   "tq_gemv launch") ? 0 : 1;
 }
@@ -421,8 +433,9 @@ tq_mlp_t tq_mlp_create(tq_linear_t gate, tq_linear_t up, tq_linear_t down, int m
         // that tq_mlp_forward never allocates.
         for (tq_linear_t l : {gate, up, down}) {
             const tq::LayerView& V = l->has_fwd_view ? l->fwd_view : l->view;
-            if (ok && max_batch >= 16)
-                ok = ensure_stage(&l->d_work, &l->work_bytes, tq::prefill_workspace_bytes(V, max_batch));
+            if (ok && max_batch >= 2)
+                ok = ensure_stage(&l->d_work, &l->work_bytes, tq::prefill_workspace_bytes(V, max_batch)) &&
+                     ensure_stage(&l->d_partial, &l->partial_bytes, tq::skinny_partial_bytes(V));
         }
         if (!ok) { delete m; return nullptr; }
         return m;
@@ -437,14 +450,14 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
         }
         hipStream_t st = static_cast<hipStream_t>(stream);
         const size_t n = (size_t)batch * m->gate->view.out_features;
-        const tq::LayerView& VG = m->gate->has_fwd_view ? m->gate->fwd_view : m->gate->view;
-        if (!tq::prefill_supported(VG, x_dtype, batch)) {
+        if (batch == 1 || x_dtype == tq::kF32) {
             // decode: three launches, the SiLU gate folded into the store of the up projection
             if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
             if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_act, tq::kF32, st, m->d_gate) != 0) return 1;
             return forward_impl(m->down, m->d_act, tq::kF32, batch, y_dev, y_dtype, st, nullptr);
         }
-        // batched: MFMA path for all three, activation handed to the down projection as bf16
+        // two or more rows of 16-bit activations: matrix-core paths for all three layers (small-batch or
+        // prefill kernel), one elementwise kernel, activation handed to the down projection as bf16
         if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
         if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_up, tq::kF32, st, nullptr) != 0) return 1;
         if (!hip_ok(tq::launch_silu_mul(m->d_gate, m->d_up, m->d_act, tq::kBF16, n, st), "silu_mul launch")) return 1;

@@ -450,9 +450,10 @@ bool prefill_supported(const LayerView& L, int x_dtype, int batch) {
     return L.in_features % kKLoad == 0;
 }
 
-hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
-                          void* workspace, hipStream_t stream) {
-    const int K = L.in_features, N = L.out_features, M = batch;
+// Rotated activations of `batch` rows as bf16 tile images in `workspace` (both rotations for dual mode).
+hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
+                               hipStream_t stream) {
+    const int K = L.in_features, M = batch;
     uint16_t* xt = static_cast<uint16_t*>(workspace);
     const int chunks = K / kChunk;
     const int slabs = (chunks + kWave - 1) / kWave;
@@ -464,7 +465,14 @@ hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int ba
         hipLaunchKernelGGL(tq_rotate_bf16_kernel, dim3(rgrid), dim3(256), 0, stream, x, x_dtype,
                            xt + (size_t)((M + kBM - 1) / kBM) * kBM * K, M, K, chunks, slabs, L.seed_residual,
                            L.block_size);
-    hipError_t e = hipGetLastError();
+    return hipGetLastError();
+}
+
+hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
+                          void* workspace, hipStream_t stream) {
+    const int K = L.in_features, N = L.out_features, M = batch;
+    uint16_t* xt = static_cast<uint16_t*>(workspace);
+    hipError_t e = launch_rotate_tiles(L, x, x_dtype, batch, workspace, stream);
     if (e != hipSuccess) return e;
 
     PrefillArgs a{};

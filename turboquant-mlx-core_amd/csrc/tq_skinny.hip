@@ -1,0 +1,188 @@
+// TQ8 small-batch forward for gfx950: 2..15 activation rows with 16-bit activations, shared-rotation
+// layers (one byte per weight).
+//
+// The batch-1 kernel multiplies every decoded weight with the activation of each batch row on the
+// vector ALU, so its time grows with the batch.  Here the batch rows are the M side of
+// v_mfma_f32_16x16x32_bf16: a decoded weight costs one table read and half a byte permute however
+// many rows there are, and the kernel stays bound by the same table-read rate as batch 1.
+//
+//   Y[m, n] = norm[n] / sqrt(in * bs) * sum_k X~[m, k] * L[n, k]
+//
+// K is cut into 512-column chunks.  A wave keeps the rotated activations of its chunk for all 16
+// (padded) batch rows in registers as MFMA A operands (64 VGPRs), walks 16-row groups of the weight
+// plane, decodes 16 x 512 weights per group through the lane-private LDS table (entries rounded to
+// bf16, as in the prefill kernel) and writes the 16 x 16 fp32 partial product of the chunk.  A
+// second small kernel adds the chunks, applies the row norm and converts.
+// The rotated activations come from tq_rotate_bf16_kernel (tile images, see tq_prefill.hip).
+#include "tq_device.h"
+
+namespace tq {
+
+typedef __bf16 sk_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float sk_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t sk_u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kSkChunk = 512;            // columns per K chunk
+constexpr int kSkThreads = 512;          // 8 waves per workgroup, one workgroup per CU
+constexpr int kSkLutBytes = 256 * 256;
+
+struct SkinnyArgs {
+    const uint16_t* xt;        // rotated activations, bf16 tile images [K/32][256 rows x 64 B] (rows >= batch unset)
+    const uint8_t* plane;      // combined bytes [N, K]
+    const float* tables;       // 256-entry sum table
+    float* partial;            // [chunks][16][N] fp32
+    int batch, N, K;
+    int chunks;                // K / 512
+    int groups;                // ceil(N / 16)
+    int wgs_per_chunk;
+};
+
+__device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t laneoff, int j) {
+    switch (j) {
+        case 0: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0400u);
+        case 1: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0500u);
+        case 2: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0600u);
+        default: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0700u);
+    }
+}
+
+__global__ __launch_bounds__(kSkThreads) void tq_skinny_kernel(SkinnyArgs a) {
+    __shared__ __align__(16) char smem[kSkLutBytes];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t laneoff = (uint32_t)lane << 2;
+
+    // Decode table -> LDS, one private column per lane, values rounded to bf16 (upper half of the dword).
+    {
+        uint4* dst = reinterpret_cast<uint4*>(smem);
+        for (int i = tid; i < 256 * 16; i += kSkThreads) {
+            const uint32_t v = (uint32_t)float_to_bf16_bits(a.tables[i >> 4]) << 16;
+            dst[i] = make_uint4(v, v, v, v);
+        }
+    }
+
+    const int chunk = blockIdx.x % a.chunks;
+    const int wg_in_chunk = blockIdx.x / a.chunks;
+    const int m = lane & 15, g = lane >> 4;               // A operand: batch row, k group; B operand: weight row, k group
+
+    // A operands of the chunk: k-step s covers columns 64 (s/2) + 16 g + 8 (s%2) + [0, 8) of the chunk,
+    // the same columns the B operand of that step decodes (any column order is fine as long as both
+    // operands agree).  Tile images: [K/32][256][32] bf16 with 16-byte slots XOR-permuted per row.
+    sk_bf16x8 afrag[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        const int off = 16 * g + 8 * (s & 1);              // column inside the 64-column piece
+        const int kt = chunk * 16 + 2 * (s >> 1) + (off >> 5);
+        const int slot = ((off & 31) >> 3) ^ ((m >> 2) & 3);
+        afrag[s] = *reinterpret_cast<const sk_bf16x8*>(reinterpret_cast<const char*>(a.xt) +
+                                                       ((size_t)kt * 256 + m) * 64 + slot * 16);
+    }
+    __syncthreads();                                       // table visible
+
+    // Row groups of this wave: the groups are dealt out evenly over all waves that share the chunk.
+    const int workers = a.wgs_per_chunk * (kSkThreads / 64);
+    const int me = wg_in_chunk * (kSkThreads / 64) + wave;
+    const int g_begin = (int)((long long)me * a.groups / workers);
+    const int g_end = (int)((long long)(me + 1) * a.groups / workers);
+
+    const size_t col0 = (size_t)chunk * kSkChunk + 16 * g;
+    auto row_ptr = [&](int grp) {
+        int row = grp * 16 + m;
+        if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
+        return a.plane + (size_t)row * a.K + col0;
+    };
+    sk_u32x4 raw[2][8];
+    auto fetch = [&](int buf, int grp) {
+        const uint8_t* p = row_ptr(grp);
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            raw[buf][q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+    };
+    auto lookup2 = [&](uint32_t w) {                       // 4 weights -> 2 registers of bf16 pairs
+        const uint32_t v0 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 0));
+        const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 1));
+        const uint32_t v2 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 2));
+        const uint32_t v3 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 3));
+        // entries are fp32 patterns with the value in the upper half: {v0.hi, v1.hi}, {v2.hi, v3.hi}
+        return make_uint2(__builtin_amdgcn_perm(v1, v0, 0x07060302u), __builtin_amdgcn_perm(v3, v2, 0x07060302u));
+    };
+    auto consume = [&](int buf, int grp) {
+        sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const sk_u32x4 w = raw[buf][q];
+            const uint2 p0 = lookup2(w.x), p1 = lookup2(w.y), p2 = lookup2(w.z), p3 = lookup2(w.w);
+            const sk_u32x4 b0 = {p0.x, p0.y, p1.x, p1.y}, b1 = {p2.x, p2.y, p3.x, p3.y};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * q], __builtin_bit_cast(sk_bf16x8, b0), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * q + 1], __builtin_bit_cast(sk_bf16x8, b1), acc, 0, 0, 0);
+        }
+        // D layout: lane holds weight row n = lane % 16 and batch rows 4 (lane / 16) + r.
+        const int n = grp * 16 + m;
+        if (n < a.N) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int b = 4 * g + r;
+                if (b < a.batch) a.partial[((size_t)chunk * 16 + b) * a.N + n] = acc[r];
+            }
+        }
+    };
+
+    if (g_begin < g_end) fetch(0, g_begin);
+    for (int grp = g_begin; grp < g_end; grp += 2) {
+        if (grp + 1 < g_end) fetch(1, grp + 1);
+        consume(0, grp);
+        if (grp + 1 < g_end) {
+            if (grp + 2 < g_end) fetch(0, grp + 2);
+            consume(1, grp + 1);
+        }
+    }
+}
+
+// y[b, n] = norm[n] * out_scale * sum over chunks of partial[c][b][n]
+__global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __restrict__ partial,
+                                                               const float* __restrict__ norms, void* __restrict__ y,
+                                                               int y_dtype, int batch, int N, int chunks, float out_scale) {
+    const size_t total = (size_t)batch * N;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int b = (int)(i / N), n = (int)(i % N);
+        float s = 0.0f;
+        for (int c = 0; c < chunks; ++c) s += partial[((size_t)c * 16 + b) * N + n];
+        store_scalar(y, y_dtype, i, s * (out_scale * norms[n]));
+    }
+}
+
+bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
+    return L.mode == kSharedLut && L.packed_combined && x_dtype != kF32 && batch >= 2 && batch < 16 &&
+           L.in_features % kSkChunk == 0;
+}
+
+size_t skinny_partial_bytes(const LayerView& L) {
+    return (size_t)(L.in_features / kSkChunk) * 16 * L.out_features * sizeof(float);
+}
+
+// xt_workspace: as for launch_prefill (prefill_workspace_bytes); partial: skinny_partial_bytes.
+hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
+                         void* xt_workspace, float* partial, int num_cus, hipStream_t stream) {
+    hipError_t e = launch_rotate_tiles(L, x, x_dtype, batch, xt_workspace, stream);
+    if (e != hipSuccess) return e;
+    SkinnyArgs a{};
+    a.xt = static_cast<const uint16_t*>(xt_workspace);
+    a.plane = L.packed_combined;
+    a.tables = L.tables;
+    a.partial = partial;
+    a.batch = batch; a.N = L.out_features; a.K = L.in_features;
+    a.chunks = L.in_features / kSkChunk;
+    a.groups = (L.out_features + 15) / 16;
+    a.wgs_per_chunk = num_cus / a.chunks > 0 ? num_cus / a.chunks : 1;
+    hipLaunchKernelGGL(tq_skinny_kernel, dim3(a.wgs_per_chunk * a.chunks), dim3(kSkThreads), 0, stream, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const size_t total = (size_t)batch * L.out_features;
+    const size_t blocks = (total + 255) / 256;
+    hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3((unsigned)(blocks > 2048 ? 2048 : blocks)), dim3(256), 0, stream,
+                       partial, L.norms, y, y_dtype, batch, L.out_features, a.chunks, L.inv_scale * L.inv_sqrt_bs);
+    return hipGetLastError();
+}
+
+}  // namespace tq
