@@ -46,7 +46,7 @@ __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t l
     }
 }
 
-__global__ __launch_bounds__(kSkThreads) void tq_skinny_kernel(SkinnyArgs a) {
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tq_skinny_kernel(SkinnyArgs a) {
     __shared__ __align__(16) char smem[kSkLutBytes];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -92,13 +92,9 @@ __global__ __launch_bounds__(kSkThreads) void tq_skinny_kernel(SkinnyArgs a) {
         if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
         return a.plane + (size_t)row * a.K + col0;
     };
-    sk_u32x4 raw[2][8];
-    auto fetch = [&](int buf, int grp) {
-        const uint8_t* p = row_ptr(grp);
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            raw[buf][q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(p + 64 * q));
-    };
+    // The 8 loads of a group live in 32 registers; as soon as one has been decoded it is replaced
+    // by the same piece of the next group, so a full group of loads is always in flight.
+    sk_u32x4 raw[8];
     auto lookup2 = [&](uint32_t w) {                       // 4 weights -> 2 registers of bf16 pairs
         const uint32_t v0 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 0));
         const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 1));
@@ -107,11 +103,21 @@ __global__ __launch_bounds__(kSkThreads) void tq_skinny_kernel(SkinnyArgs a) {
         // entries are fp32 patterns with the value in the upper half: {v0.hi, v1.hi}, {v2.hi, v3.hi}
         return make_uint2(__builtin_amdgcn_perm(v1, v0, 0x07060302u), __builtin_amdgcn_perm(v3, v2, 0x07060302u));
     };
-    auto consume = [&](int buf, int grp) {
+
+    if (g_begin < g_end) {
+        const uint8_t* p = row_ptr(g_begin);
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+    }
+    for (int grp = g_begin; grp < g_end; ++grp) {
+        const bool more = grp + 1 < g_end;
+        const uint8_t* pn = row_ptr(more ? grp + 1 : grp);
         sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            const sk_u32x4 w = raw[buf][q];
+            const sk_u32x4 w = raw[q];
+            if (more) raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
             const uint2 p0 = lookup2(w.x), p1 = lookup2(w.y), p2 = lookup2(w.z), p3 = lookup2(w.w);
             const sk_u32x4 b0 = {p0.x, p0.y, p1.x, p1.y}, b1 = {p2.x, p2.y, p3.x, p3.y};
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * q], __builtin_bit_cast(sk_bf16x8, b0), acc, 0, 0, 0);
@@ -126,16 +132,6 @@ __global__ __launch_bounds__(kSkThreads) void tq_skinny_kernel(SkinnyArgs a) {
                 if (b < a.batch) a.partial[((size_t)chunk * 16 + b) * a.N + n] = acc[r];
             }
         }
-    };
-
-    if (g_begin < g_end) fetch(0, g_begin);
-    for (int grp = g_begin; grp < g_end; grp += 2) {
-        if (grp + 1 < g_end) fetch(1, grp + 1);
-        consume(0, grp);
-        if (grp + 1 < g_end) {
-            if (grp + 2 < g_end) fetch(0, grp + 2);
-            consume(1, grp + 1);
-        }
     }
 }
 
@@ -146,9 +142,19 @@ __global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __re
     const size_t total = (size_t)batch * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const int b = (int)(i / N), n = (int)(i % N);
-        float s = 0.0f;
-        for (int c = 0; c < chunks; ++c) s += partial[((size_t)c * 16 + b) * N + n];
-        store_scalar(y, y_dtype, i, s * (out_scale * norms[n]));
+        // four independent running sums: the loads of a thread do not wait for one another
+        float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+        const float* p = partial + (size_t)b * N + n;
+        const size_t step = (size_t)16 * N;
+        int c = 0;
+        for (; c + 4 <= chunks; c += 4) {
+            s0 += p[(size_t)c * step];
+            s1 += p[(size_t)(c + 1) * step];
+            s2 += p[(size_t)(c + 2) * step];
+            s3 += p[(size_t)(c + 3) * step];
+        }
+        for (; c < chunks; ++c) s0 += p[(size_t)c * step];
+        store_scalar(y, y_dtype, i, ((s0 + s1) + (s2 + s3)) * (out_scale * norms[n]));
     }
 }
 
@@ -174,7 +180,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     a.batch = batch; a.N = L.out_features; a.K = L.in_features;
     a.chunks = L.in_features / kSkChunk;
     a.groups = (L.out_features + 15) / 16;
-    a.wgs_per_chunk = num_cus / a.chunks > 0 ? num_cus / a.chunks : 1;
+    a.wgs_per_chunk = 2 * num_cus / a.chunks > 0 ? 2 * num_cus / a.chunks : 1;   // two workgroups per CU
     hipLaunchKernelGGL(tq_skinny_kernel, dim3(a.wgs_per_chunk * a.chunks), dim3(kSkThreads), 0, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
