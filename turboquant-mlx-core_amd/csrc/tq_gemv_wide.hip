@@ -1,0 +1,319 @@
+// Fused TQ8 dequant + GEMV for gfx950, one batch row, rows of 3 to 8 slabs (4097..16384 columns).
+//
+// Same mathematics and same per-lane work as tq_gemv.hip (a lane owns 32 columns of a 2048-column
+// slab, lane-private centroid table in LDS, rotated activations in registers).  What differs is the
+// shape of the workgroup.  For these widths the narrow kernel has room for only one or two row
+// streams per workgroup, so every stream rotated the activation row for itself, which cost as much
+// as decoding a dozen rows.  Here ONE workgroup of up to 16 waves runs per CU:
+//   * the decode table is built once per CU;
+//   * the activation row is rotated once per CU: the waves split its 512-column tiles among
+//     themselves and hand the result over through an image of the whole row in LDS (up to 64 KB);
+//   * 16 / W row streams share the CU, each with W waves (one per slab) and a cross-wave sum per
+//     row group.
+// Every trip of the main loop issues the same loads whatever is left of a stream's row range
+// (past it they re-read its last row), and everything loaded is marked as consumed on every path,
+// so the compiler knows exactly how many loads are in flight and waits for no more than the row
+// it is about to decode; the prefetched group stays in flight.
+#include "tq_device.h"
+#include "tq_gemv_common.h"
+
+namespace tq {
+
+namespace {
+
+constexpr int kMaxImageCols = 16384;             // widest rotated-activation image in LDS (64 KB)
+
+// Marks a loaded value as consumed here.  A load whose result is only read on some paths stays
+// "possibly in flight" for the compiler on the others, and it then waits for it (and, as loads
+// complete in order, for every load issued before it, i.e. the prefetched weights) wherever that
+// register is reused, on every trip of the main loop.
+__device__ __forceinline__ void consumed(float v) { asm volatile("" :: "v"(v)); }
+__device__ __forceinline__ void consumed(const uint4& v) { asm volatile("" :: "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w)); }
+
+// 128-bit streaming load (weights are read exactly once): descriptor + per-lane byte offset +
+// wave-uniform byte offset, non-temporal.  No 64-bit address per lane.
+__device__ __forceinline__ uint4 load_stream16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, int row_off) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, row_off, 2);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+
+// One 512-column tile of the activation row as loaded: always two 16-byte loads, whatever the type
+// (a 16-bit tile is 16 bytes: its second load reads the same bytes again), so the number of loads
+// in flight does not depend on a branch.
+__device__ __forceinline__ TileRaw load_tile_fixed(const void* x, int x_dtype, int col) {
+    TileRaw r;
+    const int esz = (x_dtype == kF32) ? 4 : 2;
+    const char* p = static_cast<const char*>(x) + (size_t)col * esz;
+    r.a = *reinterpret_cast<const uint4*>(p);
+    r.b = *reinterpret_cast<const uint4*>(p + (esz == 4 ? 16 : 0));
+    return r;
+}
+
+// Wave w rotates tiles w, w + nwaves, ... (8 values per lane and tile) and writes them into the
+// image: value k of lane l of a slab sits at float index k*64 + l of the slab's 8 KB.  The image
+// holds img_cols columns; wider rows go through it in rounds.  Afterwards every wave picks up the
+// 32 values of the columns it owns.  raw[t] holds the activations of tile wave + t * nwaves (any
+// valid address for tiles past the row).
+template <bool SPLIT, int TILES>
+__device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_dtype, int in_features,
+                                             int img_cols, uint32_t seed, uint32_t bs, float* image, int wave,
+                                             int nwaves, int lane, int slab, bool act_a, bool act_b,
+                                             float (&xt)[kChunk]) {
+    const int rounds = (in_features + img_cols - 1) / img_cols;
+    for (int p = 0; p < rounds; ++p) {
+        if (p > 0) __syncthreads();                              // previous image has been read
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int tile0 = (wave + t * nwaves) * kTile;
+            if (tile0 < in_features && tile0 / img_cols == p) {   // wave-uniform
+                float v[8];
+                rotate_tile(raw[t], x_dtype, tile0 + lane * 8, tile0 + lane * 8 < in_features, seed, bs, lane, v);
+                const int col = tile0 % img_cols + lane * 8;      // column inside the image
+                float* dst = image + (col & ~(kSlab - 1)) + stage_index<SPLIT>(col & (kSlab - 1));
+#pragma unroll
+                for (int j = 0; j < 8; ++j) dst[j * kWave] = v[j];      // 8 columns stay inside one 16-run
+            }
+        }
+        __syncthreads();
+        if ((slab * kSlab) / img_cols == p) {
+            const float* src = image + (slab * kSlab) % img_cols + lane;
+#pragma unroll
+            for (int k = 0; k < kChunk; ++k)
+                xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
+        }
+    }
+}
+
+// MODE: kSharedLut (combined byte plane) or kPrimaryOnly.  R rows per group, TILES activation tiles
+// per wave (the host checks that TILES * waves covers the row and that blocks are at most 512 wide).
+template <int MODE, int R, int TILES>
+__global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
+    constexpr int NS = 2;                           // register ring: one group decoded, one in flight
+    constexpr int V = R;                            // sums produced per row group
+    extern __shared__ __align__(16) char smem[];    // tables | cross-wave partial sums | activation image
+    float* partial = reinterpret_cast<float*>(smem + kRegionBytes);   // [2][waves][V]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int slab = wave % a.W;
+    const int stream = wave / a.W;
+    constexpr bool combined = (MODE == kSharedLut);
+    const int col_a = slab * kSlab + (combined ? 16 * lane : 32 * lane);
+    const int col_b = combined ? col_a + 1024 : col_a + 16;
+    const bool act_a = col_a < a.L.in_features, act_b = col_b < a.L.in_features;
+    const uint32_t laneoff = (uint32_t)lane << 2;
+    const int out = a.L.out_features;
+    const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
+    constexpr bool use_res = (MODE != kPrimaryOnly);
+
+    // Contiguous row range of this stream.
+    const long long gs = (long long)blockIdx.x * a.S + stream;
+    const long long ts = (long long)gridDim.x * a.S;
+    const int r_begin = (int)(gs * out / ts);
+    const int r_end = (int)((gs + 1) * out / ts);
+    const int r_base = r_begin < out ? r_begin : out - 1;
+    const int r_last = r_end > r_begin ? r_end - 1 : r_base;
+
+    // The weight plane is read through a buffer descriptor based at the first row of the stream
+    // (offsets inside a stream's rows stay far below 2 GB; the host checks).  Idle runs re-read a
+    // valid address; their rotated activations are 0.
+    const uint8_t* pp = combined ? a.L.packed_combined : a.L.packed_primary;
+    const uint32_t off_p = combined ? (uint32_t)(act_a ? col_a : 0) : (uint32_t)(act_a ? (col_a >> 1) : 0);
+    const uint32_t off_q = (uint32_t)(act_b ? col_b : 0);          // combined plane only
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(pp) + (size_t)r_base * row_bytes, 0, 0x7fffffff, 0x00020000);
+    const int row_stride = (int)row_bytes;
+
+    uint4 P[NS][R], Q[NS][R];                 // register ring of row groups
+    float nrm[NS];                            // norm of the row this lane will store (lanes < V)
+    float gte[NS];                            // gate value of that output (the norm again when there is no gate)
+    const float* gsrc = a.gate ? a.gate : a.L.norms;
+    auto fetch = [&](int buf, int r0) {
+        // The norm (and gate value) travel ahead of their rows: loads complete in order, so they
+        // have arrived once the first weights of the group have.
+        const int rn = r0 + lane % V;
+        const int rc = rn < out ? rn : out - 1;
+        nrm[buf] = a.L.norms[rc];
+        gte[buf] = gsrc[rc];
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const int r = r0 + i < r_last ? r0 + i : r_last;
+            const int soff = (r - r_base) * row_stride;
+            P[buf][i] = load_stream16(rs, off_p, soff);
+            if constexpr (use_res) Q[buf][i] = load_stream16(rs, off_q, soff);
+        }
+    };
+
+    // Prologue.  Everything that has to come from memory is requested up front, the small things
+    // first (table values, activation tiles), then the first weight group.
+    constexpr int kEntries = (MODE == kSharedLut) ? 256 : 16;
+    constexpr int kPre = 8;                    // 4096 table slots from 512 threads up
+    float tv[kPre];
+#pragma unroll
+    for (int k = 0; k < kPre; ++k) {
+        const int i = tid + k * (int)blockDim.x;
+        tv[k] = a.L.tables[(i < kEntries * 16 ? i : 0) >> 4];
+    }
+    TileRaw raw[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {         // tiles past the row re-read its start and are not used
+        const int col = (wave + t * nwaves) * kTile + lane * 8;
+        raw[t] = load_tile_fixed(a.x, a.x_dtype, col < a.L.in_features ? col : 0);
+    }
+    fetch(0, r_begin);
+
+    // Decode tables -> LDS, one private column per lane.
+    {
+        float4* dst = reinterpret_cast<float4*>(smem);
+#pragma unroll
+        for (int k = 0; k < kPre; ++k) {
+            const int i = tid + k * (int)blockDim.x;
+            consumed(tv[k]);
+            if (i < kEntries * 16) dst[i] = make_float4(tv[k], tv[k], tv[k], tv[k]);
+        }
+        for (int i = tid + kPre * (int)blockDim.x; i < kEntries * 16; i += blockDim.x) {
+            const float v = a.L.tables[i >> 4];
+            dst[i] = make_float4(v, v, v, v);
+        }
+    }
+
+    float xt[kChunk];   // rotated activations, kept in registers for the whole kernel
+    rotate_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.img_cols, a.L.seed_primary, a.L.block_size,
+                                  reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes), wave, nwaves, lane,
+                                  slab, act_a, act_b, xt);
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
+    __syncthreads();                                          // tables visible to every wave
+
+    auto decode_row = [&](const uint4& p, const uint4& q, float& sum) {
+        float val[kChunk];
+        lookup32<MODE == kSharedLut, 0>(p, q, smem, laneoff, val);
+        float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kChunk; k += 2) {
+            s0 = __builtin_fmaf(val[k], xt[k], s0);
+            s1 = __builtin_fmaf(val[k + 1], xt[k + 1], s1);
+        }
+        sum = s0 + s1;
+    };
+
+    auto consume = [&](int buf, int r0, int it) {
+        float acc[V];
+        if (r0 + R <= r_end) {                               // wave-uniform: a full group, straight-line
+#pragma unroll
+            for (int i = 0; i < R; ++i) decode_row(P[buf][i], Q[buf][i], acc[i]);
+        } else {                                             // ragged end of the range: skip the rows past it
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                acc[i] = 0.0f;
+                if (r0 + i < r_end) decode_row(P[buf][i], Q[buf][i], acc[i]);
+            }
+        }
+        consumed(nrm[buf]); consumed(gte[buf]);
+        const float row_scale = a.out_scale * nrm[buf];
+        // Lane l < V now gets the wave total of row l of the group.
+        const float total = reduce_rec<V, 1>(acc, lane);
+        const int r = r0 + lane;
+        const bool owner = lane < V && r < r_end;
+
+        float* buf_base = partial + (it & 1) * (16 * 16);
+        if (lane < V) buf_base[wave * V + lane] = total;
+        __syncthreads();
+        if (slab == 0 && owner) {
+            float t = 0.0f;
+            for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * V + lane];
+            t *= row_scale;
+            if (a.gate) { const float g = gte[buf]; t = g / (1.0f + expf(-g)) * t; }   // silu(gate) * y
+            store_scalar(a.y, a.y_dtype, (size_t)r, t);
+        }
+    };
+
+    // Main loop over the register ring, unrolled twice so the stages are static: group it+1 is
+    // requested while group it is decoded.  The trip count is uniform over the grid.  Whole rounds
+    // of two stages run without a condition inside; an odd last group is a tail.
+    int it0 = 0;
+    for (; it0 + NS <= a.iters; it0 += NS) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            fetch((u + 1) % NS, r_begin + (it0 + u + 1) * R);
+            consume(u, r_begin + (it0 + u) * R, it0 + u);
+        }
+    }
+    if (it0 < a.iters) {
+        fetch(1, r_begin + (it0 + 1) * R);
+        consume(0, r_begin + it0 * R, it0);
+    }
+}
+
+template <int MODE, int R, int TILES>
+hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
+    const size_t lds = (size_t)kRegionBytes + kPartialBytes + (size_t)a.img_cols * sizeof(float);
+    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES>;
+    // More LDS than the default limit has to be asked for, once per kernel and device.
+    static bool asked[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || !asked[dev]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kRegionBytes + kPartialBytes + kMaxImageCols * (int)sizeof(float));
+        if (e != hipSuccess) return e;
+        if (dev >= 0 && dev < 64) asked[dev] = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a);
+    return hipGetLastError();
+}
+
+template <int MODE>
+hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
+    const int out = a.L.out_features;
+    a.S = 16 / a.W;                                          // row streams sharing the CU
+    const int threads = a.W * a.S * kWave;
+    const int padded = a.W * kSlab;
+    a.img_cols = padded < kMaxImageCols ? padded : kMaxImageCols;
+
+    int grid = (out + a.S - 1) / a.S;
+    if (grid > num_cus) grid = num_cus;
+    if (grid < 1) grid = 1;
+    const long long ts = (long long)grid * a.S;
+    const int max_rows = (int)((out + ts - 1) / ts);        // longest row range of any stream
+    const int R = max_rows >= 2 ? 2 : 1;
+    a.iters = (max_rows + R - 1) / R;
+
+    const int ntiles = (a.L.in_features + kTile - 1) / kTile;
+    const bool two = ntiles > threads / kWave;              // at most two tiles per wave: checked by the caller
+    if (R == 2) return two ? launch_wide_one<MODE, 2, 2>(a, grid, threads, stream)
+                           : launch_wide_one<MODE, 2, 1>(a, grid, threads, stream);
+    return two ? launch_wide_one<MODE, 1, 2>(a, grid, threads, stream)
+               : launch_wide_one<MODE, 1, 1>(a, grid, threads, stream);
+}
+
+}  // namespace
+
+// One batch row, 3 to 8 slabs, blocks of at most 512 columns, shared-rotation or primary-only layers
+// whose per-stream share of the plane stays below 2 GB.
+bool gemv_wide_supported(const LayerView& L, int num_cus) {
+    if (L.mode != kSharedLut && L.mode != kPrimaryOnly) return false;
+    if (L.block_size > (uint32_t)kTile) return false;
+    const int W = (L.in_features / kChunk + kWave - 1) / kWave;
+    if (W < 3 || W > 8) return false;
+    const int S = 16 / W;
+    const int ntiles = (L.in_features + kTile - 1) / kTile;
+    if (ntiles > 2 * W * S) return false;
+    const size_t row_bytes = L.mode == kSharedLut ? (size_t)L.in_features : (size_t)L.in_features / 2;
+    const long long streams = (long long)(num_cus > 0 ? num_cus : 1) * S;
+    const long long max_rows = (L.out_features + streams - 1) / streams + 2;
+    return (unsigned long long)max_rows * row_bytes < (1ull << 31);
+}
+
+hipError_t launch_gemv_wide(const GemvArgs& base, int num_cus, hipStream_t stream) {
+    GemvArgs a = base;
+    a.chunks = a.L.in_features / kChunk;
+    a.W = (a.chunks + kWave - 1) / kWave;
+    if (a.L.mode == kSharedLut) return launch_wide_mode<kSharedLut>(a, num_cus, stream);
+    return launch_wide_mode<kPrimaryOnly>(a, num_cus, stream);
+}
+
+}  // namespace tq
