@@ -106,6 +106,33 @@ def test_forward_fp32(tq, oracle, mode, out, inf, bs, batch):
     assert np.abs(y - want).max() < 0.15                     # the reference's own bound, test_linear.cpp:135
 
 
+@pytest.mark.parametrize("mode", ["shared", "primary_only"])
+@pytest.mark.parametrize("out,inf,bs", [(1000, 3072, 512), (777, 5120, 512), (5000, 5120, 128), (600, 6144, 512),
+                                        (515, 7168, 256), (300, 8192, 512), (64, 9216, 512), (260, 15360, 512),
+                                        (130, 16384, 512), (3, 5120, 512), (2049, 12288, 64)])
+def test_forward_batch1_wide_rows(tq, oracle, mode, out, inf, bs):
+    """One activation row on rows of 3 to 8 slabs (and, shared rotation, of an odd number of
+    1024-column halves, which are served two rows at a time): the one-workgroup-per-CU kernel.
+    Row counts are chosen so that streams get ragged, empty and single-row ranges; fp32 and bf16
+    activations; every output against the oracle within the fp32 tolerance."""
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    x = np.random.default_rng(out + inf).standard_normal((1, inf)).astype(np.float32)
+    want = oracle.linear_forward(qw, cbp, cbr, bs, x)
+    y = layer.forward(x)
+    assert y.shape == (1, out) and _rel(y, want) < 1e-3
+    assert np.array_equal(layer.forward(2.0 * x), 2.0 * y)                 # exact linearity in a factor 2
+    xbits = oracle.f32_to_bf16_bits(x)
+    xb = oracle.bf16_bits_to_f32(xbits)
+    yb = layer.forward(xbits, tq.BF16, tq.F32)
+    assert _rel(yb, oracle.linear_forward(qw, cbp, cbr, bs, xb)) < 1e-3
+    # three rows of fp32 activations: the first two go through the two-row kernel, the third alone
+    x3 = np.concatenate([x, -x, 0.5 * x], axis=0)
+    y3 = layer.forward(x3)
+    assert _rel(y3[2:3], 0.5 * y) < 1e-6 and _rel(y3[0:1], y) < 1e-6
+    layer.close()
+
+
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("xd", ["bf16", "f16"])
 @pytest.mark.parametrize("yd", ["f32", "bf16", "f16"])

@@ -10,6 +10,9 @@
 //     themselves and hand the result over through an image of the whole row in LDS (up to 64 KB);
 //   * 16 / W row streams share the CU, each with W waves (one per slab) and a cross-wave sum per
 //     row group.
+// Rows whose width is an odd number of 1024-column halves (5120 = 5 x 1024) would leave half of the
+// last slab's wave idle.  For those (PAIR) a wave owns one 1024-column half instead, 16 columns per
+// lane, and its two 16-byte loads fetch the same columns of two consecutive rows.
 // Every trip of the main loop issues the same loads whatever is left of a stream's row range
 // (past it they re-read its last row), and everything loaded is marked as consumed on every path,
 // so the compiler knows exactly how many loads are in flight and waits for no more than the row
@@ -54,11 +57,12 @@ __device__ __forceinline__ TileRaw load_tile_fixed(const void* x, int x_dtype, i
 // holds img_cols columns; wider rows go through it in rounds.  Afterwards every wave picks up the
 // 32 values of the columns it owns.  raw[t] holds the activations of tile wave + t * nwaves (any
 // valid address for tiles past the row).
-template <bool SPLIT, int TILES>
+// unit: the slab of the wave, or with PAIR its 1024-column half (xt then holds 16 values).
+template <bool SPLIT, int TILES, bool PAIR, int NX>
 __device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_dtype, int in_features,
                                              int img_cols, uint32_t seed, uint32_t bs, float* image, int wave,
-                                             int nwaves, int lane, int slab, bool act_a, bool act_b,
-                                             float (&xt)[kChunk]) {
+                                             int nwaves, int lane, int unit, bool act_a, bool act_b,
+                                             float (&xt)[NX]) {
     const int rounds = (in_features + img_cols - 1) / img_cols;
     for (int p = 0; p < rounds; ++p) {
         if (p > 0) __syncthreads();                              // previous image has been read
@@ -75,21 +79,33 @@ __device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_
             }
         }
         __syncthreads();
-        if ((slab * kSlab) / img_cols == p) {
-            const float* src = image + (slab * kSlab) % img_cols + lane;
+        if constexpr (PAIR) {
+            const int first = unit * (kSlab / 2);                 // first column of the half
+            if (first / img_cols == p) {
+                const float* src = image + ((first % img_cols) & ~(kSlab - 1)) + ((unit & 1) << 4) * kWave + lane;
 #pragma unroll
-            for (int k = 0; k < kChunk; ++k)
-                xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
+                for (int k = 0; k < NX; ++k) xt[k] = src[k * kWave];
+            }
+        } else {
+            if ((unit * kSlab) / img_cols == p) {
+                const float* src = image + (unit * kSlab) % img_cols + lane;
+#pragma unroll
+                for (int k = 0; k < NX; ++k)
+                    xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
+            }
         }
     }
 }
 
 // MODE: kSharedLut (combined byte plane) or kPrimaryOnly.  R rows per group, TILES activation tiles
 // per wave (the host checks that TILES * waves covers the row and that blocks are at most 512 wide).
-template <int MODE, int R, int TILES>
+// PAIR (combined plane only): a.W counts 1024-column halves; a group is R row pairs.
+template <int MODE, int R, int TILES, bool PAIR>
 __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
+    static_assert(!PAIR || MODE == kSharedLut, "row pairs need the one-byte-per-weight plane");
     constexpr int NS = 2;                           // register ring: one group decoded, one in flight
-    constexpr int V = R;                            // sums produced per row group
+    constexpr int V = PAIR ? 2 * R : R;             // rows, and sums, per row group
+    constexpr int NX = PAIR ? 16 : kChunk;          // rotated activations per lane
     extern __shared__ __align__(16) char smem[];    // tables | cross-wave partial sums | activation image
     float* partial = reinterpret_cast<float*>(smem + kRegionBytes);   // [2][waves][V]
 
@@ -100,8 +116,8 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     const int slab = wave % a.W;
     const int stream = wave / a.W;
     constexpr bool combined = (MODE == kSharedLut);
-    const int col_a = slab * kSlab + (combined ? 16 * lane : 32 * lane);
-    const int col_b = combined ? col_a + 1024 : col_a + 16;
+    const int col_a = PAIR ? slab * (kSlab / 2) + 16 * lane : slab * kSlab + (combined ? 16 * lane : 32 * lane);
+    const int col_b = PAIR ? col_a : (combined ? col_a + 1024 : col_a + 16);
     const bool act_a = col_a < a.L.in_features, act_b = col_b < a.L.in_features;
     const uint32_t laneoff = (uint32_t)lane << 2;
     const int out = a.L.out_features;
@@ -121,7 +137,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     // valid address; their rotated activations are 0.
     const uint8_t* pp = combined ? a.L.packed_combined : a.L.packed_primary;
     const uint32_t off_p = combined ? (uint32_t)(act_a ? col_a : 0) : (uint32_t)(act_a ? (col_a >> 1) : 0);
-    const uint32_t off_q = (uint32_t)(act_b ? col_b : 0);          // combined plane only
+    const uint32_t off_q = (uint32_t)(act_b ? col_b : 0);          // combined plane only (PAIR: same columns, next row)
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(pp) + (size_t)r_base * row_bytes, 0, 0x7fffffff, 0x00020000);
     const int row_stride = (int)row_bytes;
@@ -139,10 +155,16 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
         gte[buf] = gsrc[rc];
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            const int r = r0 + i < r_last ? r0 + i : r_last;
+            const int ra = PAIR ? r0 + 2 * i : r0 + i;
+            const int r = ra < r_last ? ra : r_last;
             const int soff = (r - r_base) * row_stride;
             P[buf][i] = load_stream16(rs, off_p, soff);
-            if constexpr (use_res) Q[buf][i] = load_stream16(rs, off_q, soff);
+            if constexpr (PAIR) {
+                const int rq = ra + 1 < r_last ? ra + 1 : r_last;
+                Q[buf][i] = load_stream16(rs, off_q, (rq - r_base) * row_stride);
+            } else if constexpr (use_res) {
+                Q[buf][i] = load_stream16(rs, off_q, soff);
+            }
         }
     };
 
@@ -179,36 +201,60 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
         }
     }
 
-    float xt[kChunk];   // rotated activations, kept in registers for the whole kernel
-    rotate_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.img_cols, a.L.seed_primary, a.L.block_size,
+    float xt[NX];       // rotated activations, kept in registers for the whole kernel
+    rotate_image<combined, TILES, PAIR, NX>(raw, a.x_dtype, a.L.in_features, a.img_cols, a.L.seed_primary, a.L.block_size,
                                   reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes), wave, nwaves, lane,
                                   slab, act_a, act_b, xt);
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
     __syncthreads();                                          // tables visible to every wave
 
-    auto decode_row = [&](const uint4& p, const uint4& q, float& sum) {
+    // One row (or with PAIR the same columns of two rows: p -> sum, q -> sum2).
+    auto decode_row = [&](const uint4& p, const uint4& q, float& sum, float& sum2) {
         float val[kChunk];
         lookup32<MODE == kSharedLut, 0>(p, q, smem, laneoff, val);
-        float s0 = 0.0f, s1 = 0.0f;
+        if constexpr (PAIR) {
+            float s0 = 0.0f, s1 = 0.0f, t0 = 0.0f, t1 = 0.0f;
 #pragma unroll
-        for (int k = 0; k < kChunk; k += 2) {
-            s0 = __builtin_fmaf(val[k], xt[k], s0);
-            s1 = __builtin_fmaf(val[k + 1], xt[k + 1], s1);
+            for (int k = 0; k < 16; k += 2) {
+                s0 = __builtin_fmaf(val[k], xt[k], s0);
+                s1 = __builtin_fmaf(val[k + 1], xt[k + 1], s1);
+                t0 = __builtin_fmaf(val[16 + k], xt[k], t0);
+                t1 = __builtin_fmaf(val[17 + k], xt[k + 1], t1);
+            }
+            sum = s0 + s1;
+            sum2 = t0 + t1;
+        } else {
+            float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kChunk; k += 2) {
+                s0 = __builtin_fmaf(val[k], xt[k], s0);
+                s1 = __builtin_fmaf(val[k + 1], xt[k + 1], s1);
+            }
+            sum = s0 + s1;
         }
-        sum = s0 + s1;
     };
 
     auto consume = [&](int buf, int r0, int it) {
         float acc[V];
-        if (r0 + R <= r_end) {                               // wave-uniform: a full group, straight-line
+        float unused = 0.0f;
+        if (r0 + V <= r_end) {                               // wave-uniform: a full group, straight-line
 #pragma unroll
-            for (int i = 0; i < R; ++i) decode_row(P[buf][i], Q[buf][i], acc[i]);
+            for (int i = 0; i < R; ++i) {
+                if constexpr (PAIR) decode_row(P[buf][i], Q[buf][i], acc[2 * i], acc[2 * i + 1]);
+                else decode_row(P[buf][i], Q[buf][i], acc[i], unused);
+            }
         } else {                                             // ragged end of the range: skip the rows past it
 #pragma unroll
             for (int i = 0; i < R; ++i) {
-                acc[i] = 0.0f;
-                if (r0 + i < r_end) decode_row(P[buf][i], Q[buf][i], acc[i]);
+                if constexpr (PAIR) {
+                    acc[2 * i] = 0.0f; acc[2 * i + 1] = 0.0f;
+                    // the second row of a pair past the range is decoded with the first and not stored
+                    if (r0 + 2 * i < r_end) decode_row(P[buf][i], Q[buf][i], acc[2 * i], acc[2 * i + 1]);
+                } else {
+                    acc[i] = 0.0f;
+                    if (r0 + i < r_end) decode_row(P[buf][i], Q[buf][i], acc[i], unused);
+                }
             }
         }
         consumed(nrm[buf]); consumed(gte[buf]);
@@ -237,20 +283,20 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     for (; it0 + NS <= a.iters; it0 += NS) {
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
-            fetch((u + 1) % NS, r_begin + (it0 + u + 1) * R);
-            consume(u, r_begin + (it0 + u) * R, it0 + u);
+            fetch((u + 1) % NS, r_begin + (it0 + u + 1) * V);
+            consume(u, r_begin + (it0 + u) * V, it0 + u);
         }
     }
     if (it0 < a.iters) {
-        fetch(1, r_begin + (it0 + 1) * R);
-        consume(0, r_begin + it0 * R, it0);
+        fetch(1, r_begin + (it0 + 1) * V);
+        consume(0, r_begin + it0 * V, it0);
     }
 }
 
-template <int MODE, int R, int TILES>
+template <int MODE, int R, int TILES, bool PAIR>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
     const size_t lds = (size_t)kRegionBytes + kPartialBytes + (size_t)a.img_cols * sizeof(float);
-    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES>;
+    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR>;
     // More LDS than the default limit has to be asked for, once per kernel and device.
     static bool asked[64] = {};
     int dev = 0;
@@ -266,12 +312,19 @@ hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t
     return hipGetLastError();
 }
 
-template <int MODE>
+// Row pairs are used where the width is an odd number of 1024-column halves.
+bool wants_pairs(const LayerView& L) {
+    return L.mode == kSharedLut && L.in_features % kSlab == kSlab / 2 && L.in_features / (kSlab / 2) >= 3 &&
+           L.in_features <= kMaxImageCols;
+}
+
+template <int MODE, bool PAIR>
 hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     const int out = a.L.out_features;
+    if (PAIR) a.W = a.L.in_features / (kSlab / 2);           // halves per row
     a.S = 16 / a.W;                                          // row streams sharing the CU
     const int threads = a.W * a.S * kWave;
-    const int padded = a.W * kSlab;
+    const int padded = (a.L.in_features + kSlab - 1) / kSlab * kSlab;
     a.img_cols = padded < kMaxImageCols ? padded : kMaxImageCols;
 
     int grid = (out + a.S - 1) / a.S;
@@ -279,32 +332,35 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     if (grid < 1) grid = 1;
     const long long ts = (long long)grid * a.S;
     const int max_rows = (int)((out + ts - 1) / ts);        // longest row range of any stream
-    const int R = max_rows >= 2 ? 2 : 1;
-    a.iters = (max_rows + R - 1) / R;
+    const int per_r = PAIR ? 2 : 1;                         // rows per unit of R
+    const int R = max_rows >= 2 * per_r ? 2 : 1;
+    a.iters = (max_rows + R * per_r - 1) / (R * per_r);
 
     const int ntiles = (a.L.in_features + kTile - 1) / kTile;
     const bool two = ntiles > threads / kWave;              // at most two tiles per wave: checked by the caller
-    if (R == 2) return two ? launch_wide_one<MODE, 2, 2>(a, grid, threads, stream)
-                           : launch_wide_one<MODE, 2, 1>(a, grid, threads, stream);
-    return two ? launch_wide_one<MODE, 1, 2>(a, grid, threads, stream)
-               : launch_wide_one<MODE, 1, 1>(a, grid, threads, stream);
+    if (R == 2) return two ? launch_wide_one<MODE, 2, 2, PAIR>(a, grid, threads, stream)
+                           : launch_wide_one<MODE, 2, 1, PAIR>(a, grid, threads, stream);
+    return two ? launch_wide_one<MODE, 1, 2, PAIR>(a, grid, threads, stream)
+               : launch_wide_one<MODE, 1, 1, PAIR>(a, grid, threads, stream);
 }
 
 }  // namespace
 
-// One batch row, 3 to 8 slabs, blocks of at most 512 columns, shared-rotation or primary-only layers
-// whose per-stream share of the plane stays below 2 GB.
+// One batch row, blocks of at most 512 columns, shared-rotation or primary-only layers whose
+// per-stream share of the plane stays below 2 GB; rows of 3 to 8 slabs, or (shared rotation) of an
+// odd number, 3 to 15, of 1024-column halves.
 bool gemv_wide_supported(const LayerView& L, int num_cus) {
     if (L.mode != kSharedLut && L.mode != kPrimaryOnly) return false;
     if (L.block_size > (uint32_t)kTile) return false;
-    const int W = (L.in_features / kChunk + kWave - 1) / kWave;
-    if (W < 3 || W > 8) return false;
+    int W = (L.in_features / kChunk + kWave - 1) / kWave;
+    if (wants_pairs(L)) W = L.in_features / (kSlab / 2);
+    else if (W < 3 || W > 8) return false;
     const int S = 16 / W;
     const int ntiles = (L.in_features + kTile - 1) / kTile;
     if (ntiles > 2 * W * S) return false;
     const size_t row_bytes = L.mode == kSharedLut ? (size_t)L.in_features : (size_t)L.in_features / 2;
     const long long streams = (long long)(num_cus > 0 ? num_cus : 1) * S;
-    const long long max_rows = (L.out_features + streams - 1) / streams + 2;
+    const long long max_rows = (L.out_features + streams - 1) / streams + 4;
     return (unsigned long long)max_rows * row_bytes < (1ull << 31);
 }
 
@@ -312,8 +368,10 @@ hipError_t launch_gemv_wide(const GemvArgs& base, int num_cus, hipStream_t strea
     GemvArgs a = base;
     a.chunks = a.L.in_features / kChunk;
     a.W = (a.chunks + kWave - 1) / kWave;
-    if (a.L.mode == kSharedLut) return launch_wide_mode<kSharedLut>(a, num_cus, stream);
-    return launch_wide_mode<kPrimaryOnly>(a, num_cus, stream);
+    if (a.L.mode == kSharedLut)
+        return wants_pairs(a.L) ? launch_wide_mode<kSharedLut, true>(a, num_cus, stream)
+                                : launch_wide_mode<kSharedLut, false>(a, num_cus, stream);
+    return launch_wide_mode<kPrimaryOnly, false>(a, num_cus, stream);
 }
 
 }  // namespace tq
