@@ -179,7 +179,7 @@ __device__ __forceinline__ int stage_index(int col_in_slab) {
     }
 }
 
-// One batch row, rows of 3 to 8 slabs (tq_gemv_wide.hip): one workgroup per CU, tables and rotated
+// One batch row, rows of up to 8 slabs (tq_gemv_wide.hip): one workgroup per CU, tables and rotated
 // activations built once per CU.  `a` as for the narrow kernel (x, y, gate already at the batch row).
 bool gemv_wide_supported(const LayerView& L, int num_cus);
 hipError_t launch_gemv_wide(const GemvArgs& a, int num_cus, hipStream_t stream);

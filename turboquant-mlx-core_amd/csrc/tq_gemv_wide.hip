@@ -1,15 +1,17 @@
-// Fused TQ8 dequant + GEMV for gfx950, one batch row, rows of 3 to 8 slabs (4097..16384 columns).
+// Fused TQ8 dequant + GEMV for gfx950, one batch row, rows of up to 8 slabs (16384 columns), blocks
+// of at most 512 columns, shared-rotation and primary-only layers: the batch-1 decode kernel.
 //
 // Same mathematics and same per-lane work as tq_gemv.hip (a lane owns 32 columns of a 2048-column
 // slab, lane-private centroid table in LDS, rotated activations in registers).  What differs is the
-// shape of the workgroup.  For these widths the narrow kernel has room for only one or two row
-// streams per workgroup, so every stream rotated the activation row for itself, which cost as much
-// as decoding a dozen rows.  Here ONE workgroup of up to 16 waves runs per CU:
+// shape of the workgroup.  The other kernel runs two workgroups of up to 8 waves per CU; from three
+// slabs on that leaves room for only one or two row streams per workgroup, and every stream
+// rotated the activation row for itself, which cost as much as decoding a dozen rows.  Here ONE
+// workgroup of up to 16 waves runs per CU:
 //   * the decode table is built once per CU;
 //   * the activation row is rotated once per CU: the waves split its 512-column tiles among
 //     themselves and hand the result over through an image of the whole row in LDS (up to 64 KB);
-//   * 16 / W row streams share the CU, each with W waves (one per slab) and a cross-wave sum per
-//     row group.
+//   * 16 / W row streams share the CU, each with W waves (one per slab) and, for W > 1, a
+//     cross-wave sum per row group.
 // Rows whose width is an odd number of 1024-column halves (5120 = 5 x 1024) would leave half of the
 // last slab's wave idle.  For those (PAIR) a wave owns one 1024-column half instead, 16 columns per
 // lane, and its two 16-byte loads fetch the same columns of two consecutive rows.
@@ -264,12 +266,19 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
         const int r = r0 + lane;
         const bool owner = lane < V && r < r_end;
 
-        float* buf_base = partial + (it & 1) * (16 * 16);
-        if (lane < V) buf_base[wave * V + lane] = total;
-        __syncthreads();
-        if (slab == 0 && owner) {
-            float t = 0.0f;
-            for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * V + lane];
+        float t = total;
+        bool store = owner;
+        if (a.W > 1) {                                       // cross-wave sum of the row's slabs
+            float* buf_base = partial + (it & 1) * (16 * 16);
+            if (lane < V) buf_base[wave * V + lane] = total;
+            __syncthreads();
+            store = owner && slab == 0;
+            if (store) {
+                t = 0.0f;
+                for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * V + lane];
+            }
+        }
+        if (store) {
             t *= row_scale;
             if (a.gate) { const float g = gte[buf]; t = g / (1.0f + expf(-g)) * t; }   // silu(gate) * y
             store_scalar(a.y, a.y_dtype, (size_t)r, t);
@@ -347,14 +356,14 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
 }  // namespace
 
 // One batch row, blocks of at most 512 columns, shared-rotation or primary-only layers whose
-// per-stream share of the plane stays below 2 GB; rows of 3 to 8 slabs, or (shared rotation) of an
+// per-stream share of the plane stays below 2 GB; rows of 1 to 8 slabs, or (shared rotation) of an
 // odd number, 3 to 15, of 1024-column halves.
 bool gemv_wide_supported(const LayerView& L, int num_cus) {
     if (L.mode != kSharedLut && L.mode != kPrimaryOnly) return false;
     if (L.block_size > (uint32_t)kTile) return false;
     int W = (L.in_features / kChunk + kWave - 1) / kWave;
     if (wants_pairs(L)) W = L.in_features / (kSlab / 2);
-    else if (W < 3 || W > 8) return false;
+    else if (W < 1 || W > 8) return false;
     const int S = 16 / W;
     const int ntiles = (L.in_features + kTile - 1) / kTile;
     if (ntiles > 2 * W * S) return false;
