@@ -24,7 +24,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152437.9 KiB + 647.2 KiB.
-MEASURED_TRAFFIC_BYTES = 312855552
+MEASURED_TRAFFIC_BYTES = 312822886
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
 
@@ -163,6 +163,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-extra", action="store_true", help="measure the headline configuration only")
+    ap.add_argument("--decoder-layer-only", action="store_true",
+                    help="of the extra measurements, run only the decoder-layer projections (for kernel profiles)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy three times (reference reading for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -214,7 +216,7 @@ def main():
         "us_per_layer": us,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "tq_gemv_kernel<shared,1,2,1024>", "algorithmic_bytes": B},
+                     "kernel": "tq_gemv_wide_kernel<shared, R=2, TILES=1>", "algorithmic_bytes": B},
     }
 
     # ---- CPU baseline on this host ---------------------------------------------------
@@ -252,94 +254,96 @@ def main():
     if args.skip_extra:
         finish(args, torch, extra, result)
         return
-    out1, in1 = 4096, 4096
-    copies = 32                         # 32 x 16.8 MB > 256 MB of last-level cache: HBM-resident timing
-    handles = [make_layer(tq, torch, out1, in1, bs, seed=100 + 2 * i, sigma=0.02, shared=True)[0] for i in range(copies)]
-    x1 = torch.randn(1, in1, device="cuda", generator=g)
-    y1 = torch.empty(1, out1, device="cuda", dtype=torch.float32)
-    steps1 = max(args.steps, copies) // copies * copies
-    us_hbm = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
-    us_hot = time_graph(tq, torch, handles[:1], x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
-    B1 = algorithmic_bytes(out1, in1, 1, 4, 4)
-    extra["gemv_4096x4096_f32_bs1"] = {"us_per_layer_hbm_resident": us_hbm, "us_per_layer_cache_resident": us_hot,
-                                       "weight_copies_cycled": copies, "algorithmic_bytes": B1,
-                                       "hbm_frac": B1 / (us_hbm * 1e-6) / 1e9 / HBM_PEAK_GBS}
-    for h in handles:
-        tq.lib().tq_linear_free(h)
-    # the library default of the reference is dual rotation (include/turboquant/quantizer.h:15)
-    handles = [make_layer(tq, torch, out1, in1, bs, seed=300 + 2 * i, sigma=0.02, shared=False)[0] for i in range(copies)]
-    us_dual = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
-    extra["gemv_4096x4096_f32_bs1_dual_rotation"] = {"us_per_layer_hbm_resident": us_dual,
-                                                     "hbm_frac": B1 / (us_dual * 1e-6) / 1e9 / HBM_PEAK_GBS}
-    for h in handles:
-        tq.lib().tq_linear_free(h)
-    del handles
-    torch.cuda.empty_cache()
-
-    # ---- prefill: Qwen2.5-32B up-projection 27648 x 5120, M = 512 and 2048, bf16 in / bf16 out ----
-    outp, inp = 27648, 5120
-    hp, _ = make_layer(tq, torch, outp, inp, bs, seed=500, sigma=0.01, shared=True, per_layer_codebooks=True)
-    for M in (512, 2048):
-        xp = torch.randn(M, inp, device="cuda", generator=g).to(torch.bfloat16)
-        yp = torch.empty(M, outp, device="cuda", dtype=torch.bfloat16)
-        L = tq.lib()
-        for _ in range(2):
-            if L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None) != 0:
-                raise RuntimeError(tq.last_error())
-        torch.cuda.synchronize()
-        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        reps = 10
-        st.record()
-        for _ in range(reps):
-            L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None)
-        en.record()
-        torch.cuda.synchronize()
-        usp = st.elapsed_time(en) * 1e3 / reps
-        flops = 2.0 * M * outp * inp
-        extra[f"prefill_27648x5120_M{M}_bf16"] = {"us_per_layer": usp, "tflops": flops / usp / 1e6,
-                                                  "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
-                                                  "frac_of_measured_mfma_loop_random_operands":
-                                                      flops / usp / 1e6 / probes.get("mfma_bf16_tflops_random_operands",
-                                                                                     float("nan")),
-                                                  "includes": "activation rotation kernel + dequant/MFMA GEMM kernel"}
-    tq.lib().tq_linear_free(hp)
-    torch.cuda.empty_cache()
-
-    # ---- decode MLP block, Qwen2.5-7B shape: gate/up 18944 x 3584, down 3584 x 18944, batch 1 ----
-    L = tq.lib()
-    hid, inter = 3584, 18944
-    for shared in (False, True):
-        blocks, keep = [], []
-        for c in range(2):                       # two blocks of 204 MB cycled: HBM-resident weights
-            hs = [make_layer(tq, torch, o_, i_, bs, seed=700 + 10 * c + k, sigma=0.015, shared=shared,
-                             per_layer_codebooks=True)[0]
-                  for k, (o_, i_) in enumerate([(inter, hid), (inter, hid), (hid, inter)])]
-            m = L.tq_mlp_create(hs[0], hs[1], hs[2], 1)
-            if not m:
-                raise RuntimeError(tq.last_error())
-            blocks.append(m); keep.append(hs)
-        xm = torch.randn(1, hid, device="cuda", generator=g).to(torch.bfloat16)
-        ym = torch.empty(1, hid, device="cuda", dtype=torch.float32)
-        turn = [0]
-
-        def mlp_step(s):
-            if L.tq_mlp_forward(blocks[turn[0] % 2], xm.data_ptr(), tq.BF16, 1, ym.data_ptr(), tq.F32, s) != 0:
-                raise RuntimeError(tq.last_error())
-            turn[0] += 1
-        steps_m = max(2, args.steps // 2 * 2)
-        us_m = time_graph_fn(torch, mlp_step, steps_m, 2) * 1e6
-        Bm = 2 * algorithmic_bytes(inter, hid, 1, 2, 4) + algorithmic_bytes(hid, inter, 1, 4, 4)
-        extra["mlp_block_7b_bs1_" + ("shared_rotation" if shared else "dual_rotation")] = {
-            "us_per_block": us_m, "algorithmic_bytes": Bm, "hbm_frac": Bm / (us_m * 1e-6) / 1e9 / HBM_PEAK_GBS,
-            "kernels_per_block": 3}
-        for m in blocks:
-            L.tq_mlp_free(m)
-        for hs in keep:
-            for h in hs:
-                L.tq_linear_free(h)
+    if not args.decoder_layer_only:
+        out1, in1 = 4096, 4096
+        copies = 32                         # 32 x 16.8 MB > 256 MB of last-level cache: HBM-resident timing
+        handles = [make_layer(tq, torch, out1, in1, bs, seed=100 + 2 * i, sigma=0.02, shared=True)[0] for i in range(copies)]
+        x1 = torch.randn(1, in1, device="cuda", generator=g)
+        y1 = torch.empty(1, out1, device="cuda", dtype=torch.float32)
+        steps1 = max(args.steps, copies) // copies * copies
+        us_hbm = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
+        us_hot = time_graph(tq, torch, handles[:1], x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
+        B1 = algorithmic_bytes(out1, in1, 1, 4, 4)
+        extra["gemv_4096x4096_f32_bs1"] = {"us_per_layer_hbm_resident": us_hbm, "us_per_layer_cache_resident": us_hot,
+                                           "weight_copies_cycled": copies, "algorithmic_bytes": B1,
+                                           "hbm_frac": B1 / (us_hbm * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        for h in handles:
+            tq.lib().tq_linear_free(h)
+        # the library default of the reference is dual rotation (include/turboquant/quantizer.h:15)
+        handles = [make_layer(tq, torch, out1, in1, bs, seed=300 + 2 * i, sigma=0.02, shared=False)[0] for i in range(copies)]
+        us_dual = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
+        extra["gemv_4096x4096_f32_bs1_dual_rotation"] = {"us_per_layer_hbm_resident": us_dual,
+                                                         "hbm_frac": B1 / (us_dual * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        for h in handles:
+            tq.lib().tq_linear_free(h)
+        del handles
         torch.cuda.empty_cache()
 
+        # ---- prefill: Qwen2.5-32B up-projection 27648 x 5120, M = 512 and 2048, bf16 in / bf16 out ----
+        outp, inp = 27648, 5120
+        hp, _ = make_layer(tq, torch, outp, inp, bs, seed=500, sigma=0.01, shared=True, per_layer_codebooks=True)
+        for M in (512, 2048):
+            xp = torch.randn(M, inp, device="cuda", generator=g).to(torch.bfloat16)
+            yp = torch.empty(M, outp, device="cuda", dtype=torch.bfloat16)
+            L = tq.lib()
+            for _ in range(2):
+                if L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None) != 0:
+                    raise RuntimeError(tq.last_error())
+            torch.cuda.synchronize()
+            st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 10
+            st.record()
+            for _ in range(reps):
+                L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None)
+            en.record()
+            torch.cuda.synchronize()
+            usp = st.elapsed_time(en) * 1e3 / reps
+            flops = 2.0 * M * outp * inp
+            extra[f"prefill_27648x5120_M{M}_bf16"] = {"us_per_layer": usp, "tflops": flops / usp / 1e6,
+                                                      "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
+                                                      "frac_of_measured_mfma_loop_random_operands":
+                                                          flops / usp / 1e6 / probes.get("mfma_bf16_tflops_random_operands",
+                                                                                         float("nan")),
+                                                      "includes": "activation rotation kernel + dequant/MFMA GEMM kernel"}
+        tq.lib().tq_linear_free(hp)
+        torch.cuda.empty_cache()
+
+        # ---- decode MLP block, Qwen2.5-7B shape: gate/up 18944 x 3584, down 3584 x 18944, batch 1 ----
+        L = tq.lib()
+        hid, inter = 3584, 18944
+        for shared in (False, True):
+            blocks, keep = [], []
+            for c in range(2):                       # two blocks of 204 MB cycled: HBM-resident weights
+                hs = [make_layer(tq, torch, o_, i_, bs, seed=700 + 10 * c + k, sigma=0.015, shared=shared,
+                                 per_layer_codebooks=True)[0]
+                      for k, (o_, i_) in enumerate([(inter, hid), (inter, hid), (hid, inter)])]
+                m = L.tq_mlp_create(hs[0], hs[1], hs[2], 1)
+                if not m:
+                    raise RuntimeError(tq.last_error())
+                blocks.append(m); keep.append(hs)
+            xm = torch.randn(1, hid, device="cuda", generator=g).to(torch.bfloat16)
+            ym = torch.empty(1, hid, device="cuda", dtype=torch.float32)
+            turn = [0]
+
+            def mlp_step(s):
+                if L.tq_mlp_forward(blocks[turn[0] % 2], xm.data_ptr(), tq.BF16, 1, ym.data_ptr(), tq.F32, s) != 0:
+                    raise RuntimeError(tq.last_error())
+                turn[0] += 1
+            steps_m = max(2, args.steps // 2 * 2)
+            us_m = time_graph_fn(torch, mlp_step, steps_m, 2) * 1e6
+            Bm = 2 * algorithmic_bytes(inter, hid, 1, 2, 4) + algorithmic_bytes(hid, inter, 1, 4, 4)
+            extra["mlp_block_7b_bs1_" + ("shared_rotation" if shared else "dual_rotation")] = {
+                "us_per_block": us_m, "algorithmic_bytes": Bm, "hbm_frac": Bm / (us_m * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                "kernels_per_block": 3}
+            for m in blocks:
+                L.tq_mlp_free(m)
+            for hs in keep:
+                for h in hs:
+                    L.tq_linear_free(h)
+            torch.cuda.empty_cache()
+
     # ---- decoder-layer projections, Qwen2.5-32B shape, batch 1 / 4 / 8, bf16 activations ----
+    L = tq.lib()
     shapes = [("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120, 5120),
               ("gate", 27648, 5120), ("up", 27648, 5120), ("down", 5120, 27648)]
     layers = [(n_, o_, i_, make_layer(tq, torch, o_, i_, bs, seed=900 + k, sigma=0.01, shared=True,
