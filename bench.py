@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152437.9 KiB + 647.2 KiB.
+# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152421.1 KiB + 648.9 KiB.
 MEASURED_TRAFFIC_BYTES = 312822886
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
