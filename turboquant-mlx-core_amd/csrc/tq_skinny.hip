@@ -15,6 +15,7 @@
 // second small kernel adds the chunks, applies the row norm and converts.
 // The rotated activations come from tq_rotate_bf16_kernel (tile images, see tq_prefill.hip).
 #include "tq_device.h"
+#include "tq_gemv_common.h"
 
 namespace tq {
 
@@ -27,7 +28,10 @@ constexpr int kSkThreads = 512;          // 8 waves per workgroup, one workgroup
 constexpr int kSkLutBytes = 256 * 256;
 
 struct SkinnyArgs {
-    const uint16_t* xt;        // rotated activations, bf16 tile images [K/32][256 rows x 64 B] (rows >= batch unset)
+    const void* x;             // FUSED: activations [batch, K], f16 or bf16
+    int x_dtype;
+    uint32_t seed, block_size; // FUSED: rotation of the layer (blocks of at most 512 columns)
+    const uint16_t* xt;        // otherwise: rotated activations, bf16 tile images [K/32][256 rows x 64 B] (rows >= batch unset)
     const uint8_t* plane;      // combined bytes [N, K]
     const float* tables;       // 256-entry sum table
     float* partial;            // [chunks][16][N] fp32
@@ -46,6 +50,9 @@ __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t l
     }
 }
 
+// FUSED: the workgroup rotates the 16 x 512 activations of its chunk itself (blocks of at most 512
+// columns: a block never leaves the chunk), instead of reading tile images a separate kernel wrote.
+template <bool FUSED>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tq_skinny_kernel(SkinnyArgs a) {
     __shared__ __align__(16) char smem[kSkLutBytes];
     const int tid = threadIdx.x;
@@ -53,30 +60,71 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t laneoff = (uint32_t)lane << 2;
 
-    // Decode table -> LDS, one private column per lane, values rounded to bf16 (upper half of the dword).
-    {
-        uint4* dst = reinterpret_cast<uint4*>(smem);
-        for (int i = tid; i < 256 * 16; i += kSkThreads) {
-            const uint32_t v = (uint32_t)float_to_bf16_bits(a.tables[i >> 4]) << 16;
-            dst[i] = make_uint4(v, v, v, v);
-        }
-    }
-
     const int chunk = blockIdx.x % a.chunks;
     const int wg_in_chunk = blockIdx.x / a.chunks;
     const int m = lane & 15, g = lane >> 4;               // A operand: batch row, k group; B operand: weight row, k group
 
+    // Table values of this thread's LDS slots, requested before anything else.
+    constexpr int kSlots = 256 * 16 / kSkThreads;
+    float tv[kSlots];
+#pragma unroll
+    for (int k = 0; k < kSlots; ++k) tv[k] = a.tables[(tid + k * kSkThreads) >> 4];
+
+    sk_bf16x8 afrag[16];
+    if constexpr (FUSED) {
+        // Wave w rotates batch rows w and w + 8 of the chunk (one 512-column tile each, 8 values per
+        // lane) and writes them as bf16 into the first 16 KB of the table region, [16 rows][512];
+        // rows past the batch are zero.  The A operands are read back before the table is built.
+        constexpr int kPitch = kSkChunk * 2;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int b = wave + 8 * t;
+            const int col = chunk * kSkChunk + lane * 8;
+            uint4 packed = make_uint4(0, 0, 0, 0);
+            if (b < a.batch) {                              // wave-uniform
+                TileRaw raw;
+                raw.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) + (size_t)b * a.K + col);
+                raw.b = make_uint4(0, 0, 0, 0);
+                float v[8];
+                rotate_tile(raw, a.x_dtype, col, true, a.seed, a.block_size, lane, v);
+                packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+                packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+                packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
+                packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
+            }
+            *reinterpret_cast<uint4*>(smem + b * kPitch + lane * 16) = packed;
+        }
+        __syncthreads();
+        // k-step s covers columns 64 (s/2) + 16 g + 8 (s%2) + [0, 8) of the chunk, the same columns
+        // the B operand of that step decodes.
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+            afrag[s] = *reinterpret_cast<const sk_bf16x8*>(smem + m * kPitch + (64 * (s >> 1) + 16 * g + 8 * (s & 1)) * 2);
+        __syncthreads();                                    // everyone has its A operands: the region is free
+    }
+
+    // Decode table -> LDS, one private column per lane, values rounded to bf16 (upper half of the dword).
+    {
+        uint4* dst = reinterpret_cast<uint4*>(smem);
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) {
+            const uint32_t v = (uint32_t)float_to_bf16_bits(tv[k]) << 16;
+            dst[tid + k * kSkThreads] = make_uint4(v, v, v, v);
+        }
+    }
+
     // A operands of the chunk: k-step s covers columns 64 (s/2) + 16 g + 8 (s%2) + [0, 8) of the chunk,
     // the same columns the B operand of that step decodes (any column order is fine as long as both
     // operands agree).  Tile images: [K/32][256][32] bf16 with 16-byte slots XOR-permuted per row.
-    sk_bf16x8 afrag[16];
+    if constexpr (!FUSED) {
 #pragma unroll
-    for (int s = 0; s < 16; ++s) {
-        const int off = 16 * g + 8 * (s & 1);              // column inside the 64-column piece
-        const int kt = chunk * 16 + 2 * (s >> 1) + (off >> 5);
-        const int slot = ((off & 31) >> 3) ^ ((m >> 2) & 3);
-        afrag[s] = *reinterpret_cast<const sk_bf16x8*>(reinterpret_cast<const char*>(a.xt) +
-                                                       ((size_t)kt * 256 + m) * 64 + slot * 16);
+        for (int s = 0; s < 16; ++s) {
+            const int off = 16 * g + 8 * (s & 1);              // column inside the 64-column piece
+            const int kt = chunk * 16 + 2 * (s >> 1) + (off >> 5);
+            const int slot = ((off & 31) >> 3) ^ ((m >> 2) & 3);
+            afrag[s] = *reinterpret_cast<const sk_bf16x8*>(reinterpret_cast<const char*>(a.xt) +
+                                                           ((size_t)kt * 256 + m) * 64 + slot * 16);
+        }
     }
     __syncthreads();                                       // table visible
 
@@ -170,9 +218,14 @@ size_t skinny_partial_bytes(const LayerView& L) {
 // xt_workspace: as for launch_prefill (prefill_workspace_bytes); partial: skinny_partial_bytes.
 hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                          void* xt_workspace, float* partial, int num_cus, hipStream_t stream) {
-    hipError_t e = launch_rotate_tiles(L, x, x_dtype, batch, xt_workspace, stream);
-    if (e != hipSuccess) return e;
+    const bool fused = L.block_size <= (uint32_t)kSkChunk;
+    hipError_t e = hipSuccess;
+    if (!fused) {
+        e = launch_rotate_tiles(L, x, x_dtype, batch, xt_workspace, stream);
+        if (e != hipSuccess) return e;
+    }
     SkinnyArgs a{};
+    a.x = x; a.x_dtype = x_dtype; a.seed = L.seed_primary; a.block_size = L.block_size;
     a.xt = static_cast<const uint16_t*>(xt_workspace);
     a.plane = L.packed_combined;
     a.tables = L.tables;
@@ -181,7 +234,8 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     a.chunks = L.in_features / kSkChunk;
     a.groups = (L.out_features + 15) / 16;
     a.wgs_per_chunk = 2 * num_cus / a.chunks > 0 ? 2 * num_cus / a.chunks : 1;   // two workgroups per CU
-    hipLaunchKernelGGL(tq_skinny_kernel, dim3(a.wgs_per_chunk * a.chunks), dim3(kSkThreads), 0, stream, a);
+    if (fused) hipLaunchKernelGGL(tq_skinny_kernel<true>, dim3(a.wgs_per_chunk * a.chunks), dim3(kSkThreads), 0, stream, a);
+    else hipLaunchKernelGGL(tq_skinny_kernel<false>, dim3(a.wgs_per_chunk * a.chunks), dim3(kSkThreads), 0, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     const size_t total = (size_t)batch * L.out_features;
