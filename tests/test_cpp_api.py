@@ -220,3 +220,117 @@ def test_tq_model_dequant_directory(tmp_path, oracle, passthrough_dtype):
             assert got[k].dtype == np.float16
             assert np.array_equal(got[k], w_ref.astype(np.float16)), k
         assert np.array_equal(got["model.norm.weight"], np.linspace(-1, 1, 8).astype(np.float16))
+
+
+# --------------------------------------------------------------------------- command-line tools
+CLI = os.path.join(entry.ROOT, "turboquant-mlx-core_amd", "bin")
+
+
+def test_cli_usage_and_version():
+    """tq-convert / tq-dequant-model (reference tools/): argument handling needs no GPU."""
+    for exe in ("tq-convert", "tq-dequant-model"):
+        assert os.path.exists(os.path.join(CLI, exe)), "build first (python __graft_entry__.py)"
+    p = subprocess.run([os.path.join(CLI, "tq-convert"), "--version"], capture_output=True, text=True)
+    assert p.returncode == 0 and p.stdout.startswith("tq-convert ")
+    p = subprocess.run([os.path.join(CLI, "tq-convert")], capture_output=True, text=True)
+    assert p.returncode == 1 and "Usage: tq-convert --model" in p.stdout
+    p = subprocess.run([os.path.join(CLI, "tq-convert"), "--bits", "4"], capture_output=True, text=True)
+    assert p.returncode == 1 and "--model is required" in p.stderr
+    p = subprocess.run([os.path.join(CLI, "tq-dequant-model"), "only-one-argument"], capture_output=True, text=True)
+    assert p.returncode == 1 and "Usage:" in p.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("per_layer,shared", [(True, True), (False, False)])
+def test_cli_convert_then_dequant_model_directory(tmp_path, oracle, per_layer, shared):
+    """tq-convert on a small HuggingFace-style directory written with the `safetensors` package,
+    then tq-dequant-model on its output.  Checked: which tensors are quantized (2-D "*.weight"
+    outside the sensitive first / last layer), the TQ8 tensor names, shapes, dtypes and metadata,
+    the block size chosen per layer, config.json, the pass-through shard, that the packed bytes
+    are the ones the CPU oracle's quantizer produces from the same weight and codebooks, and that
+    the round trip returns every tensor (quantized ones within the 8-bit quantization error)."""
+    rng = np.random.default_rng(7)
+    src = tmp_path / "model"
+    src.mkdir()
+    (src / "config.json").write_text(json.dumps({"model_type": "toy", "num_hidden_layers": 4}, indent=2))
+    (src / "tokenizer.txt").write_text("not a tensor file")
+    tensors = {"model.embed_tokens.weight": (rng.standard_normal((96, 64)) * 0.05).astype(np.float16),
+               "lm_head.weight": (rng.standard_normal((96, 64)) * 0.05).astype(np.float32),
+               "model.norm.weight": np.ones(64, np.float32),
+               "model.layers.1.mlp.odd.weight": (rng.standard_normal((8, 48)) * 0.05).astype(np.float32)}
+    for n in range(4):
+        tensors[f"model.layers.{n}.self_attn.q_proj.weight"] = (rng.standard_normal((64, 64)) * 0.05).astype(np.float32)
+        tensors[f"model.layers.{n}.mlp.up_proj.weight"] = (rng.standard_normal((160, 1536)) * 0.02).astype(np.float16)
+        tensors[f"model.layers.{n}.self_attn.q_proj.bias"] = rng.standard_normal(64).astype(np.float32)
+        tensors[f"model.layers.{n}.input_layernorm.weight"] = np.ones(64, np.float32)
+    save_file(tensors, str(src / "model.safetensors"))
+
+    out = tmp_path / "model-tq"
+    args = [os.path.join(CLI, "tq-convert"), "--model", str(src), "--output", str(out), "--sensitive-layers", "1"]
+    if per_layer:
+        args.append("--per-layer-codebooks")
+    if shared:
+        args.append("--shared-rotation")
+    p = subprocess.run(args, capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "Sensitive layers: 4 weights kept at fp16, 6 weights quantized" in p.stdout
+    assert "model.layers.1.mlp.odd.weight [8, 48] left unquantized" in p.stderr
+
+    cfg = json.loads((out / "config.json").read_text())
+    assert cfg["model_type"] == "toy"
+    assert cfg["quantization_config"] == {"quantization_method": "turboquant", "tq_version": "1", "bits": 4,
+                                          "residual_bits": 4, "block_size": 512, "shared_rotation": shared,
+                                          "sensitive_layers_start": 1, "sensitive_layers_end": 1}
+    assert (out / "tokenizer.txt").read_text() == "not a tensor file"
+
+    meta = _metadata(str(out / "model.safetensors"))
+    assert meta["quantization_method"] == "turboquant" and meta["tq_version"] == "1"
+    assert meta["tq_primary_bits"] == "4" and meta["tq_residual_bits"] == "4" and meta["tq_total_bits"] == "8"
+    assert (meta.get("tq_per_layer_codebooks") == "true") == per_layer
+    tq_t = load_file(str(out / "model.safetensors"))
+    pt = load_file(str(out / "model_passthrough.safetensors"))
+    quantized = ["model.embed_tokens", "lm_head"] + [f"model.layers.{n}.{m}" for n in (1, 2)
+                                                      for m in ("self_attn.q_proj", "mlp.up_proj")]
+    assert sorted(k[:-len(".packed_primary")] for k in tq_t if k.endswith(".packed_primary")) == sorted(quantized)
+    for name in quantized:
+        w = tensors[name + ".weight"].astype(np.float32)
+        o_f, i_f = w.shape
+        bs = 512 if i_f == 1536 else 64                              # largest power of two <= 512 dividing the width
+        assert tq_t[name + ".packed_primary"].shape == (o_f, i_f // 2) and tq_t[name + ".packed_primary"].dtype == np.uint8
+        assert tq_t[name + ".packed_residual"].shape == (o_f, i_f // 2)
+        assert tq_t[name + ".norms"].shape == (o_f,) and tq_t[name + ".norms"].dtype == np.float32
+        seeds = tq_t[name + ".seeds"]
+        assert seeds.dtype == np.uint32 and seeds.shape == (3,) and seeds[2] == bs
+        assert (seeds[1] == 0) == shared
+        assert (name + ".codebook_primary" in tq_t) == per_layer
+        # the same weight through the CPU oracle's quantizer with the codebooks of the file
+        cbp = oracle.Codebook(tq_t[name + ".codebook_primary"] if per_layer else tq_t["tq_codebook_primary"], 4)
+        cbr = oracle.Codebook(tq_t[name + ".codebook_residual"] if per_layer else tq_t["tq_codebook_residual"], 4)
+        qw = oracle.quantize_weight(w, cbp, cbr, 4, 4, bs, shared)
+        assert np.array_equal(qw.seeds, seeds)
+        same = np.mean(qw.packed_primary == tq_t[name + ".packed_primary"])
+        assert same > 0.999                                          # boundary ties may round differently on the GPU
+        assert np.allclose(qw.norms, tq_t[name + ".norms"], rtol=1e-4)
+    # pass-through: 1-D tensors, biases, the sensitive layers 0 and 3, the weight the quantizer cannot take
+    kept = [k for k in tensors if k not in {q + ".weight" for q in quantized}]
+    assert sorted(pt) == sorted(kept)
+    for k in kept:
+        assert pt[k].dtype == tensors[k].dtype and np.array_equal(pt[k], tensors[k])
+
+    deq = tmp_path / "model-deq"
+    p = subprocess.run([os.path.join(CLI, "tq-dequant-model"), str(out), str(deq)], capture_output=True, text=True,
+                       timeout=600)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "quantization_config" not in json.loads((deq / "config.json").read_text())
+    back = {}
+    for f in os.listdir(deq):
+        if f.endswith(".safetensors"):
+            back.update(load_file(str(deq / f)))
+    assert sorted(back) == sorted(tensors)
+    for k, v in tensors.items():
+        got = back[k].astype(np.float32)
+        if k[:-len(".weight")] in quantized:
+            rel = np.linalg.norm(got - v.astype(np.float32)) / np.linalg.norm(v.astype(np.float32))
+            assert rel < 0.15, (k, rel)                              # the bound of the reference's own round-trip tests
+        else:
+            assert np.array_equal(got, v.astype(np.float32))
