@@ -106,13 +106,14 @@ def test_forward_fp32(tq, oracle, mode, out, inf, bs, batch):
     assert np.abs(y - want).max() < 0.15                     # the reference's own bound, test_linear.cpp:135
 
 
-@pytest.mark.parametrize("mode", ["shared", "primary_only"])
+@pytest.mark.parametrize("mode", ["shared", "primary_only", "dual"])
 @pytest.mark.parametrize("out,inf,bs", [(1000, 3072, 512), (777, 5120, 512), (5000, 5120, 128), (600, 6144, 512),
                                         (515, 7168, 256), (300, 8192, 512), (64, 9216, 512), (260, 15360, 512),
                                         (130, 16384, 512), (3, 5120, 512), (2049, 12288, 64)])
 def test_forward_batch1_wide_rows(tq, oracle, mode, out, inf, bs):
     """One activation row on rows of 3 to 8 slabs (and, shared rotation, of an odd number of
-    1024-column halves, which are served two rows at a time): the one-workgroup-per-CU kernel.
+    1024-column halves, which are served two rows at a time; dual rotation up to 4 slabs, the waves
+    of a row split by plane): the one-workgroup-per-CU kernel.
     Row counts are chosen so that streams get ragged, empty and single-row ranges; fp32 and bf16
     activations; every output against the oracle within the fp32 tolerance."""
     qw, cbp, cbr = _make(oracle, out, inf, bs, mode)

@@ -385,7 +385,8 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
         hipError_t e;
         int step = 1;
         if constexpr (MODE == kDual) {
-            e = (W <= 8) ? launch_nb<MODE, 1, 512>(a, num_cus, stream) : launch_nb<MODE, 1, 1024>(a, num_cus, stream);
+            if (gemv_wide_supported(a.L, num_cus)) e = launch_gemv_wide(a, num_cus, stream);
+            else e = (W <= 8) ? launch_nb<MODE, 1, 512>(a, num_cus, stream) : launch_nb<MODE, 1, 1024>(a, num_cus, stream);
         } else {
             if (left >= 4 && W <= 8)      { step = 4; e = launch_nb<MODE, 4, 512>(a, num_cus, stream); }
             else if (left >= 2 && W <= 8) { step = 2; e = launch_nb<MODE, 2, 512>(a, num_cus, stream); }

@@ -15,6 +15,12 @@
 // Rows whose width is an odd number of 1024-column halves (5120 = 5 x 1024) would leave half of the
 // last slab's wave idle.  For those (PAIR) a wave owns one 1024-column half instead, 16 columns per
 // lane, and its two 16-byte loads fetch the same columns of two consecutive rows.
+// Dual rotation (two nibble planes, each with its own rotation and 16-entry table): the waves of a
+// row are split by plane, even units decode the primary plane against the primary rotation, odd
+// units the residual plane against the residual rotation, and the cross-wave sum adds the two.
+// A wave then needs one rotated activation vector and one table, as for a primary-only layer, and
+// the kernel keeps its 16 waves per CU (the other kernel, holding both rotations in registers,
+// fits 8).
 // Every trip of the main loop issues the same loads whatever is left of a stream's row range
 // (past it they re-read its last row), and everything loaded is marked as consumed on every path,
 // so the compiler knows exactly how many loads are in flight and waits for no more than the row
@@ -60,10 +66,11 @@ __device__ __forceinline__ TileRaw load_tile_fixed(const void* x, int x_dtype, i
 // 32 values of the columns it owns.  raw[t] holds the activations of tile wave + t * nwaves (any
 // valid address for tiles past the row).
 // unit: the slab of the wave, or with PAIR its 1024-column half (xt then holds 16 values).
+// take: whether this wave picks up its values from this rotation (dual rotation runs two).
 template <bool SPLIT, int TILES, bool PAIR, int NX>
 __device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_dtype, int in_features,
                                              int img_cols, uint32_t seed, uint32_t bs, float* image, int wave,
-                                             int nwaves, int lane, int unit, bool act_a, bool act_b,
+                                             int nwaves, int lane, int unit, bool act_a, bool act_b, bool take,
                                              float (&xt)[NX]) {
     const int rounds = (in_features + img_cols - 1) / img_cols;
     for (int p = 0; p < rounds; ++p) {
@@ -83,13 +90,13 @@ __device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_
         __syncthreads();
         if constexpr (PAIR) {
             const int first = unit * (kSlab / 2);                 // first column of the half
-            if (first / img_cols == p) {
+            if (take && first / img_cols == p) {
                 const float* src = image + ((first % img_cols) & ~(kSlab - 1)) + ((unit & 1) << 4) * kWave + lane;
 #pragma unroll
                 for (int k = 0; k < NX; ++k) xt[k] = src[k * kWave];
             }
         } else {
-            if ((unit * kSlab) / img_cols == p) {
+            if (take && (unit * kSlab) / img_cols == p) {
                 const float* src = image + (unit * kSlab) % img_cols + lane;
 #pragma unroll
                 for (int k = 0; k < NX; ++k)
@@ -99,7 +106,8 @@ __device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_
     }
 }
 
-// MODE: kSharedLut (combined byte plane) or kPrimaryOnly.  R rows per group, TILES activation tiles
+// MODE: kSharedLut (combined byte plane), kPrimaryOnly, or kDual (a.W counts slab-plane pairs: unit
+// 2 s is slab s of the primary plane, unit 2 s + 1 slab s of the residual plane).  R rows per group, TILES activation tiles
 // per wave (the host checks that TILES * waves covers the row and that blocks are at most 512 wide).
 // PAIR (combined plane only): a.W counts 1024-column halves; a group is R row pairs.
 template <int MODE, int R, int TILES, bool PAIR>
@@ -115,8 +123,10 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = blockDim.x >> 6;
-    const int slab = wave % a.W;
+    const int unit = wave % a.W;
     const int stream = wave / a.W;
+    const int slab = (MODE == kDual) ? unit >> 1 : unit;
+    const int plane = (MODE == kDual) ? unit & 1 : 0;       // 0: primary plane / rotation / table
     constexpr bool combined = (MODE == kSharedLut);
     const int col_a = PAIR ? slab * (kSlab / 2) + 16 * lane : slab * kSlab + (combined ? 16 * lane : 32 * lane);
     const int col_b = PAIR ? col_a : (combined ? col_a + 1024 : col_a + 16);
@@ -124,7 +134,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     const uint32_t laneoff = (uint32_t)lane << 2;
     const int out = a.L.out_features;
     const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
-    constexpr bool use_res = (MODE != kPrimaryOnly);
+    constexpr bool use_res = (MODE == kSharedLut);          // second 16-byte load per row
 
     // Contiguous row range of this stream.
     const long long gs = (long long)blockIdx.x * a.S + stream;
@@ -137,7 +147,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     // The weight plane is read through a buffer descriptor based at the first row of the stream
     // (offsets inside a stream's rows stay far below 2 GB; the host checks).  Idle runs re-read a
     // valid address; their rotated activations are 0.
-    const uint8_t* pp = combined ? a.L.packed_combined : a.L.packed_primary;
+    const uint8_t* pp = combined ? a.L.packed_combined : (plane ? a.L.packed_residual : a.L.packed_primary);
     const uint32_t off_p = combined ? (uint32_t)(act_a ? col_a : 0) : (uint32_t)(act_a ? (col_a >> 1) : 0);
     const uint32_t off_q = (uint32_t)(act_b ? col_b : 0);          // combined plane only (PAIR: same columns, next row)
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
@@ -172,7 +182,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
 
     // Prologue.  Everything that has to come from memory is requested up front, the small things
     // first (table values, activation tiles), then the first weight group.
-    constexpr int kEntries = (MODE == kSharedLut) ? 256 : 16;
+    constexpr int kEntries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
     constexpr int kPre = 8;                    // 4096 table slots from 512 threads up
     float tv[kPre];
 #pragma unroll
@@ -204,9 +214,15 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     }
 
     float xt[NX];       // rotated activations, kept in registers for the whole kernel
+    float* const image = reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes);
     rotate_image<combined, TILES, PAIR, NX>(raw, a.x_dtype, a.L.in_features, a.img_cols, a.L.seed_primary, a.L.block_size,
-                                  reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes), wave, nwaves, lane,
-                                  slab, act_a, act_b, xt);
+                                            image, wave, nwaves, lane, slab, act_a, act_b, plane == 0, xt);
+    if constexpr (MODE == kDual) {
+        __syncthreads();                                      // everyone has read the first rotation
+        rotate_image<combined, TILES, PAIR, NX>(raw, a.x_dtype, a.L.in_features, a.img_cols, a.L.seed_residual,
+                                                a.L.block_size, image, wave, nwaves, lane, slab, act_a, act_b,
+                                                plane == 1, xt);
+    }
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
     __syncthreads();                                          // tables visible to every wave
@@ -214,7 +230,8 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     // One row (or with PAIR the same columns of two rows: p -> sum, q -> sum2).
     auto decode_row = [&](const uint4& p, const uint4& q, float& sum, float& sum2) {
         float val[kChunk];
-        lookup32<MODE == kSharedLut, 0>(p, q, smem, laneoff, val);
+        // (dual rotation: the residual table follows the primary one, 16 entries of 256 bytes each)
+        lookup32<MODE == kSharedLut, 0>(p, q, smem + plane * kTab16Bytes, laneoff, val);
         if constexpr (PAIR) {
             float s0 = 0.0f, s1 = 0.0f, t0 = 0.0f, t1 = 0.0f;
 #pragma unroll
@@ -272,7 +289,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
             float* buf_base = partial + (it & 1) * (16 * 16);
             if (lane < V) buf_base[wave * V + lane] = total;
             __syncthreads();
-            store = owner && slab == 0;
+            store = owner && unit == 0;
             if (store) {
                 t = 0.0f;
                 for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * V + lane];
@@ -330,10 +347,12 @@ bool wants_pairs(const LayerView& L) {
 template <int MODE, bool PAIR>
 hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     const int out = a.L.out_features;
+    const int slabs = a.W;
     if (PAIR) a.W = a.L.in_features / (kSlab / 2);           // halves per row
+    if (MODE == kDual) a.W = 2 * slabs;                      // (slab, plane) pairs per row
     a.S = 16 / a.W;                                          // row streams sharing the CU
     const int threads = a.W * a.S * kWave;
-    const int padded = (a.L.in_features + kSlab - 1) / kSlab * kSlab;
+    const int padded = slabs * kSlab;
     a.img_cols = padded < kMaxImageCols ? padded : kMaxImageCols;
 
     int grid = (out + a.S - 1) / a.S;
@@ -355,18 +374,20 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
 
 }  // namespace
 
-// One batch row, blocks of at most 512 columns, shared-rotation or primary-only layers whose
-// per-stream share of the plane stays below 2 GB; rows of 1 to 8 slabs, or (shared rotation) of an
-// odd number, 3 to 15, of 1024-column halves.
+// One batch row, blocks of at most 512 columns, per-stream share of the plane below 2 GB.
+// Shared rotation and primary only: rows of 1 to 8 slabs, or (shared rotation) of an odd number,
+// 3 to 15, of 1024-column halves.  Dual rotation: rows of 1 to 4 slabs.
 bool gemv_wide_supported(const LayerView& L, int num_cus) {
-    if (L.mode != kSharedLut && L.mode != kPrimaryOnly) return false;
+    if (L.mode != kSharedLut && L.mode != kPrimaryOnly && L.mode != kDual) return false;
     if (L.block_size > (uint32_t)kTile) return false;
-    int W = (L.in_features / kChunk + kWave - 1) / kWave;
+    const int slabs = (L.in_features / kChunk + kWave - 1) / kWave;
+    int W = slabs;
     if (wants_pairs(L)) W = L.in_features / (kSlab / 2);
-    else if (W < 1 || W > 8) return false;
+    else if (L.mode == kDual) { if (slabs > 4) return false; W = 2 * slabs; }   // two waves per slab
+    else if (slabs < 1 || slabs > 8) return false;
     const int S = 16 / W;
     const int ntiles = (L.in_features + kTile - 1) / kTile;
-    if (ntiles > 2 * W * S) return false;
+    if (ntiles > (L.mode == kDual ? 1 : 2) * W * S) return false;
     const size_t row_bytes = L.mode == kSharedLut ? (size_t)L.in_features : (size_t)L.in_features / 2;
     const long long streams = (long long)(num_cus > 0 ? num_cus : 1) * S;
     const long long max_rows = (L.out_features + streams - 1) / streams + 4;
@@ -380,6 +401,7 @@ hipError_t launch_gemv_wide(const GemvArgs& base, int num_cus, hipStream_t strea
     if (a.L.mode == kSharedLut)
         return wants_pairs(a.L) ? launch_wide_mode<kSharedLut, true>(a, num_cus, stream)
                                 : launch_wide_mode<kSharedLut, false>(a, num_cus, stream);
+    if (a.L.mode == kDual) return launch_wide_mode<kDual, false>(a, num_cus, stream);
     return launch_wide_mode<kPrimaryOnly, false>(a, num_cus, stream);
 }
 
