@@ -376,18 +376,18 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
 
 // One batch row, blocks of at most 512 columns, per-stream share of the plane below 2 GB.
 // Shared rotation and primary only: rows of 1 to 8 slabs, or (shared rotation) of an odd number,
-// 3 to 15, of 1024-column halves.  Dual rotation: rows of 1 to 4 slabs.
+// 3 to 15, of 1024-column halves.  Dual rotation: rows of 1 to 8 slabs.
 bool gemv_wide_supported(const LayerView& L, int num_cus) {
     if (L.mode != kSharedLut && L.mode != kPrimaryOnly && L.mode != kDual) return false;
     if (L.block_size > (uint32_t)kTile) return false;
     const int slabs = (L.in_features / kChunk + kWave - 1) / kWave;
     int W = slabs;
     if (wants_pairs(L)) W = L.in_features / (kSlab / 2);
-    else if (L.mode == kDual) { if (slabs > 4) return false; W = 2 * slabs; }   // two waves per slab
+    else if (L.mode == kDual) { if (slabs > 8) return false; W = 2 * slabs; }   // two waves per slab
     else if (slabs < 1 || slabs > 8) return false;
     const int S = 16 / W;
     const int ntiles = (L.in_features + kTile - 1) / kTile;
-    if (ntiles > (L.mode == kDual ? 1 : 2) * W * S) return false;
+    if (ntiles > 2 * W * S) return false;
     const size_t row_bytes = L.mode == kSharedLut ? (size_t)L.in_features : (size_t)L.in_features / 2;
     const long long streams = (long long)(num_cus > 0 ? num_cus : 1) * S;
     const long long max_rows = (L.out_features + streams - 1) / streams + 4;
