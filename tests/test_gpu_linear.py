@@ -211,13 +211,15 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
 
 
 # ------------------------------------------------------------------ small batches on the matrix cores
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("out,inf,bs,batch", [(64, 512, 512, 2), (300, 1024, 256, 5), (513, 2048, 512, 15),
                                               (1000, 5120, 512, 8), (16, 512, 64, 3), (47, 1536, 128, 9)])
-def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, out, inf, bs, batch):
-    """2..15 rows of 16-bit activations on a shared-rotation layer whose width is a multiple of 512
-    take the small-batch MFMA kernel (bf16 weights and rotated activations, fp32 accumulation over
-    512-column chunks): 5e-3 relative L2, ragged row counts, every row equal to its batch-1 result."""
-    qw, cbp, cbr = _make(oracle, out, inf, bs, "shared")
+def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, inf, bs, batch):
+    """2..15 rows of 16-bit activations on a layer whose width is a multiple of 512 take the
+    small-batch MFMA kernels (bf16 weights and rotated activations, fp32 accumulation over
+    512-column chunks; for dual rotation one pass per plane, each with its own rotation):
+    5e-3 relative L2, ragged row counts, every row equal to its batch-1 result."""
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
     x32 = np.random.default_rng(100 + batch).standard_normal((batch, inf)).astype(np.float32)
     xbits = oracle.f32_to_bf16_bits(x32)
     want = oracle.linear_forward(qw, cbp, cbr, bs, oracle.bf16_bits_to_f32(xbits))

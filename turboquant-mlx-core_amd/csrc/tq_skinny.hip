@@ -183,6 +183,133 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     }
 }
 
+// Nibble planes (dual rotation, primary only): the same scheme on a plane of two weights per
+// byte with a 16-entry table.  A work unit is (512-column chunk, plane): units of the primary plane
+// use the primary rotation and table, units of the residual plane the residual ones, and the
+// reduction kernel adds all units, which is the sum of the two passes.  Blocks of at most 512
+// columns only (the workgroup rotates its chunk itself).
+struct SkinnyNibbleArgs {
+    const void* x;             // activations [batch, K], f16 or bf16
+    int x_dtype;
+    uint32_t seed[2], block_size;
+    const uint8_t* plane[2];   // [N, K/2] each; plane[1] unused for primary-only layers
+    const float* tables;       // 16 primary centroids, then 16 residual ones
+    float* partial;            // [units][16][N] fp32
+    int batch, N, K;
+    int units;                 // (K / 512) * planes
+    int planes;                // 1 or 2
+    int groups;                // ceil(N / 16)
+    int wgs_per_unit;
+};
+
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
+    __shared__ __align__(16) char smem[16 * 1024];         // 16 x 512 bf16 activations, then the 4 KB table
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t laneoff = (uint32_t)lane << 2;
+
+    const int unit = blockIdx.x % a.units;
+    const int wg_in_unit = blockIdx.x / a.units;
+    const int chunk = unit / a.planes, pl = unit % a.planes;
+    const int m = lane & 15, g = lane >> 4;
+
+    const float tval = a.tables[16 * pl + (tid >> 4 & 15)];        // threads 0..255 fill the 256 table slots
+
+    // Rotate batch rows w and w + 8 of the chunk with this plane's seed -> bf16 [16][512] in LDS.
+    constexpr int kPitch = kSkChunk * 2;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int b = wave + 8 * t;
+        const int col = chunk * kSkChunk + lane * 8;
+        uint4 packed = make_uint4(0, 0, 0, 0);
+        if (b < a.batch) {                                  // wave-uniform
+            TileRaw raw;
+            raw.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) + (size_t)b * a.K + col);
+            raw.b = make_uint4(0, 0, 0, 0);
+            float v[8];
+            rotate_tile(raw, a.x_dtype, col, true, a.seed[pl], a.block_size, lane, v);
+            packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+            packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+            packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
+            packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
+        }
+        *reinterpret_cast<uint4*>(smem + b * kPitch + lane * 16) = packed;
+    }
+    __syncthreads();
+    // A operands.  Matrix step s = 4 q + d multiplies columns 128 q + 32 g + 8 d + [0, 8) of the chunk:
+    // the 8 nibbles of dword d of the lane's 16-byte piece q (piece q of lane group g starts at byte
+    // 64 q + 16 g of the row's 256 bytes).
+    sk_bf16x8 afrag[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s)
+        afrag[s] = *reinterpret_cast<const sk_bf16x8*>(smem + m * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
+    __syncthreads();                                        // everyone has its A operands: the region is free
+    if (tid < 256) {                                        // 16 entries x 16 slots of 16 bytes, values rounded to bf16
+        const uint32_t v = (uint32_t)float_to_bf16_bits(tval) << 16;
+        reinterpret_cast<uint4*>(smem)[tid] = make_uint4(v, v, v, v);
+    }
+    __syncthreads();
+
+    const int workers = a.wgs_per_unit * (kSkThreads / 64);
+    const int me = wg_in_unit * (kSkThreads / 64) + wave;
+    const int g_begin = (int)((long long)me * a.groups / workers);
+    const int g_end = (int)((long long)(me + 1) * a.groups / workers);
+
+    const uint8_t* plane = a.plane[pl];
+    const size_t row_bytes = (size_t)a.K >> 1;
+    const size_t byte0 = (size_t)chunk * (kSkChunk / 2) + 16 * g;
+    auto row_ptr = [&](int grp) {
+        int row = grp * 16 + m;
+        if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
+        return plane + (size_t)row * row_bytes + byte0;
+    };
+    // One dword = 8 weights of 8 consecutive columns (low nibble first) -> one B operand.
+    auto operand = [&](uint32_t w) {
+        const uint32_t ce = w & 0x0F0F0F0Fu, co = (w >> 4) & 0x0F0F0F0Fu;
+        uint32_t e[4], o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            e[j] = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(ce, laneoff, j));
+            o[j] = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(co, laneoff, j));
+        }
+        // entries are fp32 patterns with the value in the upper half: {even.hi, odd.hi} per column pair
+        const sk_u32x4 r = {__builtin_amdgcn_perm(o[0], e[0], 0x07060302u), __builtin_amdgcn_perm(o[1], e[1], 0x07060302u),
+                            __builtin_amdgcn_perm(o[2], e[2], 0x07060302u), __builtin_amdgcn_perm(o[3], e[3], 0x07060302u)};
+        return __builtin_bit_cast(sk_bf16x8, r);
+    };
+
+    sk_u32x4 raw[4];
+    if (g_begin < g_end) {
+        const uint8_t* p = row_ptr(g_begin);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+    }
+    for (int grp = g_begin; grp < g_end; ++grp) {
+        const bool more = grp + 1 < g_end;
+        const uint8_t* pn = row_ptr(more ? grp + 1 : grp);
+        sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const sk_u32x4 w = raw[q];
+            if (more) raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 0], operand(w.x), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 1], operand(w.y), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 2], operand(w.z), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 3], operand(w.w), acc, 0, 0, 0);
+        }
+        const int n = grp * 16 + m;
+        if (n < a.N) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int b = 4 * g + r;
+                if (b < a.batch) a.partial[((size_t)unit * 16 + b) * a.N + n] = acc[r];
+            }
+        }
+    }
+}
+
 // y[b, n] = norm[n] * out_scale * sum over chunks of partial[c][b][n]
 __global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __restrict__ partial,
                                                                const float* __restrict__ norms, void* __restrict__ y,
@@ -206,18 +333,43 @@ __global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __re
     }
 }
 
+static bool skinny_nibble(const LayerView& L) {
+    return (L.mode == kDual || L.mode == kPrimaryOnly) && L.block_size <= (uint32_t)kSkChunk;
+}
+
 bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
-    return L.mode == kSharedLut && L.packed_combined && x_dtype != kF32 && batch >= 2 && batch < 16 &&
-           L.in_features % kSkChunk == 0;
+    if (x_dtype == kF32 || batch < 2 || batch >= 16 || L.in_features % kSkChunk != 0) return false;
+    return (L.mode == kSharedLut && L.packed_combined) || skinny_nibble(L);
 }
 
 size_t skinny_partial_bytes(const LayerView& L) {
-    return (size_t)(L.in_features / kSkChunk) * 16 * L.out_features * sizeof(float);
+    const size_t units = (size_t)(L.in_features / kSkChunk) * (L.mode == kDual ? 2 : 1);
+    return units * 16 * L.out_features * sizeof(float);
 }
 
 // xt_workspace: as for launch_prefill (prefill_workspace_bytes); partial: skinny_partial_bytes.
 hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                          void* xt_workspace, float* partial, int num_cus, hipStream_t stream) {
+    if (skinny_nibble(L)) {
+        SkinnyNibbleArgs n{};
+        n.x = x; n.x_dtype = x_dtype; n.seed[0] = L.seed_primary; n.seed[1] = L.seed_residual; n.block_size = L.block_size;
+        n.plane[0] = L.packed_primary; n.plane[1] = L.packed_residual;
+        n.tables = L.tables;
+        n.partial = partial;
+        n.batch = batch; n.N = L.out_features; n.K = L.in_features;
+        n.planes = L.mode == kDual ? 2 : 1;
+        n.units = L.in_features / kSkChunk * n.planes;
+        n.groups = (L.out_features + 15) / 16;
+        n.wgs_per_unit = 2 * num_cus / n.units > 0 ? 2 * num_cus / n.units : 1;
+        hipLaunchKernelGGL(tq_skinny_nibble_kernel, dim3(n.wgs_per_unit * n.units), dim3(kSkThreads), 0, stream, n);
+        hipError_t en = hipGetLastError();
+        if (en != hipSuccess) return en;
+        const size_t total_n = (size_t)batch * L.out_features;
+        const size_t blocks_n = (total_n + 255) / 256;
+        hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3((unsigned)(blocks_n > 2048 ? 2048 : blocks_n)), dim3(256), 0, stream,
+                           partial, L.norms, y, y_dtype, batch, L.out_features, n.units, L.inv_scale * L.inv_sqrt_bs);
+        return hipGetLastError();
+    }
     const bool fused = L.block_size <= (uint32_t)kSkChunk;
     hipError_t e = hipSuccess;
     if (!fused) {
