@@ -140,6 +140,9 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
         return a.plane + (size_t)row * a.K + col0;
     };
+    // Plain loads, not streaming ones: a load instruction touches 64 bytes of each of 16 rows, half
+    // a cache line, and the other half is asked for by a later instruction; with the streaming
+    // hint that half was fetched from memory again (13 % more time).
     // The 8 loads of a group live in 32 registers; as soon as one has been decoded it is replaced
     // by the same piece of the next group, so a full group of loads is always in flight.
     sk_u32x4 raw[8];
@@ -156,7 +159,7 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         const uint8_t* p = row_ptr(g_begin);
 #pragma unroll
         for (int q = 0; q < 8; ++q)
-            raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+            raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
     }
     for (int grp = g_begin; grp < g_end; ++grp) {
         const bool more = grp + 1 < g_end;
@@ -165,7 +168,7 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             const sk_u32x4 w = raw[q];
-            if (more) raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
+            if (more) raw[q] = (*reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
             const uint2 p0 = lookup2(w.x), p1 = lookup2(w.y), p2 = lookup2(w.z), p3 = lookup2(w.w);
             const sk_u32x4 b0 = {p0.x, p0.y, p1.x, p1.y}, b1 = {p2.x, p2.y, p3.x, p3.y};
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * q], __builtin_bit_cast(sk_bf16x8, b0), acc, 0, 0, 0);
@@ -284,7 +287,7 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         const uint8_t* p = row_ptr(g_begin);
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+            raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
     }
     for (int grp = g_begin; grp < g_end; ++grp) {
         const bool more = grp + 1 < g_end;
@@ -293,7 +296,7 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const sk_u32x4 w = raw[q];
-            if (more) raw[q] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
+            if (more) raw[q] = (*reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 0], operand(w.x), acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 1], operand(w.y), acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 2], operand(w.z), acc, 0, 0, 0);
