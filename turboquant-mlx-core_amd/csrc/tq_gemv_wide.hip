@@ -25,6 +25,12 @@
 // (past it they re-read its last row), and everything loaded is marked as consumed on every path,
 // so the compiler knows exactly how many loads are in flight and waits for no more than the row
 // it is about to decode; the prefetched group stays in flight.
+// The start of the kernel is kept short, because with 16 waves per CU everything a wave does there
+// is done 16 times on shared units: no integer division on the device (the waves of a CU share one
+// scalar unit; the host passes quotients), table values through scalar loads (every vector memory
+// instruction holds the CU's address unit for 16 cycles), one barrier, and the second stage of the
+// register ring requested behind that barrier.  Rows of one slab are handed to the waves of a CU
+// group by group from a counter in LDS.
 #include "tq_device.h"
 #include "tq_gemv_common.h"
 
@@ -61,48 +67,42 @@ __device__ __forceinline__ TileRaw load_tile_fixed(const void* x, int x_dtype, i
 }
 
 // Wave w rotates tiles w, w + nwaves, ... (8 values per lane and tile) and writes them into the
-// image: value k of lane l of a slab sits at float index k*64 + l of the slab's 8 KB.  The image
-// holds img_cols columns; wider rows go through it in rounds.  Afterwards every wave picks up the
-// 32 values of the columns it owns.  raw[t] holds the activations of tile wave + t * nwaves (any
+// image of the whole row (the host checks that it fits): value k of lane l of a slab sits at float
+// index k*64 + l of the slab's 8 KB.  raw[t] holds the activations of tile wave + t * nwaves (any
 // valid address for tiles past the row).
+template <bool SPLIT, int TILES>
+__device__ __forceinline__ void rotate_to_image(const TileRaw (&raw)[TILES], int x_dtype, int in_features,
+                                                uint32_t seed, uint32_t bs, float* image, int wave, int nwaves,
+                                                int lane) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        const int tile0 = (wave + t * nwaves) * kTile;
+        if (tile0 < in_features) {                                // wave-uniform
+            float v[8];
+            rotate_tile(raw[t], x_dtype, tile0 + lane * 8, tile0 + lane * 8 < in_features, seed, bs, lane, v);
+            const int col = tile0 + lane * 8;
+            float* dst = image + (col & ~(kSlab - 1)) + stage_index<SPLIT>(col & (kSlab - 1));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dst[j * kWave] = v[j];      // 8 columns stay inside one 16-run
+        }
+    }
+}
+
+// After the barrier that follows: a wave picks up the 32 values of the columns it owns.
 // unit: the slab of the wave, or with PAIR its 1024-column half (xt then holds 16 values).
-// take: whether this wave picks up its values from this rotation (dual rotation runs two).
-template <bool SPLIT, int TILES, bool PAIR, int NX>
-__device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_dtype, int in_features,
-                                             int img_cols, uint32_t seed, uint32_t bs, float* image, int wave,
-                                             int nwaves, int lane, int unit, bool act_a, bool act_b, bool take,
-                                             float (&xt)[NX]) {
-    const int rounds = (in_features + img_cols - 1) / img_cols;
-    for (int p = 0; p < rounds; ++p) {
-        if (p > 0) __syncthreads();                              // previous image has been read
+template <bool PAIR, int NX>
+__device__ __forceinline__ void take_from_image(const float* image, int lane, int unit, bool act_a, bool act_b,
+                                                float (&xt)[NX]) {
+    if constexpr (PAIR) {
+        const int first = unit * (kSlab / 2);                     // first column of the half
+        const float* src = image + (first & ~(kSlab - 1)) + ((unit & 1) << 4) * kWave + lane;
 #pragma unroll
-        for (int t = 0; t < TILES; ++t) {
-            const int tile0 = (wave + t * nwaves) * kTile;
-            if (tile0 < in_features && tile0 / img_cols == p) {   // wave-uniform
-                float v[8];
-                rotate_tile(raw[t], x_dtype, tile0 + lane * 8, tile0 + lane * 8 < in_features, seed, bs, lane, v);
-                const int col = tile0 % img_cols + lane * 8;      // column inside the image
-                float* dst = image + (col & ~(kSlab - 1)) + stage_index<SPLIT>(col & (kSlab - 1));
+        for (int k = 0; k < NX; ++k) xt[k] = src[k * kWave];
+    } else {
+        const float* src = image + unit * kSlab + lane;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) dst[j * kWave] = v[j];      // 8 columns stay inside one 16-run
-            }
-        }
-        __syncthreads();
-        if constexpr (PAIR) {
-            const int first = unit * (kSlab / 2);                 // first column of the half
-            if (take && first / img_cols == p) {
-                const float* src = image + ((first % img_cols) & ~(kSlab - 1)) + ((unit & 1) << 4) * kWave + lane;
-#pragma unroll
-                for (int k = 0; k < NX; ++k) xt[k] = src[k * kWave];
-            }
-        } else {
-            if (take && (unit * kSlab) / img_cols == p) {
-                const float* src = image + (unit * kSlab) % img_cols + lane;
-#pragma unroll
-                for (int k = 0; k < NX; ++k)
-                    xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
-            }
-        }
+        for (int k = 0; k < NX; ++k)
+            xt[k] = ((k < 16) ? act_a : act_b) ? src[k * kWave] : 0.0f;   // idle runs contribute 0
     }
 }
 
@@ -110,9 +110,15 @@ __device__ __forceinline__ void rotate_image(const TileRaw (&raw)[TILES], int x_
 // 2 s is slab s of the primary plane, unit 2 s + 1 slab s of the residual plane).  R rows per group, TILES activation tiles
 // per wave (the host checks that TILES * waves covers the row and that blocks are at most 512 wide).
 // PAIR (combined plane only): a.W counts 1024-column halves; a group is R row pairs.
-template <int MODE, int R, int TILES, bool PAIR>
+// DYN (rows of one slab, a.W == 1): the waves of a workgroup do not own fixed row ranges.  The
+// workgroup owns a contiguous range, cut into row groups, and every wave takes its next group from a
+// counter in LDS.  Waves of one CU progress at different rates (the spread between the first and the
+// last wave of a CU to finish equal shares was a fifth of the run time); with the counter they all
+// finish within one row group of each other.
+template <int MODE, int R, int TILES, bool PAIR, bool DYN>
 __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     static_assert(!PAIR || MODE == kSharedLut, "row pairs need the one-byte-per-weight plane");
+    static_assert(!DYN || (!PAIR && MODE != kDual), "the group counter serves one-wave row streams");
     constexpr int NS = 2;                           // register ring: one group decoded, one in flight
     constexpr int V = PAIR ? 2 * R : R;             // rows, and sums, per row group
     constexpr int NX = PAIR ? 16 : kChunk;          // rotated activations per lane
@@ -123,8 +129,10 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = blockDim.x >> 6;
-    const int unit = wave % a.W;
-    const int stream = wave / a.W;
+    // (divisions cost a few hundred scalar instructions per wave, and all waves of a CU share one
+    // scalar unit: the host supplies the quotients)
+    const int stream = (wave * a.w_inv) >> 8;               // wave / a.W
+    const int unit = wave - stream * a.W;
     const int slab = (MODE == kDual) ? unit >> 1 : unit;
     const int plane = (MODE == kDual) ? unit & 1 : 0;       // 0: primary plane / rotation / table
     constexpr bool combined = (MODE == kSharedLut);
@@ -136,11 +144,11 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
     constexpr bool use_res = (MODE == kSharedLut);          // second 16-byte load per row
 
-    // Contiguous row range of this stream.
-    const long long gs = (long long)blockIdx.x * a.S + stream;
-    const long long ts = (long long)gridDim.x * a.S;
-    const int r_begin = (int)(gs * out / ts);
-    const int r_end = (int)((gs + 1) * out / ts);
+    // Contiguous row range of this stream (DYN: of the workgroup): rows_q rows, one more for the
+    // first rows_rem ranges.
+    const int gs = DYN ? (int)blockIdx.x : (int)blockIdx.x * a.S + stream;
+    const int r_begin = gs * a.rows_q + (gs < a.rows_rem ? gs : a.rows_rem);
+    const int r_end = r_begin + a.rows_q + (gs < a.rows_rem ? 1 : 0);
     const int r_base = r_begin < out ? r_begin : out - 1;
     const int r_last = r_end > r_begin ? r_end - 1 : r_base;
 
@@ -180,52 +188,64 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
         }
     };
 
-    // Prologue.  Everything that has to come from memory is requested up front, the small things
-    // first (table values, activation tiles), then the first weight group.
+    // Prologue.  Everything that has to come from memory is requested up front: the activation
+    // tiles, then the weights.  (Every vector memory instruction of a wave occupies the CU's
+    // address unit for 16 cycles, and 16 waves share it: the table values, which are the same for
+    // all lanes, come through scalar loads instead.)
     constexpr int kEntries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
-    constexpr int kPre = 8;                    // 4096 table slots from 512 threads up
-    float tv[kPre];
+    // Wave w writes table entries 16 w .. 16 w + 15 (then 16 (w + nwaves) ..); the first 16 values
+    // are requested here.
+    typedef const __attribute__((address_space(4))) float cfloat;     // uniform address: scalar load
+    cfloat* const tab = (cfloat*)a.L.tables;
+    const int e0 = wave * 16 < kEntries ? wave * 16 : 0;
+    float tv[16];
 #pragma unroll
-    for (int k = 0; k < kPre; ++k) {
-        const int i = tid + k * (int)blockDim.x;
-        tv[k] = a.L.tables[(i < kEntries * 16 ? i : 0) >> 4];
-    }
+    for (int e = 0; e < 16; ++e) tv[e] = tab[e0 + e];
     TileRaw raw[TILES];
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {         // tiles past the row re-read its start and are not used
         const int col = (wave + t * nwaves) * kTile + lane * 8;
         raw[t] = load_tile_fixed(a.x, a.x_dtype, col < a.L.in_features ? col : 0);
     }
-    fetch(0, r_begin);
+    // The weight requests stay behind the small ones: loads complete in order, and the rotation
+    // must not wait for weights.
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(0, DYN ? r_begin + wave * V : r_begin);
 
     // Decode tables -> LDS, one private column per lane.
+    int* const next_group = reinterpret_cast<int*>(partial);    // DYN: first group nobody has taken yet
+    if (DYN && tid == 0) *next_group = 2 * nwaves;              // (groups w and w + nwaves are wave w's first two)
     {
-        float4* dst = reinterpret_cast<float4*>(smem);
+        // Lane l stores each entry's value into its own column, 4 l bytes into the entry's 256.
+        float* const dst = reinterpret_cast<float*>(smem) + lane;
+        if (wave * 16 < kEntries) {
 #pragma unroll
-        for (int k = 0; k < kPre; ++k) {
-            const int i = tid + k * (int)blockDim.x;
-            consumed(tv[k]);
-            if (i < kEntries * 16) dst[i] = make_float4(tv[k], tv[k], tv[k], tv[k]);
+            for (int e = 0; e < 16; ++e) dst[(e0 + e) * kWave] = tv[e];
         }
-        for (int i = tid + kPre * (int)blockDim.x; i < kEntries * 16; i += blockDim.x) {
-            const float v = a.L.tables[i >> 4];
-            dst[i] = make_float4(v, v, v, v);
+        for (int c = wave + nwaves; c * 16 < kEntries; c += nwaves) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) dst[(c * 16 + e) * kWave] = tab[c * 16 + e];
         }
     }
 
     float xt[NX];       // rotated activations, kept in registers for the whole kernel
     float* const image = reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes);
-    rotate_image<combined, TILES, PAIR, NX>(raw, a.x_dtype, a.L.in_features, a.img_cols, a.L.seed_primary, a.L.block_size,
-                                            image, wave, nwaves, lane, slab, act_a, act_b, plane == 0, xt);
+    rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_primary, a.L.block_size, image, wave,
+                                     nwaves, lane);
+    __syncthreads();                  // image and tables (and the group counter) visible to every wave
+    // The second stage of the ring is requested behind the barrier: a wave whose requests queue up
+    // in the memory pipeline would otherwise keep the whole workgroup waiting there.
+    fetch(1, DYN ? r_begin + (wave + nwaves) * V : r_begin + V);
+    if (plane == 0) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xt);
     if constexpr (MODE == kDual) {
         __syncthreads();                                      // everyone has read the first rotation
-        rotate_image<combined, TILES, PAIR, NX>(raw, a.x_dtype, a.L.in_features, a.img_cols, a.L.seed_residual,
-                                                a.L.block_size, image, wave, nwaves, lane, slab, act_a, act_b,
-                                                plane == 1, xt);
+        rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_residual, a.L.block_size, image,
+                                         wave, nwaves, lane);
+        __syncthreads();
+        if (plane == 1) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xt);
     }
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
-    __syncthreads();                                          // tables visible to every wave
 
     // One row (or with PAIR the same columns of two rows: p -> sum, q -> sum2).
     auto decode_row = [&](const uint4& p, const uint4& q, float& sum, float& sum2) {
@@ -285,7 +305,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
 
         float t = total;
         bool store = owner;
-        if (a.W > 1) {                                       // cross-wave sum of the row's slabs
+        if (!DYN && a.W > 1) {                               // cross-wave sum of the row's slabs
             float* buf_base = partial + (it & 1) * (16 * 16);
             if (lane < V) buf_base[wave * V + lane] = total;
             __syncthreads();
@@ -302,27 +322,48 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
         }
     };
 
-    // Main loop over the register ring, unrolled twice so the stages are static: group it+1 is
-    // requested while group it is decoded.  The trip count is uniform over the grid.  Whole rounds
-    // of two stages run without a condition inside; an odd last group is a tail.
+    // Main loop over the register ring, unrolled twice so the stages are static: a stage is
+    // requested again as soon as it has been decoded, so two groups are in flight or being decoded
+    // at any time.  The trip count is uniform over the grid.  Whole rounds of two stages run
+    // without a condition inside; an odd last group is a tail.
+    if constexpr (DYN) {
+        const int groups = (r_end - r_begin + V - 1) / V;
+        int g0 = wave, g1 = wave + nwaves;                  // groups held by the two ring stages
+        // Takes the group for the stage being emptied.  Every lane adds to a slot of its own, lane
+        // 0's is the counter (no branch around the LDS operation); the answer is picked up after the
+        // decode, when it has long arrived.  Groups are handed out in increasing order.
+        int* const slot = next_group + lane;
+        auto take = [&]() { return __hip_atomic_fetch_add(slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); };
+        auto taken = [&](int t) { asm volatile("" : "+v"(t)); return __builtin_amdgcn_readfirstlane(t); };
+        int t = take();
+        while (g0 < groups) {
+            consume(0, r_begin + g0 * V, 0);
+            g0 = taken(t);
+            t = take();
+            fetch(0, r_begin + g0 * V);
+            if (g1 >= groups) break;
+            consume(1, r_begin + g1 * V, 0);
+            g1 = taken(t);
+            t = take();
+            fetch(1, r_begin + g1 * V);
+        }
+        return;
+    }
     int it0 = 0;
     for (; it0 + NS <= a.iters; it0 += NS) {
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
-            fetch((u + 1) % NS, r_begin + (it0 + u + 1) * V);
             consume(u, r_begin + (it0 + u) * V, it0 + u);
+            fetch(u, r_begin + (it0 + u + NS) * V);
         }
     }
-    if (it0 < a.iters) {
-        fetch(1, r_begin + (it0 + 1) * V);
-        consume(0, r_begin + it0 * V, it0);
-    }
+    if (it0 < a.iters) consume(0, r_begin + it0 * V, it0);
 }
 
-template <int MODE, int R, int TILES, bool PAIR>
+template <int MODE, int R, int TILES, bool PAIR, bool DYN = false>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
     const size_t lds = (size_t)kRegionBytes + kPartialBytes + (size_t)a.img_cols * sizeof(float);
-    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR>;
+    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN>;
     // More LDS than the default limit has to be asked for, once per kernel and device.
     static bool asked[64] = {};
     int dev = 0;
@@ -353,19 +394,31 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     a.S = 16 / a.W;                                          // row streams sharing the CU
     const int threads = a.W * a.S * kWave;
     const int padded = slabs * kSlab;
-    a.img_cols = padded < kMaxImageCols ? padded : kMaxImageCols;
+    if (padded > kMaxImageCols) return hipErrorInvalidValue;   // gemv_wide_supported() rules this out
+    a.img_cols = padded;
 
     int grid = (out + a.S - 1) / a.S;
     if (grid > num_cus) grid = num_cus;
     if (grid < 1) grid = 1;
-    const long long ts = (long long)grid * a.S;
-    const int max_rows = (int)((out + ts - 1) / ts);        // longest row range of any stream
+    const bool shared_range = !PAIR && MODE != kDual && a.W == 1;   // one range per workgroup (group counter)
+    const int ts = shared_range ? grid : grid * a.S;        // row ranges
+    a.rows_q = out / ts;
+    a.rows_rem = out % ts;
+    a.w_inv = (256 + a.W - 1) / a.W;                        // (w * w_inv) >> 8 == w / W for w < 16, W <= 16
+    const int max_rows = (int)(((long long)out + grid * a.S - 1) / (grid * a.S));   // longest share of a stream
     const int per_r = PAIR ? 2 : 1;                         // rows per unit of R
     const int R = max_rows >= 2 * per_r ? 2 : 1;
     a.iters = (max_rows + R * per_r - 1) / (R * per_r);
 
     const int ntiles = (a.L.in_features + kTile - 1) / kTile;
     const bool two = ntiles > threads / kWave;              // at most two tiles per wave: checked by the caller
+    if constexpr (!PAIR && MODE != kDual) {
+        if (a.W == 1) {                                     // one slab: 16 one-wave streams fed from a group counter
+            const int rows_wg = (out + grid - 1) / grid;
+            if (rows_wg >= 4 * a.S) return launch_wide_one<MODE, 2, 1, false, true>(a, grid, threads, stream);
+            return launch_wide_one<MODE, 1, 1, false, true>(a, grid, threads, stream);
+        }
+    }
     if (R == 2) return two ? launch_wide_one<MODE, 2, 2, PAIR>(a, grid, threads, stream)
                            : launch_wide_one<MODE, 2, 1, PAIR>(a, grid, threads, stream);
     return two ? launch_wide_one<MODE, 1, 2, PAIR>(a, grid, threads, stream)
@@ -389,7 +442,8 @@ bool gemv_wide_supported(const LayerView& L, int num_cus) {
     const int ntiles = (L.in_features + kTile - 1) / kTile;
     if (ntiles > 2 * W * S) return false;
     const size_t row_bytes = L.mode == kSharedLut ? (size_t)L.in_features : (size_t)L.in_features / 2;
-    const long long streams = (long long)(num_cus > 0 ? num_cus : 1) * S;
+    const bool shared_range = W == 1 && L.mode != kDual;    // one row range per workgroup, shared by its waves
+    const long long streams = (long long)(num_cus > 0 ? num_cus : 1) * (shared_range ? 1 : S);
     const long long max_rows = (L.out_features + streams - 1) / streams + 4;
     return (unsigned long long)max_rows * row_bytes < (1ull << 31);
 }
