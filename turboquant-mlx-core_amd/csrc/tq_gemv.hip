@@ -134,8 +134,10 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = blockDim.x >> 6;
-    const int slab = wave % a.W;
-    const int stream = wave / a.W;
+    // (no integer division on the device: the waves of a CU share one scalar unit and a division
+    // is a few hundred instructions; the host passes the quotients)
+    const int stream = (wave * a.w_inv) >> 8;               // wave / a.W
+    const int slab = wave - stream * a.W;
     // Shared-rotation mode streams the combined plane (one byte per weight); the other modes
     // stream 16 B from each nibble plane.  See stage_index for the column ownership.
     constexpr bool combined = (MODE == kSharedLut);
@@ -147,11 +149,10 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
     constexpr bool use_res = (MODE != kPrimaryOnly);
 
-    // Contiguous row range of this stream.
-    const long long gs = (long long)blockIdx.x * a.S + stream;
-    const long long ts = (long long)gridDim.x * a.S;
-    const int r_begin = (int)(gs * out / ts);
-    const int r_end = (int)((gs + 1) * out / ts);
+    // Contiguous row range of this stream: rows_q rows, one more for the first rows_rem streams.
+    const int gs = (int)blockIdx.x * a.S + stream;
+    const int r_begin = gs * a.rows_q + (gs < a.rows_rem ? gs : a.rows_rem);
+    const int r_end = r_begin + a.rows_q + (gs < a.rows_rem ? 1 : 0);
 
     // Idle runs re-read a valid address; their rotated activations are 0.
     // Row bases are wave-uniform (scalar); the lane adds a fixed 32-bit byte offset.
@@ -189,13 +190,10 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     // first (table values, activations), then the first NS-1 weight groups: loads complete in
     // order, so the prologue only waits for what it needs while the weights keep streaming in.
     constexpr int kEntries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
-    constexpr int kPre = 8;
-    float tv[kPre];
-#pragma unroll
-    for (int k = 0; k < kPre; ++k) {
-        const int i = tid + k * (int)blockDim.x;
-        tv[k] = a.L.tables[(i < kEntries * 16 ? i : 0) >> 4];
-    }
+    // (table values are the same for all lanes: scalar loads, which leave the CU's vector memory
+    // address unit to the weights)
+    typedef const __attribute__((address_space(4))) float cfloat;
+    cfloat* const tab = (cfloat*)a.L.tables;
     constexpr bool kEarlyX = (NB == 1 && MODE != kDual);
     const bool shared_rot = (a.S >= 4 && a.L.block_size <= (uint32_t)kTile);      // W <= 2: at most 8 tiles
     TileRaw raw[NB];
@@ -213,17 +211,13 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
 #pragma unroll
     for (int u = 0; u < NS - 1; ++u) fetch(u, r_begin + u * R);
 
-    // Decode tables -> LDS, one private column per lane.
+    // Decode tables -> LDS, one private column per lane: wave w writes entries 16 w .. 16 w + 15,
+    // then 16 (w + nwaves) .., lane l into bytes 4 l .. of each entry's 256.
     {
-        float4* dst = reinterpret_cast<float4*>(smem);
+        float* const dst = reinterpret_cast<float*>(smem) + lane;
+        for (int c = wave; c * 16 < kEntries; c += nwaves) {
 #pragma unroll
-        for (int k = 0; k < kPre; ++k) {
-            const int i = tid + k * (int)blockDim.x;
-            if (i < kEntries * 16) dst[i] = make_float4(tv[k], tv[k], tv[k], tv[k]);
-        }
-        for (int i = tid + kPre * (int)blockDim.x; i < kEntries * 16; i += blockDim.x) {
-            const float v = a.L.tables[i >> 4];
-            dst[i] = make_float4(v, v, v, v);
+            for (int e = 0; e < 16; ++e) dst[(c * 16 + e) * kWave] = tab[c * 16 + e];
         }
     }
 
@@ -352,8 +346,11 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     int grid = (out + a.S - 1) / a.S;
     if (grid > max_grid) grid = max_grid;
     if (grid < 1) grid = 1;
-    const long long ts = (long long)grid * a.S;
-    const int max_rows = (int)((out + ts - 1) / ts);        // longest row range of any stream
+    const int ts = grid * a.S;                              // row streams
+    a.rows_q = out / ts;
+    a.rows_rem = out % ts;
+    a.w_inv = (256 + a.W - 1) / a.W;                        // (w * w_inv) >> 8 == w / W for w < 16, W <= 16
+    const int max_rows = a.rows_q + (a.rows_rem ? 1 : 0);   // longest row range of any stream
     // Four rows per group only where the register budget allows it without spilling.
     int R = (max_rows >= 4 && MAXT <= 512 && NB < 4) ? 4 : (max_rows >= 2 ? 2 : 1);
     if (MODE == kDual && MAXT > 512) R = 1;
