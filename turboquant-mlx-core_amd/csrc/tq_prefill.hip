@@ -407,9 +407,8 @@ __global__ __launch_bounds__(256) void tq_rotate_bf16_kernel(const void* __restr
                                                              uint16_t* __restrict__ out, int rows, int cols,
                                                              int chunks, int slabs, uint32_t seed, uint32_t bs) {
     const int lane = threadIdx.x & 63;
-    const long long wid = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int row = (int)(wid / slabs);
-    const int slab = (int)(wid % slabs);
+    const int row = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);     // grid = row quads x slabs
+    const int slab = blockIdx.y;
     if (row >= rows) return;
     const int chunk = slab * kWave + lane;
     const bool active = chunk < chunks;
@@ -457,12 +456,11 @@ hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, i
     uint16_t* xt = static_cast<uint16_t*>(workspace);
     const int chunks = K / kChunk;
     const int slabs = (chunks + kWave - 1) / kWave;
-    const long long waves = (long long)M * slabs;
-    const unsigned rgrid = (unsigned)((waves + 3) / 4);
-    hipLaunchKernelGGL(tq_rotate_bf16_kernel, dim3(rgrid), dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
+    const dim3 rgrid((unsigned)((M + 3) / 4), (unsigned)slabs);
+    hipLaunchKernelGGL(tq_rotate_bf16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
                        L.seed_primary, L.block_size);
     if (L.mode == kDual)
-        hipLaunchKernelGGL(tq_rotate_bf16_kernel, dim3(rgrid), dim3(256), 0, stream, x, x_dtype,
+        hipLaunchKernelGGL(tq_rotate_bf16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype,
                            xt + (size_t)((M + kBM - 1) / kBM) * kBM * K, M, K, chunks, slabs, L.seed_residual,
                            L.block_size);
     return hipGetLastError();

@@ -39,6 +39,7 @@ struct SkinnyArgs {
     int chunks;                // K / 512
     int groups;                // ceil(N / 16)
     int wgs_per_chunk;
+    int groups_q, groups_rem;  // groups / workers and groups % workers (workers = waves sharing a chunk)
 };
 
 __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t laneoff, int j) {
@@ -60,8 +61,10 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t laneoff = (uint32_t)lane << 2;
 
-    const int chunk = blockIdx.x % a.chunks;
-    const int wg_in_chunk = blockIdx.x / a.chunks;
+    // (grid = chunks x workgroups per chunk; no integer division in the kernel: the waves of a CU
+    // share one scalar unit and a division is a few hundred instructions)
+    const int chunk = blockIdx.x;
+    const int wg_in_chunk = blockIdx.y;
     const int m = lane & 15, g = lane >> 4;               // A operand: batch row, k group; B operand: weight row, k group
 
     // Table values of this thread's LDS slots, requested before anything else.
@@ -129,10 +132,9 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     __syncthreads();                                       // table visible
 
     // Row groups of this wave: the groups are dealt out evenly over all waves that share the chunk.
-    const int workers = a.wgs_per_chunk * (kSkThreads / 64);
     const int me = wg_in_chunk * (kSkThreads / 64) + wave;
-    const int g_begin = (int)((long long)me * a.groups / workers);
-    const int g_end = (int)((long long)(me + 1) * a.groups / workers);
+    const int g_begin = me * a.groups_q + (me < a.groups_rem ? me : a.groups_rem);
+    const int g_end = g_begin + a.groups_q + (me < a.groups_rem ? 1 : 0);
 
     const size_t col0 = (size_t)chunk * kSkChunk + 16 * g;
     auto row_ptr = [&](int grp) {
@@ -203,6 +205,7 @@ struct SkinnyNibbleArgs {
     int planes;                // 1 or 2
     int groups;                // ceil(N / 16)
     int wgs_per_unit;
+    int groups_q, groups_rem;  // groups / workers and groups % workers (workers = waves sharing a unit)
 };
 
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
@@ -212,9 +215,10 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t laneoff = (uint32_t)lane << 2;
 
-    const int unit = blockIdx.x % a.units;
-    const int wg_in_unit = blockIdx.x / a.units;
-    const int chunk = unit / a.planes, pl = unit % a.planes;
+    // (grid = units x workgroups per unit; unit = chunk * planes + plane)
+    const int unit = blockIdx.x;
+    const int wg_in_unit = blockIdx.y;
+    const int chunk = a.planes == 2 ? unit >> 1 : unit, pl = a.planes == 2 ? unit & 1 : 0;
     const int m = lane & 15, g = lane >> 4;
 
     const float tval = a.tables[16 * pl + (tid >> 4 & 15)];        // threads 0..255 fill the 256 table slots
@@ -254,10 +258,9 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     }
     __syncthreads();
 
-    const int workers = a.wgs_per_unit * (kSkThreads / 64);
     const int me = wg_in_unit * (kSkThreads / 64) + wave;
-    const int g_begin = (int)((long long)me * a.groups / workers);
-    const int g_end = (int)((long long)(me + 1) * a.groups / workers);
+    const int g_begin = me * a.groups_q + (me < a.groups_rem ? me : a.groups_rem);
+    const int g_end = g_begin + a.groups_q + (me < a.groups_rem ? 1 : 0);
 
     const uint8_t* plane = a.plane[pl];
     const size_t row_bytes = (size_t)a.K >> 1;
@@ -317,9 +320,9 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
 __global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __restrict__ partial,
                                                                const float* __restrict__ norms, void* __restrict__ y,
                                                                int y_dtype, int batch, int N, int chunks, float out_scale) {
-    const size_t total = (size_t)batch * N;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const int b = (int)(i / N), n = (int)(i % N);
+    // grid = column blocks x batch rows (no division per element)
+    const int b = blockIdx.y;
+    for (int n = blockIdx.x * blockDim.x + threadIdx.x; n < N; n += gridDim.x * blockDim.x) {
         // four independent running sums: the loads of a thread do not wait for one another
         float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
         const float* p = partial + (size_t)b * N + n;
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __re
             s3 += p[(size_t)(c + 3) * step];
         }
         for (; c < chunks; ++c) s0 += p[(size_t)c * step];
-        store_scalar(y, y_dtype, i, ((s0 + s1) + (s2 + s3)) * (out_scale * norms[n]));
+        store_scalar(y, y_dtype, (size_t)b * N + n, ((s0 + s1) + (s2 + s3)) * (out_scale * norms[n]));
     }
 }
 
@@ -364,12 +367,14 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         n.units = L.in_features / kSkChunk * n.planes;
         n.groups = (L.out_features + 15) / 16;
         n.wgs_per_unit = 2 * num_cus / n.units > 0 ? 2 * num_cus / n.units : 1;
-        hipLaunchKernelGGL(tq_skinny_nibble_kernel, dim3(n.wgs_per_unit * n.units), dim3(kSkThreads), 0, stream, n);
+        const int workers_n = n.wgs_per_unit * (kSkThreads / 64);
+        n.groups_q = n.groups / workers_n;
+        n.groups_rem = n.groups % workers_n;
+        hipLaunchKernelGGL(tq_skinny_nibble_kernel, dim3(n.units, n.wgs_per_unit), dim3(kSkThreads), 0, stream, n);
         hipError_t en = hipGetLastError();
         if (en != hipSuccess) return en;
-        const size_t total_n = (size_t)batch * L.out_features;
-        const size_t blocks_n = (total_n + 255) / 256;
-        hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3((unsigned)(blocks_n > 2048 ? 2048 : blocks_n)), dim3(256), 0, stream,
+        const unsigned blocks_n = (unsigned)((L.out_features + 255) / 256);
+        hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks_n > 1024 ? 1024 : blocks_n, batch), dim3(256), 0, stream,
                            partial, L.norms, y, y_dtype, batch, L.out_features, n.units, L.inv_scale * L.inv_sqrt_bs);
         return hipGetLastError();
     }
@@ -389,13 +394,15 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     a.chunks = L.in_features / kSkChunk;
     a.groups = (L.out_features + 15) / 16;
     a.wgs_per_chunk = 2 * num_cus / a.chunks > 0 ? 2 * num_cus / a.chunks : 1;   // two workgroups per CU
-    if (fused) hipLaunchKernelGGL(tq_skinny_kernel<true>, dim3(a.wgs_per_chunk * a.chunks), dim3(kSkThreads), 0, stream, a);
-    else hipLaunchKernelGGL(tq_skinny_kernel<false>, dim3(a.wgs_per_chunk * a.chunks), dim3(kSkThreads), 0, stream, a);
+    const int workers = a.wgs_per_chunk * (kSkThreads / 64);
+    a.groups_q = a.groups / workers;
+    a.groups_rem = a.groups % workers;
+    if (fused) hipLaunchKernelGGL(tq_skinny_kernel<true>, dim3(a.chunks, a.wgs_per_chunk), dim3(kSkThreads), 0, stream, a);
+    else hipLaunchKernelGGL(tq_skinny_kernel<false>, dim3(a.chunks, a.wgs_per_chunk), dim3(kSkThreads), 0, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const size_t total = (size_t)batch * L.out_features;
-    const size_t blocks = (total + 255) / 256;
-    hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3((unsigned)(blocks > 2048 ? 2048 : blocks)), dim3(256), 0, stream,
+    const unsigned blocks = (unsigned)((L.out_features + 255) / 256);
+    hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks > 1024 ? 1024 : blocks, batch), dim3(256), 0, stream,
                        partial, L.norms, y, y_dtype, batch, L.out_features, a.chunks, L.inv_scale * L.inv_sqrt_bs);
     return hipGetLastError();
 }
