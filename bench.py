@@ -28,6 +28,12 @@ MEASURED_TRAFFIC_BYTES = 312822886
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
 
+# Untimed replays of a captured graph before the timed one.  The first replay uploads the graph; the
+# replay after it still runs 4-5 % slower than all later ones (power management settling under the
+# load), so the timed replay is the fourth.
+UNTIMED_REPLAYS = 3
+
+
 def algorithmic_bytes(out, inf, batch, x_bytes, y_bytes):
     # packed primary + residual (one byte per weight), norms, two codebooks, x, y
     return out * inf + 4 * out + 128 + batch * inf * x_bytes + batch * out * y_bytes
@@ -99,7 +105,8 @@ def time_graph(tq, torch, handles, x, y, xcode, batch, steps, warmup, spread=Non
         enqueue(steps, stream)
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
-        graph.replay()                     # untimed replay: graph upload
+        for _ in range(UNTIMED_REPLAYS):   # untimed: graph upload, then clocks and memory settle under load
+            graph.replay()
         stream.synchronize()
         torch.cuda.synchronize()
         start.record(stream)
@@ -131,7 +138,8 @@ def time_graph_fn(torch, enqueue_step, steps, warmup):
             enqueue_step(stream.cuda_stream)
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
-        graph.replay()
+        for _ in range(UNTIMED_REPLAYS):   # untimed: graph upload, then clocks and memory settle under load
+            graph.replay()
         stream.synchronize()
         torch.cuda.synchronize()
         start.record(stream)
@@ -215,6 +223,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "untimed_graph_replays_before_timing": UNTIMED_REPLAYS,
         "ms_per_step": us * 1e-3,
         "higher_is_better": True,
         "scaling": "weak",

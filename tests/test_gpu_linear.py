@@ -134,6 +134,33 @@ def test_forward_batch1_wide_rows(tq, oracle, mode, out, inf, bs):
     layer.close()
 
 
+@pytest.mark.parametrize("mode", ["shared", "primary_only", "dual"])
+@pytest.mark.parametrize("out,inf,bs", [(600, 27648, 512), (515, 18944, 256), (257, 17408, 512), (40, 20480, 2048)])
+def test_forward_batch1_rows_beyond_16384_columns(tq, oracle, mode, out, inf, bs):
+    """One activation row on rows of 9 to 14 slabs: the row is rotated once by a kernel of its own
+    (blocks of at most 512 columns; larger blocks are rotated inside the product kernel) and every
+    workgroup picks the result up.  fp32, bf16 and f16 activations, ragged row ranges, every output
+    against the oracle within the fp32 tolerance; two calls in a row on one handle reuse the scratch."""
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    x = np.random.default_rng(out + inf).standard_normal((1, inf)).astype(np.float32)
+    want = oracle.linear_forward(qw, cbp, cbr, bs, x)
+    y = layer.forward(x)
+    assert y.shape == (1, out) and _rel(y, want) < 1e-3
+    assert np.array_equal(layer.forward(2.0 * x), 2.0 * y)                 # exact linearity in a factor 2
+    xbits = oracle.f32_to_bf16_bits(x)
+    yb = layer.forward(xbits, tq.BF16, tq.F32)
+    assert _rel(yb, oracle.linear_forward(qw, cbp, cbr, bs, oracle.bf16_bits_to_f32(xbits))) < 1e-3
+    xh = x.astype(np.float16)
+    yh = layer.forward(xh, tq.F16, tq.F32)
+    assert _rel(yh, oracle.linear_forward(qw, cbp, cbr, bs, xh.astype(np.float32))) < 1e-3
+    assert np.array_equal(layer.forward(x), y)                             # the scratch holds nothing stale
+    x3 = np.concatenate([x, -x, 0.5 * x], axis=0)                          # three rows, one launch pair each
+    y3 = layer.forward(x3)
+    assert _rel(y3[2:3], 0.5 * y) < 1e-6 and _rel(y3[0:1], y) < 1e-6 and _rel(y3[1:2], -y) < 1e-6
+    layer.close()
+
+
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("xd", ["bf16", "f16"])
 @pytest.mark.parametrize("yd", ["f32", "bf16", "f16"])

@@ -37,6 +37,8 @@ struct LayerView {
     int mode;
     float inv_scale;                 // 1/sqrt(in), computed on the host as the reference does
     float inv_sqrt_bs;               // 1/sqrt(block_size), host computed
+    float* xrot_work;                // scratch of 2 * in_features floats (rows wider than 16384 columns: the
+                                     // batch-1 path rotates the activations once, in a kernel of its own), or NULL
 };
 
 // Launchers (tq_gemv.hip, tq_dequant.hip).  All return hipError_t of the launch.

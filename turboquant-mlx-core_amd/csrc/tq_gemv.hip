@@ -239,9 +239,14 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
         for (int b = 0; b < NB; ++b) {
             if constexpr (!kEarlyX)  // register budget: load late, one batch row at a time
                 load_owned<combined>(a.x, a.x_dtype, (size_t)b * a.L.in_features, col_a, col_b, act_a, act_b, xt[b]);
-            if constexpr (MODE == kDual)
-                rotate_private<combined>(xt[b], col_a, col_b, a.L.seed_residual, a.L.block_size, lane, xr[b]);
-            rotate_private<combined>(xt[b], col_a, col_b, a.L.seed_primary, a.L.block_size, lane, xt[b]);
+            if (a.pre_rotated) {     // rotated by tq_rotate_row_kernel (one batch row): nothing to do but pick them up
+                if constexpr (MODE == kDual)
+                    load_owned<combined>(a.x, a.x_dtype, (size_t)a.L.in_features, col_a, col_b, act_a, act_b, xr[b]);
+            } else {
+                if constexpr (MODE == kDual)
+                    rotate_private<combined>(xt[b], col_a, col_b, a.L.seed_residual, a.L.block_size, lane, xr[b]);
+                rotate_private<combined>(xt[b], col_a, col_b, a.L.seed_primary, a.L.block_size, lane, xt[b]);
+            }
         }
     }
     __syncthreads();                                          // tables visible to every wave
@@ -325,6 +330,28 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
     }
 }
 
+// H (s (.) x) of one activation row for one or two seeds, fp32, natural column order: out[p * cols + c].
+// One wave per 512-column tile (blocks of at most 512 columns).  Rows wider than 16384 columns run one
+// workgroup per CU whose waves would otherwise each rotate a slab of the row on their own, the same
+// work on every CU, which took a quarter of the kernel's time.
+__global__ __launch_bounds__(256) void tq_rotate_row_kernel(const void* __restrict__ x, int x_dtype,
+                                                            float* __restrict__ out, int cols, uint32_t seed0,
+                                                            uint32_t seed1, uint32_t bs) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int tile0 = ((int)blockIdx.x * 4 + (int)(threadIdx.x >> 6)) * kTile;
+    if (tile0 >= cols) return;
+    const int col = tile0 + lane * 8;
+    const bool active = col < cols;
+    const TileRaw raw = load_tile_raw(x, x_dtype, 0, active ? col : 0);
+    float v[8];
+    rotate_tile(raw, x_dtype, col, active, blockIdx.y ? seed1 : seed0, bs, lane, v);
+    if (active) {
+        float4* dst = reinterpret_cast<float4*>(out + (size_t)blockIdx.y * cols + col);
+        dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+        dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
 template <int MODE, int NB, int R, int MAXT, int NS>
 static hipError_t launch_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
     hipLaunchKernelGGL((tq_gemv_kernel<MODE, NB, R, MAXT, NS>), dim3(grid), dim3(threads), 0, stream, a);
@@ -363,6 +390,19 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
     }
 }
 
+// One batch row of a layer wider than 16384 columns: rotate it once for the whole grid (if the layer
+// has the scratch for it and blocks of at most 512 columns) and hand the kernel the result.
+static void pre_rotate(GemvArgs& a, hipStream_t stream) {
+    const LayerView& L = a.L;
+    if (!L.xrot_work || L.block_size > (uint32_t)kTile || L.in_features % 8 != 0) return;
+    const int tiles = (L.in_features + kTile - 1) / kTile;
+    hipLaunchKernelGGL(tq_rotate_row_kernel, dim3((tiles + 3) / 4, L.mode == kDual ? 2 : 1), dim3(256), 0, stream,
+                       a.x, a.x_dtype, L.xrot_work, L.in_features, L.seed_primary, L.seed_residual, L.block_size);
+    a.x = L.xrot_work;
+    a.x_dtype = kF32;
+    a.pre_rotated = 1;
+}
+
 // Batch rows are served 4, 2 or 1 per launch: the rotated activations of every
 // batch row live in registers, which bounds how many fit next to the weight
 // buffers (workgroups of up to 512 threads get 256 VGPRs per lane, larger ones 128).
@@ -383,12 +423,14 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
         int step = 1;
         if constexpr (MODE == kDual) {
             if (gemv_wide_supported(a.L, num_cus)) e = launch_gemv_wide(a, num_cus, stream);
-            else e = (W <= 8) ? launch_nb<MODE, 1, 512>(a, num_cus, stream) : launch_nb<MODE, 1, 1024>(a, num_cus, stream);
+            else if (W <= 8) e = launch_nb<MODE, 1, 512>(a, num_cus, stream);
+            else { pre_rotate(a, stream); e = launch_nb<MODE, 1, 1024>(a, num_cus, stream); }
         } else {
             if (left >= 4 && W <= 8)      { step = 4; e = launch_nb<MODE, 4, 512>(a, num_cus, stream); }
             else if (left >= 2 && W <= 8) { step = 2; e = launch_nb<MODE, 2, 512>(a, num_cus, stream); }
             else if (gemv_wide_supported(a.L, num_cus)) { step = 1; e = launch_gemv_wide(a, num_cus, stream); }
-            else                          { step = 1; e = launch_nb<MODE, 1, 1024>(a, num_cus, stream); }
+            else                          { step = 1; if (W > 8) pre_rotate(a, stream);
+                                            e = launch_nb<MODE, 1, 1024>(a, num_cus, stream); }
         }
         if (e != hipSuccess) return e;
         done += step;

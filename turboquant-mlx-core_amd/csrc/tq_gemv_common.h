@@ -17,8 +17,9 @@ struct GemvArgs {
     float out_scale; // inv_scale * inv_sqrt_bs
     const float* gate;   // optional [batch, out] fp32: the stored value becomes silu(gate) * y (gated MLP)
     int img_cols;    // wide kernel only: columns of the rotated-activation image in LDS (a multiple of 2048)
-    int rows_q, rows_rem;   // wide kernel only: rows per row range, and how many ranges hold one more
-    int w_inv;       // wide kernel only: (w * w_inv) >> 8 == w / W
+    int rows_q, rows_rem;   // rows per row range, and how many ranges hold one more
+    int w_inv;       // (w * w_inv) >> 8 == w / W
+    int pre_rotated; // narrow kernel: x holds fp32 rotated activations (second rotation in_features further on)
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

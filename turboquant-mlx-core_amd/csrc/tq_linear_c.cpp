@@ -71,6 +71,8 @@ struct tq_linear_s {
     void* d_work = nullptr; size_t work_bytes = 0;
     // Per-chunk partial products of the small-batch path.
     void* d_partial = nullptr; size_t partial_bytes = 0;
+    // Rotated activation row (both rotations) of the batch-1 path, layers wider than 16384 columns only.
+    float* d_xrot = nullptr;
 
     ~tq_linear_s() {
         if (d_primary) (void)hipFree(d_primary);
@@ -83,6 +85,7 @@ struct tq_linear_s {
         if (d_stage_y) (void)hipFree(d_stage_y);
         if (d_work) (void)hipFree(d_work);
         if (d_partial) (void)hipFree(d_partial);
+        if (d_xrot) (void)hipFree(d_xrot);
     }
 };
 
@@ -229,6 +232,12 @@ tq_linear_t create_impl(int in_features, int out_features,
     v.mode = mode;
     v.inv_scale = 1.0f / std::sqrt(static_cast<float>(in_features));      // src/dequantizer.cpp:76
     v.inv_sqrt_bs = 1.0f / std::sqrt(static_cast<float>(block_size));     // src/rotation.cpp:333
+    if (in_features > 16384) {     // allocated here so that a forward call never allocates on the batch-1 path
+        if (!hip_ok(hipMalloc((void**)&h->d_xrot, (size_t)2 * in_features * sizeof(float)), "hipMalloc(rotated row)")) {
+            delete h; return nullptr;
+        }
+    }
+    v.xrot_work = h->d_xrot;
     if (fused5) {
         h->fwd_view = v;
         h->fwd_view.mode = tq::kSharedLut;
