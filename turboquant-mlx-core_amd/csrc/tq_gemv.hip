@@ -429,8 +429,12 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
             if (left >= 4 && W <= 8)      { step = 4; e = launch_nb<MODE, 4, 512>(a, num_cus, stream); }
             else if (left >= 2 && W <= 8) { step = 2; e = launch_nb<MODE, 2, 512>(a, num_cus, stream); }
             else if (gemv_wide_supported(a.L, num_cus)) { step = 1; e = launch_gemv_wide(a, num_cus, stream); }
-            else                          { step = 1; if (W > 8) pre_rotate(a, stream);
-                                            e = launch_nb<MODE, 1, 1024>(a, num_cus, stream); }
+            else {
+                step = 1;
+                if (W > 8) pre_rotate(a, stream);
+                if (a.pre_rotated && gemv_wide_supported(a.L, num_cus, true)) e = launch_gemv_wide(a, num_cus, stream);
+                else e = launch_nb<MODE, 1, 1024>(a, num_cus, stream);
+            }
         }
         if (e != hipSuccess) return e;
         done += step;

@@ -184,7 +184,7 @@ __device__ __forceinline__ int stage_index(int col_in_slab) {
 
 // One batch row, rows of up to 8 slabs (tq_gemv_wide.hip): one workgroup per CU, tables and rotated
 // activations built once per CU.  `a` as for the narrow kernel (x, y, gate already at the batch row).
-bool gemv_wide_supported(const LayerView& L, int num_cus);
+bool gemv_wide_supported(const LayerView& L, int num_cus, bool pre_rotated = false);
 hipError_t launch_gemv_wide(const GemvArgs& a, int num_cus, hipStream_t stream);
 
 }  // namespace tq

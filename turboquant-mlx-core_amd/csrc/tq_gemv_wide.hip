@@ -115,8 +115,11 @@ __device__ __forceinline__ void take_from_image(const float* image, int lane, in
 // counter in LDS.  Waves of one CU progress at different rates (the spread between the first and the
 // last wave of a CU to finish equal shares was a fifth of the run time); with the counter they all
 // finish within one row group of each other.
-template <int MODE, int R, int TILES, bool PAIR, bool DYN>
+// PRE (rows of 9 to 16 slabs): a.x holds the rotated activations as fp32 (tq_rotate_row_kernel); the
+// waves pick their columns up from there, and no image is kept in LDS.
+template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false>
 __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
+    static_assert(!PRE || (!PAIR && !DYN && MODE != kDual && TILES == 1), "pre-rotated rows: plain slab streams");
     static_assert(!PAIR || MODE == kSharedLut, "row pairs need the one-byte-per-weight plane");
     static_assert(!DYN || (!PAIR && MODE != kDual), "the group counter serves one-wave row streams");
     constexpr int NS = 2;                           // register ring: one group decoded, one in flight
@@ -202,10 +205,22 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) tv[e] = tab[e0 + e];
     TileRaw raw[TILES];
+    float xt[NX];       // rotated activations, kept in registers for the whole kernel
+    if constexpr (PRE) {
+        const float4* pa = reinterpret_cast<const float4*>(static_cast<const float*>(a.x) + (act_a ? col_a : 0));
+        const float4* pb = reinterpret_cast<const float4*>(static_cast<const float*>(a.x) + (act_b ? col_b : 0));
 #pragma unroll
-    for (int t = 0; t < TILES; ++t) {         // tiles past the row re-read its start and are not used
-        const int col = (wave + t * nwaves) * kTile + lane * 8;
-        raw[t] = load_tile_fixed(a.x, a.x_dtype, col < a.L.in_features ? col : 0);
+        for (int i = 0; i < 4; ++i) {
+            const float4 u = pa[i], w = pb[i];
+            xt[4 * i] = u.x; xt[4 * i + 1] = u.y; xt[4 * i + 2] = u.z; xt[4 * i + 3] = u.w;
+            xt[16 + 4 * i] = w.x; xt[17 + 4 * i] = w.y; xt[18 + 4 * i] = w.z; xt[19 + 4 * i] = w.w;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {     // tiles past the row re-read its start and are not used
+            const int col = (wave + t * nwaves) * kTile + lane * 8;
+            raw[t] = load_tile_fixed(a.x, a.x_dtype, col < a.L.in_features ? col : 0);
+        }
     }
     // The weight requests stay behind the small ones: loads complete in order, and the rotation
     // must not wait for weights.
@@ -228,7 +243,12 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
         }
     }
 
-    float xt[NX];       // rotated activations, kept in registers for the whole kernel
+    if constexpr (PRE) {
+        __syncthreads();              // tables visible to every wave
+        fetch(1, r_begin + V);
+#pragma unroll
+        for (int k = 0; k < NX; ++k) xt[k] = ((k < 16) ? act_a : act_b) ? xt[k] : 0.0f;   // idle runs contribute 0
+    } else {
     float* const image = reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes);
     rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_primary, a.L.block_size, image, wave,
                                      nwaves, lane);
@@ -246,6 +266,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     }
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
+    }
 
     // One row (or with PAIR the same columns of two rows: p -> sum, q -> sum2).
     auto decode_row = [&](const uint4& p, const uint4& q, float& sum, float& sum2) {
@@ -360,10 +381,10 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     if (it0 < a.iters) consume(0, r_begin + it0 * V, it0);
 }
 
-template <int MODE, int R, int TILES, bool PAIR, bool DYN = false>
+template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
-    const size_t lds = (size_t)kRegionBytes + kPartialBytes + (size_t)a.img_cols * sizeof(float);
-    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN>;
+    const size_t lds = (size_t)kRegionBytes + kPartialBytes + (PRE ? 0 : (size_t)a.img_cols * sizeof(float));
+    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE>;
     // More LDS than the default limit has to be asked for, once per kernel and device.
     static bool asked[64] = {};
     int dev = 0;
@@ -394,7 +415,7 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     a.S = 16 / a.W;                                          // row streams sharing the CU
     const int threads = a.W * a.S * kWave;
     const int padded = slabs * kSlab;
-    if (padded > kMaxImageCols) return hipErrorInvalidValue;   // gemv_wide_supported() rules this out
+    if (padded > kMaxImageCols && !a.pre_rotated) return hipErrorInvalidValue;   // gemv_wide_supported() rules this out
     a.img_cols = padded;
 
     int grid = (out + a.S - 1) / a.S;
@@ -410,6 +431,10 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     const int R = max_rows >= 2 * per_r ? 2 : 1;
     a.iters = (max_rows + R * per_r - 1) / (R * per_r);
 
+    if constexpr (!PAIR && MODE != kDual) {
+        if (a.pre_rotated) return R == 2 ? launch_wide_one<MODE, 2, 1, false, false, true>(a, grid, threads, stream)
+                                         : launch_wide_one<MODE, 1, 1, false, false, true>(a, grid, threads, stream);
+    }
     const int ntiles = (a.L.in_features + kTile - 1) / kTile;
     const bool two = ntiles > threads / kWave;              // at most two tiles per wave: checked by the caller
     if constexpr (!PAIR && MODE != kDual) {
@@ -430,17 +455,18 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
 // One batch row, blocks of at most 512 columns, per-stream share of the plane below 2 GB.
 // Shared rotation and primary only: rows of 1 to 8 slabs, or (shared rotation) of an odd number,
 // 3 to 15, of 1024-column halves.  Dual rotation: rows of 1 to 8 slabs.
-bool gemv_wide_supported(const LayerView& L, int num_cus) {
+bool gemv_wide_supported(const LayerView& L, int num_cus, bool pre_rotated) {
     if (L.mode != kSharedLut && L.mode != kPrimaryOnly && L.mode != kDual) return false;
     if (L.block_size > (uint32_t)kTile) return false;
     const int slabs = (L.in_features / kChunk + kWave - 1) / kWave;
     int W = slabs;
-    if (wants_pairs(L)) W = L.in_features / (kSlab / 2);
+    if (pre_rotated) { if (L.mode == kDual || slabs < 9 || slabs > 16) return false; }
+    else if (wants_pairs(L)) W = L.in_features / (kSlab / 2);
     else if (L.mode == kDual) { if (slabs > 8) return false; W = 2 * slabs; }   // two waves per slab
     else if (slabs < 1 || slabs > 8) return false;
     const int S = 16 / W;
     const int ntiles = (L.in_features + kTile - 1) / kTile;
-    if (ntiles > 2 * W * S) return false;
+    if (!pre_rotated && ntiles > 2 * W * S) return false;
     const size_t row_bytes = L.mode == kSharedLut ? (size_t)L.in_features : (size_t)L.in_features / 2;
     const bool shared_range = W == 1 && L.mode != kDual;    // one row range per workgroup, shared by its waves
     const long long streams = (long long)(num_cus > 0 ? num_cus : 1) * (shared_range ? 1 : S);
@@ -453,7 +479,7 @@ hipError_t launch_gemv_wide(const GemvArgs& base, int num_cus, hipStream_t strea
     a.chunks = a.L.in_features / kChunk;
     a.W = (a.chunks + kWave - 1) / kWave;
     if (a.L.mode == kSharedLut)
-        return wants_pairs(a.L) ? launch_wide_mode<kSharedLut, true>(a, num_cus, stream)
+        return (!a.pre_rotated && wants_pairs(a.L)) ? launch_wide_mode<kSharedLut, true>(a, num_cus, stream)
                                 : launch_wide_mode<kSharedLut, false>(a, num_cus, stream);
     if (a.L.mode == kDual) return launch_wide_mode<kDual, false>(a, num_cus, stream);
     return launch_wide_mode<kPrimaryOnly, false>(a, num_cus, stream);
