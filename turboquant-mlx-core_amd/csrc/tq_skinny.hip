@@ -26,6 +26,7 @@ typedef uint32_t sk_u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kSkChunk = 512;            // columns per K chunk
 constexpr int kSkThreads = 512;          // 8 waves per workgroup, one workgroup per CU
 constexpr int kSkLutBytes = 256 * 256;
+constexpr int kSkStageBytes = 16 * kSkChunk * 2;   // 16 rows x 512 bf16 rotated activations
 
 struct SkinnyArgs {
     const void* x;             // FUSED: activations [batch, K], f16 or bf16
@@ -54,8 +55,10 @@ __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t l
 // FUSED: the workgroup rotates the 16 x 512 activations of its chunk itself (blocks of at most 512
 // columns: a block never leaves the chunk), instead of reading tile images a separate kernel wrote.
 template <bool FUSED>
-__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tq_skinny_kernel(SkinnyArgs a) {
-    __shared__ __align__(16) char smem[kSkLutBytes];
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_kernel(SkinnyArgs a) {
+    // table | 16 x 512 bf16 rotated activations (FUSED).  One workgroup of 8 waves per CU: 16 waves
+    // gained nothing, and 8 have the registers for two row groups in flight.
+    __shared__ __align__(16) char smem[kSkLutBytes + kSkStageBytes];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -67,44 +70,45 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const int wg_in_chunk = blockIdx.y;
     const int m = lane & 15, g = lane >> 4;               // A operand: batch row, k group; B operand: weight row, k group
 
-    // Table values of this thread's LDS slots, requested before anything else.
+    // Row groups of this wave: the groups are dealt out evenly over all waves that share the chunk.
+    const int me = wg_in_chunk * (kSkThreads / 64) + wave;
+    const int g_begin = me * a.groups_q + (me < a.groups_rem ? me : a.groups_rem);
+    const int g_end = g_begin + a.groups_q + (me < a.groups_rem ? 1 : 0);
+    const size_t col0 = (size_t)chunk * kSkChunk + 16 * g;
+    auto row_ptr = [&](int grp) {
+        int row = grp * 16 + m;
+        if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
+        return a.plane + (size_t)row * a.K + col0;
+    };
+
+    // Everything that has to come from memory is requested up front, the small things first (loads
+    // complete in order): table values, the activations this wave rotates, then the first row group,
+    // which travels while the activations are rotated and the table is built.
     constexpr int kSlots = 256 * 16 / kSkThreads;
     float tv[kSlots];
 #pragma unroll
     for (int k = 0; k < kSlots; ++k) tv[k] = a.tables[(tid + k * kSkThreads) >> 4];
-
-    sk_bf16x8 afrag[16];
+    TileRaw xin[2];
     if constexpr (FUSED) {
-        // Wave w rotates batch rows w and w + 8 of the chunk (one 512-column tile each, 8 values per
-        // lane) and writes them as bf16 into the first 16 KB of the table region, [16 rows][512];
-        // rows past the batch are zero.  The A operands are read back before the table is built.
-        constexpr int kPitch = kSkChunk * 2;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 2; ++t) {                      // batch rows w and w + 8 (row 0 again past the batch: not used)
             const int b = wave + 8 * t;
-            const int col = chunk * kSkChunk + lane * 8;
-            uint4 packed = make_uint4(0, 0, 0, 0);
-            if (b < a.batch) {                              // wave-uniform
-                TileRaw raw;
-                raw.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) + (size_t)b * a.K + col);
-                raw.b = make_uint4(0, 0, 0, 0);
-                float v[8];
-                rotate_tile(raw, a.x_dtype, col, true, a.seed, a.block_size, lane, v);
-                packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-                packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-                packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
-                packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
-            }
-            *reinterpret_cast<uint4*>(smem + b * kPitch + lane * 16) = packed;
+            xin[t].a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) +
+                                                       (size_t)(b < a.batch ? b : 0) * a.K + chunk * kSkChunk + lane * 8);
+            xin[t].b = make_uint4(0, 0, 0, 0);
         }
-        __syncthreads();
-        // k-step s covers columns 64 (s/2) + 16 g + 8 (s%2) + [0, 8) of the chunk, the same columns
-        // the B operand of that step decodes.
-#pragma unroll
-        for (int s = 0; s < 16; ++s)
-            afrag[s] = *reinterpret_cast<const sk_bf16x8*>(smem + m * kPitch + (64 * (s >> 1) + 16 * g + 8 * (s & 1)) * 2);
-        __syncthreads();                                    // everyone has its A operands: the region is free
     }
+    __builtin_amdgcn_sched_barrier(0);
+    // Plain loads, not streaming ones: a load instruction touches 64 bytes of each of 16 rows, half
+    // a cache line, and the other half is asked for by a later instruction; with the streaming
+    // hint that half was fetched from memory again (13 % more time).
+    sk_u32x4 rawA[8], rawB[8];                             // two row groups: one decoded, one in flight
+    auto request = [&](sk_u32x4 (&raw)[8], int grp) {
+        const uint8_t* p = row_ptr(grp);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+    };
+    if (g_begin < g_end) request(rawA, g_begin);
 
     // Decode table -> LDS, one private column per lane, values rounded to bf16 (upper half of the dword).
     {
@@ -116,10 +120,37 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         }
     }
 
-    // A operands of the chunk: k-step s covers columns 64 (s/2) + 16 g + 8 (s%2) + [0, 8) of the chunk,
-    // the same columns the B operand of that step decodes (any column order is fine as long as both
-    // operands agree).  Tile images: [K/32][256][32] bf16 with 16-byte slots XOR-permuted per row.
-    if constexpr (!FUSED) {
+    sk_bf16x8 afrag[16];
+    char* const stage = smem + kSkLutBytes;
+    if constexpr (FUSED) {
+        // Wave w rotates batch rows w and w + 8 of the chunk (one 512-column tile each, 8 values per
+        // lane; blocks of at most 512 columns: a block never leaves the chunk) and writes them as bf16,
+        // [16 rows][512]; rows past the batch are zero.
+        constexpr int kPitch = kSkChunk * 2;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int b = wave + 8 * t;
+            const int col = chunk * kSkChunk + lane * 8;
+            uint4 packed = make_uint4(0, 0, 0, 0);
+            if (b < a.batch) {                              // wave-uniform
+                float v[8];
+                rotate_tile(xin[t], a.x_dtype, col, true, a.seed, a.block_size, lane, v);
+                packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+                packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+                packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
+                packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
+            }
+            *reinterpret_cast<uint4*>(stage + b * kPitch + lane * 16) = packed;
+        }
+        __syncthreads();                                    // table and activations visible
+        // k-step s covers columns 64 (s/2) + 16 g + 8 (s%2) + [0, 8) of the chunk, the same columns
+        // the B operand of that step decodes (any column order is fine as long as both agree).
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+            afrag[s] = *reinterpret_cast<const sk_bf16x8*>(stage + m * kPitch + (64 * (s >> 1) + 16 * g + 8 * (s & 1)) * 2);
+    } else {
+        // Tile images written by tq_rotate_bf16_kernel: [K/32][256][32] bf16 with 16-byte slots
+        // XOR-permuted per row; same column order as above.
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
             const int off = 16 * g + 8 * (s & 1);              // column inside the 64-column piece
@@ -128,26 +159,9 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
             afrag[s] = *reinterpret_cast<const sk_bf16x8*>(reinterpret_cast<const char*>(a.xt) +
                                                            ((size_t)kt * 256 + m) * 64 + slot * 16);
         }
+        __syncthreads();                                    // table visible
     }
-    __syncthreads();                                       // table visible
 
-    // Row groups of this wave: the groups are dealt out evenly over all waves that share the chunk.
-    const int me = wg_in_chunk * (kSkThreads / 64) + wave;
-    const int g_begin = me * a.groups_q + (me < a.groups_rem ? me : a.groups_rem);
-    const int g_end = g_begin + a.groups_q + (me < a.groups_rem ? 1 : 0);
-
-    const size_t col0 = (size_t)chunk * kSkChunk + 16 * g;
-    auto row_ptr = [&](int grp) {
-        int row = grp * 16 + m;
-        if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
-        return a.plane + (size_t)row * a.K + col0;
-    };
-    // Plain loads, not streaming ones: a load instruction touches 64 bytes of each of 16 rows, half
-    // a cache line, and the other half is asked for by a later instruction; with the streaming
-    // hint that half was fetched from memory again (13 % more time).
-    // The 8 loads of a group live in 32 registers; as soon as one has been decoded it is replaced
-    // by the same piece of the next group, so a full group of loads is always in flight.
-    sk_u32x4 raw[8];
     auto lookup2 = [&](uint32_t w) {                       // 4 weights -> 2 registers of bf16 pairs
         const uint32_t v0 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 0));
         const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 1));
@@ -156,21 +170,12 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         // entries are fp32 patterns with the value in the upper half: {v0.hi, v1.hi}, {v2.hi, v3.hi}
         return make_uint2(__builtin_amdgcn_perm(v1, v0, 0x07060302u), __builtin_amdgcn_perm(v3, v2, 0x07060302u));
     };
-
-    if (g_begin < g_end) {
-        const uint8_t* p = row_ptr(g_begin);
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
-    }
-    for (int grp = g_begin; grp < g_end; ++grp) {
-        const bool more = grp + 1 < g_end;
-        const uint8_t* pn = row_ptr(more ? grp + 1 : grp);
+    // One row group: 16 x 512 weights of the chunk -> 16 x 16 partial product.
+    auto multiply = [&](const sk_u32x4 (&raw)[8], int grp) {
         sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             const sk_u32x4 w = raw[q];
-            if (more) raw[q] = (*reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
             const uint2 p0 = lookup2(w.x), p1 = lookup2(w.y), p2 = lookup2(w.z), p3 = lookup2(w.w);
             const sk_u32x4 b0 = {p0.x, p0.y, p1.x, p1.y}, b1 = {p2.x, p2.y, p3.x, p3.y};
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * q], __builtin_bit_cast(sk_bf16x8, b0), acc, 0, 0, 0);
@@ -185,6 +190,15 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
                 if (b < a.batch) a.partial[((size_t)chunk * 16 + b) * a.N + n] = acc[r];
             }
         }
+    };
+
+    // The next group is requested before the current one is decoded (unrolled twice: static buffers).
+    for (int grp = g_begin; grp < g_end; grp += 2) {
+        if (grp + 1 < g_end) request(rawB, grp + 1);
+        multiply(rawA, grp);
+        if (grp + 1 >= g_end) break;
+        if (grp + 2 < g_end) request(rawA, grp + 2);
+        multiply(rawB, grp + 1);
     }
 }
 
@@ -208,60 +222,23 @@ struct SkinnyNibbleArgs {
     int groups_q, groups_rem;  // groups / workers and groups % workers (workers = waves sharing a unit)
 };
 
-__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
-    __shared__ __align__(16) char smem[16 * 1024];         // 16 x 512 bf16 activations, then the 4 KB table
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
+    constexpr int kTabBytes = 16 * 256;                    // 16 entries, one private column per lane
+    __shared__ __align__(16) char smem[kTabBytes + kSkStageBytes];   // table | 16 x 512 bf16 rotated activations
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t laneoff = (uint32_t)lane << 2;
 
-    // (grid = units x workgroups per unit; unit = chunk * planes + plane)
+    // (grid = units x workgroups per unit; unit = chunk * planes + plane; one workgroup per CU)
     const int unit = blockIdx.x;
     const int wg_in_unit = blockIdx.y;
     const int chunk = a.planes == 2 ? unit >> 1 : unit, pl = a.planes == 2 ? unit & 1 : 0;
     const int m = lane & 15, g = lane >> 4;
 
-    const float tval = a.tables[16 * pl + (tid >> 4 & 15)];        // threads 0..255 fill the 256 table slots
-
-    // Rotate batch rows w and w + 8 of the chunk with this plane's seed -> bf16 [16][512] in LDS.
-    constexpr int kPitch = kSkChunk * 2;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int b = wave + 8 * t;
-        const int col = chunk * kSkChunk + lane * 8;
-        uint4 packed = make_uint4(0, 0, 0, 0);
-        if (b < a.batch) {                                  // wave-uniform
-            TileRaw raw;
-            raw.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) + (size_t)b * a.K + col);
-            raw.b = make_uint4(0, 0, 0, 0);
-            float v[8];
-            rotate_tile(raw, a.x_dtype, col, true, a.seed[pl], a.block_size, lane, v);
-            packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-            packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-            packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
-            packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
-        }
-        *reinterpret_cast<uint4*>(smem + b * kPitch + lane * 16) = packed;
-    }
-    __syncthreads();
-    // A operands.  Matrix step s = 4 q + d multiplies columns 128 q + 32 g + 8 d + [0, 8) of the chunk:
-    // the 8 nibbles of dword d of the lane's 16-byte piece q (piece q of lane group g starts at byte
-    // 64 q + 16 g of the row's 256 bytes).
-    sk_bf16x8 afrag[16];
-#pragma unroll
-    for (int s = 0; s < 16; ++s)
-        afrag[s] = *reinterpret_cast<const sk_bf16x8*>(smem + m * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
-    __syncthreads();                                        // everyone has its A operands: the region is free
-    if (tid < 256) {                                        // 16 entries x 16 slots of 16 bytes, values rounded to bf16
-        const uint32_t v = (uint32_t)float_to_bf16_bits(tval) << 16;
-        reinterpret_cast<uint4*>(smem)[tid] = make_uint4(v, v, v, v);
-    }
-    __syncthreads();
-
     const int me = wg_in_unit * (kSkThreads / 64) + wave;
     const int g_begin = me * a.groups_q + (me < a.groups_rem ? me : a.groups_rem);
     const int g_end = g_begin + a.groups_q + (me < a.groups_rem ? 1 : 0);
-
     const uint8_t* plane = a.plane[pl];
     const size_t row_bytes = (size_t)a.K >> 1;
     const size_t byte0 = (size_t)chunk * (kSkChunk / 2) + 16 * g;
@@ -270,6 +247,58 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
         return plane + (size_t)row * row_bytes + byte0;
     };
+
+    // Small loads first (they complete in order), then the first row group, which travels while the
+    // activations are rotated.
+    const float tval = a.tables[16 * pl + (tid >> 4 & 15)];        // threads 0..255 fill the 256 table slots
+    TileRaw xin[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {                          // batch rows w and w + 8 (row 0 again past the batch: not used)
+        const int b = wave + 8 * t;
+        xin[t].a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) +
+                                                   (size_t)(b < a.batch ? b : 0) * a.K + chunk * kSkChunk + lane * 8);
+        xin[t].b = make_uint4(0, 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    sk_u32x4 rawA[4], rawB[4];                             // two row groups: one decoded, one in flight
+    auto request = [&](sk_u32x4 (&raw)[4], int grp) {
+        const uint8_t* p = row_ptr(grp);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+    };
+    if (g_begin < g_end) request(rawA, g_begin);
+
+    if (tid < 256) {                                        // 16 entries x 16 slots of 16 bytes, values rounded to bf16
+        const uint32_t v = (uint32_t)float_to_bf16_bits(tval) << 16;
+        reinterpret_cast<uint4*>(smem)[tid] = make_uint4(v, v, v, v);
+    }
+    // Rotate batch rows w and w + 8 of the chunk with this plane's seed -> bf16 [16][512] in LDS.
+    constexpr int kPitch = kSkChunk * 2;
+    char* const stage = smem + kTabBytes;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int b = wave + 8 * t;
+        const int col = chunk * kSkChunk + lane * 8;
+        uint4 packed = make_uint4(0, 0, 0, 0);
+        if (b < a.batch) {                                  // wave-uniform
+            float v[8];
+            rotate_tile(xin[t], a.x_dtype, col, true, a.seed[pl], a.block_size, lane, v);
+            packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+            packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+            packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
+            packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
+        }
+        *reinterpret_cast<uint4*>(stage + b * kPitch + lane * 16) = packed;
+    }
+    __syncthreads();                                        // table and activations visible
+    // A operands.  Matrix step s = 4 q + d multiplies columns 128 q + 32 g + 8 d + [0, 8) of the chunk:
+    // the 8 nibbles of dword d of the lane's 16-byte piece q (piece q of lane group g starts at byte
+    // 64 q + 16 g of the row's 256 bytes).
+    sk_bf16x8 afrag[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s)
+        afrag[s] = *reinterpret_cast<const sk_bf16x8*>(stage + m * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
+
     // One dword = 8 weights of 8 consecutive columns (low nibble first) -> one B operand.
     auto operand = [&](uint32_t w) {
         const uint32_t ce = w & 0x0F0F0F0Fu, co = (w >> 4) & 0x0F0F0F0Fu;
@@ -284,22 +313,11 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
                             __builtin_amdgcn_perm(o[2], e[2], 0x07060302u), __builtin_amdgcn_perm(o[3], e[3], 0x07060302u)};
         return __builtin_bit_cast(sk_bf16x8, r);
     };
-
-    sk_u32x4 raw[4];
-    if (g_begin < g_end) {
-        const uint8_t* p = row_ptr(g_begin);
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-            raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
-    }
-    for (int grp = g_begin; grp < g_end; ++grp) {
-        const bool more = grp + 1 < g_end;
-        const uint8_t* pn = row_ptr(more ? grp + 1 : grp);
+    auto multiply = [&](const sk_u32x4 (&raw)[4], int grp) {
         sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const sk_u32x4 w = raw[q];
-            if (more) raw[q] = (*reinterpret_cast<const sk_u32x4*>(pn + 64 * q));
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 0], operand(w.x), acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 1], operand(w.y), acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 2], operand(w.z), acc, 0, 0, 0);
@@ -313,6 +331,14 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(4, 4
                 if (b < a.batch) a.partial[((size_t)unit * 16 + b) * a.N + n] = acc[r];
             }
         }
+    };
+    // The next group is requested before the current one is decoded (unrolled twice: static buffers).
+    for (int grp = g_begin; grp < g_end; grp += 2) {
+        if (grp + 1 < g_end) request(rawB, grp + 1);
+        multiply(rawA, grp);
+        if (grp + 1 >= g_end) break;
+        if (grp + 2 < g_end) request(rawA, grp + 2);
+        multiply(rawB, grp + 1);
     }
 }
 
@@ -366,7 +392,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         n.planes = L.mode == kDual ? 2 : 1;
         n.units = L.in_features / kSkChunk * n.planes;
         n.groups = (L.out_features + 15) / 16;
-        n.wgs_per_unit = 2 * num_cus / n.units > 0 ? 2 * num_cus / n.units : 1;
+        n.wgs_per_unit = num_cus / n.units > 0 ? num_cus / n.units : 1;   // one workgroup per CU
         const int workers_n = n.wgs_per_unit * (kSkThreads / 64);
         n.groups_q = n.groups / workers_n;
         n.groups_rem = n.groups % workers_n;
@@ -393,7 +419,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     a.batch = batch; a.N = L.out_features; a.K = L.in_features;
     a.chunks = L.in_features / kSkChunk;
     a.groups = (L.out_features + 15) / 16;
-    a.wgs_per_chunk = 2 * num_cus / a.chunks > 0 ? 2 * num_cus / a.chunks : 1;   // two workgroups per CU
+    a.wgs_per_chunk = num_cus / a.chunks > 0 ? num_cus / a.chunks : 1;   // one workgroup per CU
     const int workers = a.wgs_per_chunk * (kSkThreads / 64);
     a.groups_q = a.groups / workers;
     a.groups_rem = a.groups % workers;
