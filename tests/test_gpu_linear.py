@@ -127,10 +127,12 @@ def test_forward_batch1_wide_rows(tq, oracle, mode, out, inf, bs):
     xb = oracle.bf16_bits_to_f32(xbits)
     yb = layer.forward(xbits, tq.BF16, tq.F32)
     assert _rel(yb, oracle.linear_forward(qw, cbp, cbr, bs, xb)) < 1e-3
-    # three rows of fp32 activations: the first two go through the two-row kernel, the third alone
+    # three rows of fp32 activations: the first two go through the two-row kernel, the third alone.
+    # (Nibble planes: the one-row kernel reads centroid pairs rounded to fp16, the two-row kernel fp32
+    # centroids, so the two agree to the fp32 tolerance only.)
     x3 = np.concatenate([x, -x, 0.5 * x], axis=0)
     y3 = layer.forward(x3)
-    assert _rel(y3[2:3], 0.5 * y) < 1e-6 and _rel(y3[0:1], y) < 1e-6
+    assert _rel(y3[2:3], 0.5 * y) < 1e-6 and _rel(y3[0:1], y) < (1e-6 if mode == "shared" else 1e-3)
     layer.close()
 
 

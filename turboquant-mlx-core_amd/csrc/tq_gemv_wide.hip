@@ -39,6 +39,7 @@ namespace tq {
 namespace {
 
 constexpr int kMaxImageCols = 16384;             // widest rotated-activation image in LDS (64 KB)
+constexpr int kPairDualSlabs = 3;                // dual rotation with byte-pair tables: 2 x 64 KB of tables leave 24 KB
 
 // Marks a loaded value as consumed here.  A load whose result is only read on some paths stays
 // "possibly in flight" for the compiler on the others, and it then waits for it (and, as loads
@@ -117,8 +118,13 @@ __device__ __forceinline__ void take_from_image(const float* image, int lane, in
 // finish within one row group of each other.
 // PRE (rows of 9 to 16 slabs): a.x holds the rotated activations as fp32 (tq_rotate_row_kernel); the
 // waves pick their columns up from there, and no image is kept in LDS.
-template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false>
+// PT (nibble planes): the table is indexed by a whole byte of the plane and an entry holds the
+// centroids of both its nibbles, rounded to fp16: one table read and two mixed-precision FMAs
+// (v_fma_mix_f32) per byte instead of two reads, two permutes and two FMAs.  64 KB per plane.
+template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false>
 __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
+    static_assert(!PT || MODE != kSharedLut, "pair tables serve the nibble planes");
+    constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;   // decode tables
     static_assert(!PRE || (!PAIR && !DYN && MODE != kDual && TILES == 1), "pre-rotated rows: plain slab streams");
     static_assert(!PAIR || MODE == kSharedLut, "row pairs need the one-byte-per-weight plane");
     static_assert(!DYN || (!PAIR && MODE != kDual), "the group counter serves one-wave row streams");
@@ -126,7 +132,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     constexpr int V = PAIR ? 2 * R : R;             // rows, and sums, per row group
     constexpr int NX = PAIR ? 16 : kChunk;          // rotated activations per lane
     extern __shared__ __align__(16) char smem[];    // tables | cross-wave partial sums | activation image
-    float* partial = reinterpret_cast<float*>(smem + kRegionBytes);   // [2][waves][V]
+    float* partial = reinterpret_cast<float*>(smem + kRegion);   // [2][waves][V]
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -195,7 +201,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     // tiles, then the weights.  (Every vector memory instruction of a wave occupies the CU's
     // address unit for 16 cycles, and 16 waves share it: the table values, which are the same for
     // all lanes, come through scalar loads instead.)
-    constexpr int kEntries = (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
+    constexpr int kEntries = PT ? (MODE == kDual ? 512 : 256) : (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
     // Wave w writes table entries 16 w .. 16 w + 15 (then 16 (w + nwaves) ..); the first 16 values
     // are requested here.
     typedef const __attribute__((address_space(4))) float cfloat;     // uniform address: scalar load
@@ -203,7 +209,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     const int e0 = wave * 16 < kEntries ? wave * 16 : 0;
     float tv[16];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) tv[e] = tab[e0 + e];
+    for (int e = 0; e < 16; ++e) tv[e] = PT ? 0.0f : tab[e0 + e];
     TileRaw raw[TILES];
     float xt[NX];       // rotated activations, kept in registers for the whole kernel
     if constexpr (PRE) {
@@ -230,7 +236,18 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     // Decode tables -> LDS, one private column per lane.
     int* const next_group = reinterpret_cast<int*>(partial);    // DYN: first group nobody has taken yet
     if (DYN && tid == 0) *next_group = 2 * nwaves;              // (groups w and w + nwaves are wave w's first two)
-    {
+    if constexpr (PT) {
+        // Entry e of a plane's table: fp16 centroid of nibble e & 15 in the low half, of nibble e >> 4
+        // in the high half.  Chunk c = 16 entries with the same high nibble; chunks 16.. are plane 1.
+        uint32_t* const dst = reinterpret_cast<uint32_t*>(smem) + lane;
+        for (int c = wave; c * 16 < kEntries; c += nwaves) {
+            const int pl = c >> 4;
+            const uint32_t hi = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)tab[16 * pl + (c & 15)]) << 16;
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                dst[(c * 16 + e) * kWave] = hi | (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)tab[16 * pl + e]);
+        }
+    } else {
         // Lane l stores each entry's value into its own column, 4 l bytes into the entry's 256.
         float* const dst = reinterpret_cast<float*>(smem) + lane;
         if (wave * 16 < kEntries) {
@@ -249,7 +266,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
 #pragma unroll
         for (int k = 0; k < NX; ++k) xt[k] = ((k < 16) ? act_a : act_b) ? xt[k] : 0.0f;   // idle runs contribute 0
     } else {
-    float* const image = reinterpret_cast<float*>(smem + kRegionBytes + kPartialBytes);
+    float* const image = reinterpret_cast<float*>(smem + kRegion + kPartialBytes);
     rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_primary, a.L.block_size, image, wave,
                                      nwaves, lane);
     __syncthreads();                  // image and tables (and the group counter) visible to every wave
@@ -270,6 +287,28 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
 
     // One row (or with PAIR the same columns of two rows: p -> sum, q -> sum2).
     auto decode_row = [&](const uint4& p, const uint4& q, float& sum, float& sum2) {
+        if constexpr (PT) {
+            const char* tabp = smem + plane * kLut256Bytes;
+            const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
+            uint32_t pv[16];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                pv[4 * d + 0] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<0>(pw[d], laneoff));
+                pv[4 * d + 1] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<1>(pw[d], laneoff));
+                pv[4 * d + 2] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<2>(pw[d], laneoff));
+                pv[4 * d + 3] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<3>(pw[d], laneoff));
+            }
+            float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {       // byte i: columns 2 i (low nibble) and 2 i + 1
+                const _Float16 lo = __builtin_bit_cast(_Float16, (uint16_t)(pv[i] & 0xffffu));
+                const _Float16 hi = __builtin_bit_cast(_Float16, (uint16_t)(pv[i] >> 16));
+                s0 = __builtin_fmaf((float)lo, xt[2 * i], s0);
+                s1 = __builtin_fmaf((float)hi, xt[2 * i + 1], s1);
+            }
+            sum = s0 + s1;
+            return;
+        }
         float val[kChunk];
         // (dual rotation: the residual table follows the primary one, 16 entries of 256 bytes each)
         lookup32<MODE == kSharedLut, 0>(p, q, smem + plane * kTab16Bytes, laneoff, val);
@@ -381,10 +420,11 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     if (it0 < a.iters) consume(0, r_begin + it0 * V, it0);
 }
 
-template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false>
+template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false, bool PT = false>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
-    const size_t lds = (size_t)kRegionBytes + kPartialBytes + (PRE ? 0 : (size_t)a.img_cols * sizeof(float));
-    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE>;
+    constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
+    const size_t lds = (size_t)kRegion + kPartialBytes + (PRE ? 0 : (size_t)a.img_cols * sizeof(float));
+    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE, PT>;
     // More LDS than the default limit has to be asked for, once per kernel and device.
     static bool asked[64] = {};
     int dev = 0;
@@ -392,7 +432,8 @@ hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 64 || !asked[dev]) {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kRegionBytes + kPartialBytes + kMaxImageCols * (int)sizeof(float));
+                                kRegion + kPartialBytes +
+                                    ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float));
         if (e != hipSuccess) return e;
         if (dev >= 0 && dev < 64) asked[dev] = true;
     }
@@ -404,6 +445,27 @@ hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t
 bool wants_pairs(const LayerView& L) {
     return L.mode == kSharedLut && L.in_features % kSlab == kSlab / 2 && L.in_features / (kSlab / 2) >= 3 &&
            L.in_features <= kMaxImageCols;
+}
+
+template <int MODE, bool PAIR, bool PT>
+hipError_t launch_wide_shape(const GemvArgs& a, int grid, int threads, int R, bool two, int out, hipStream_t stream) {
+    if constexpr (!PAIR && MODE != kDual) {
+        if (a.pre_rotated) return R == 2 ? launch_wide_one<MODE, 2, 1, false, false, true, PT>(a, grid, threads, stream)
+                                         : launch_wide_one<MODE, 1, 1, false, false, true, PT>(a, grid, threads, stream);
+        if (a.W == 1) {                                     // one slab: 16 one-wave streams fed from a group counter
+            const int rows_wg = (out + grid - 1) / grid;
+            if (rows_wg >= 4 * a.S) return launch_wide_one<MODE, 2, 1, false, true, false, PT>(a, grid, threads, stream);
+            return launch_wide_one<MODE, 1, 1, false, true, false, PT>(a, grid, threads, stream);
+        }
+    }
+    if constexpr (MODE != kSharedLut) {
+        if (R == 4) return two ? launch_wide_one<MODE, 4, 2, PAIR, false, false, PT>(a, grid, threads, stream)
+                               : launch_wide_one<MODE, 4, 1, PAIR, false, false, PT>(a, grid, threads, stream);
+    }
+    if (R == 2) return two ? launch_wide_one<MODE, 2, 2, PAIR, false, false, PT>(a, grid, threads, stream)
+                           : launch_wide_one<MODE, 2, 1, PAIR, false, false, PT>(a, grid, threads, stream);
+    return two ? launch_wide_one<MODE, 1, 2, PAIR, false, false, PT>(a, grid, threads, stream)
+               : launch_wide_one<MODE, 1, 1, PAIR, false, false, PT>(a, grid, threads, stream);
 }
 
 template <int MODE, bool PAIR>
@@ -428,26 +490,16 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     a.w_inv = (256 + a.W - 1) / a.W;                        // (w * w_inv) >> 8 == w / W for w < 16, W <= 16
     const int max_rows = (int)(((long long)out + grid * a.S - 1) / (grid * a.S));   // longest share of a stream
     const int per_r = PAIR ? 2 : 1;                         // rows per unit of R
-    const int R = max_rows >= 2 * per_r ? 2 : 1;
+    // (nibble planes: a row is 16 bytes per lane, so four rows make the group of loads of two byte-plane rows)
+    const int R = (MODE != kSharedLut && !a.pre_rotated && max_rows >= 4) ? 4 : max_rows >= 2 * per_r ? 2 : 1;
     a.iters = (max_rows + R * per_r - 1) / (R * per_r);
 
-    if constexpr (!PAIR && MODE != kDual) {
-        if (a.pre_rotated) return R == 2 ? launch_wide_one<MODE, 2, 1, false, false, true>(a, grid, threads, stream)
-                                         : launch_wide_one<MODE, 1, 1, false, false, true>(a, grid, threads, stream);
-    }
     const int ntiles = (a.L.in_features + kTile - 1) / kTile;
     const bool two = ntiles > threads / kWave;              // at most two tiles per wave: checked by the caller
-    if constexpr (!PAIR && MODE != kDual) {
-        if (a.W == 1) {                                     // one slab: 16 one-wave streams fed from a group counter
-            const int rows_wg = (out + grid - 1) / grid;
-            if (rows_wg >= 4 * a.S) return launch_wide_one<MODE, 2, 1, false, true>(a, grid, threads, stream);
-            return launch_wide_one<MODE, 1, 1, false, true>(a, grid, threads, stream);
-        }
-    }
-    if (R == 2) return two ? launch_wide_one<MODE, 2, 2, PAIR>(a, grid, threads, stream)
-                           : launch_wide_one<MODE, 2, 1, PAIR>(a, grid, threads, stream);
-    return two ? launch_wide_one<MODE, 1, 2, PAIR>(a, grid, threads, stream)
-               : launch_wide_one<MODE, 1, 1, PAIR>(a, grid, threads, stream);
+    if constexpr (MODE == kSharedLut) return launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
+    else if constexpr (MODE == kPrimaryOnly) return launch_wide_shape<MODE, PAIR, true>(a, grid, threads, R, two, out, stream);
+    else return slabs <= kPairDualSlabs ? launch_wide_shape<MODE, PAIR, true>(a, grid, threads, R, two, out, stream)
+                                        : launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
 }
 
 }  // namespace
