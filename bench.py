@@ -24,7 +24,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152421.1 KiB + 648.9 KiB.
-MEASURED_TRAFFIC_BYTES = 312822886
+MEASURED_TRAFFIC_BYTES = 312965325
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
 
@@ -241,7 +241,7 @@ def main():
                                               "p90": float(np.percentile(spread_us, 90))},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "tq_gemv_wide_kernel<shared, R=2, TILES=1>", "algorithmic_bytes": B},
+                     "kernel": "tq_gemv_wide_kernel<shared, R=2, TILES=1, rows from an LDS counter>", "algorithmic_bytes": B},
     }
 
     # ---- CPU baseline on this host ---------------------------------------------------
@@ -393,7 +393,8 @@ def main():
             Bm = 2 * algorithmic_bytes(inter, hid, 1, 2, 4) + algorithmic_bytes(hid, inter, 1, 4, 4)
             extra["mlp_block_7b_bs1_" + ("shared_rotation" if shared else "dual_rotation")] = {
                 "us_per_block": us_m, "algorithmic_bytes": Bm, "hbm_frac": Bm / (us_m * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                "kernels_per_block": 3}
+                "kernels_per_block": 4,
+                "kernels": "gate, up (gated store), rotation of the 18944-wide intermediate row, down"}
             for m in blocks:
                 L.tq_mlp_free(m)
             for hs in keep:
