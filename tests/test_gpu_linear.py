@@ -137,6 +137,28 @@ def test_forward_batch1_wide_rows(tq, oracle, mode, out, inf, bs):
 
 
 @pytest.mark.parametrize("mode", ["shared", "primary_only", "dual"])
+@pytest.mark.parametrize("out,inf,bs", [(20001, 2048, 512), (16500, 1024, 256), (33003, 1536, 512), (4099, 2048, 128)])
+def test_forward_batch1_one_slab_rows(tq, oracle, mode, out, inf, bs):
+    """One activation row on rows of one slab (at most 2048 columns) with enough rows for groups of
+    two rows per wave: shared rotation and primary only hand the row groups of a workgroup to its
+    waves from a counter in LDS, dual rotation splits the waves by plane.  Row counts leave ragged
+    last groups and workgroups of unequal ranges; fp32 and bf16 activations against the oracle."""
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    x = np.random.default_rng(out + inf).standard_normal((1, inf)).astype(np.float32)
+    want = oracle.linear_forward(qw, cbp, cbr, bs, x)
+    y = layer.forward(x)
+    assert y.shape == (1, out) and _rel(y, want) < 1e-3
+    assert np.abs(y - want).max() < 1e-2 * np.abs(want).max()             # no row left out or taken twice
+    assert np.array_equal(layer.forward(2.0 * x), 2.0 * y)
+    assert np.array_equal(layer.forward(x), y)                             # same result on every call
+    xbits = oracle.f32_to_bf16_bits(x)
+    yb = layer.forward(xbits, tq.BF16, tq.F32)
+    assert _rel(yb, oracle.linear_forward(qw, cbp, cbr, bs, oracle.bf16_bits_to_f32(xbits))) < 1e-3
+    layer.close()
+
+
+@pytest.mark.parametrize("mode", ["shared", "primary_only", "dual"])
 @pytest.mark.parametrize("out,inf,bs", [(600, 27648, 512), (515, 18944, 256), (257, 17408, 512), (40, 20480, 2048)])
 def test_forward_batch1_rows_beyond_16384_columns(tq, oracle, mode, out, inf, bs):
     """One activation row on rows of 9 to 14 slabs: the row is rotated once by a kernel of its own
