@@ -343,25 +343,35 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 }
 
 // y[b, n] = norm[n] * out_scale * sum over chunks of partial[c][b][n]
+// grid = blocks of 64 columns x batch rows.  The four waves of a block share the chunks of those 64
+// columns (wave w takes chunks w, w + 4, ..., eight loads in flight at a time) and add up through
+// LDS: a single thread per output walking all chunks four at a time spent one memory latency per
+// four chunks, 4.5 us for a kernel that moves a few hundred KB.
 __global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __restrict__ partial,
                                                                const float* __restrict__ norms, void* __restrict__ y,
                                                                int y_dtype, int batch, int N, int chunks, float out_scale) {
-    // grid = column blocks x batch rows (no division per element)
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int b = blockIdx.y;
-    for (int n = blockIdx.x * blockDim.x + threadIdx.x; n < N; n += gridDim.x * blockDim.x) {
-        // four independent running sums: the loads of a thread do not wait for one another
-        float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
-        const float* p = partial + (size_t)b * N + n;
-        const size_t step = (size_t)16 * N;
-        int c = 0;
-        for (; c + 4 <= chunks; c += 4) {
-            s0 += p[(size_t)c * step];
-            s1 += p[(size_t)(c + 1) * step];
-            s2 += p[(size_t)(c + 2) * step];
-            s3 += p[(size_t)(c + 3) * step];
-        }
-        for (; c < chunks; ++c) s0 += p[(size_t)c * step];
-        store_scalar(y, y_dtype, (size_t)b * N + n, ((s0 + s1) + (s2 + s3)) * (out_scale * norms[n]));
+    const int n = blockIdx.x * 64 + lane;
+    const bool live = n < N;
+    const float nrm = live ? norms[n] : 0.0f;
+    const float* p = partial + (size_t)b * N + (live ? n : 0);
+    const size_t step = (size_t)16 * N;
+    float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    int c = wave;
+    for (; c + 28 < chunks; c += 32) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) s[k] += p[(size_t)(c + 4 * k) * step];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        if (c + 4 * k < chunks) s[k] += p[(size_t)(c + 4 * k) * step];
+    part[wave][lane] = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+    __syncthreads();
+    if (wave == 0 && live) {
+        const float t = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+        store_scalar(y, y_dtype, (size_t)b * N + n, t * (out_scale * nrm));
     }
 }
 
@@ -399,8 +409,8 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         hipLaunchKernelGGL(tq_skinny_nibble_kernel, dim3(n.units, n.wgs_per_unit), dim3(kSkThreads), 0, stream, n);
         hipError_t en = hipGetLastError();
         if (en != hipSuccess) return en;
-        const unsigned blocks_n = (unsigned)((L.out_features + 255) / 256);
-        hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks_n > 1024 ? 1024 : blocks_n, batch), dim3(256), 0, stream,
+        const unsigned blocks_n = (unsigned)((L.out_features + 63) / 64);
+        hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks_n, batch), dim3(256), 0, stream,
                            partial, L.norms, y, y_dtype, batch, L.out_features, n.units, L.inv_scale * L.inv_sqrt_bs);
         return hipGetLastError();
     }
@@ -427,8 +437,8 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     else hipLaunchKernelGGL(tq_skinny_kernel<false>, dim3(a.chunks, a.wgs_per_chunk), dim3(kSkThreads), 0, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const unsigned blocks = (unsigned)((L.out_features + 255) / 256);
-    hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks > 1024 ? 1024 : blocks, batch), dim3(256), 0, stream,
+    const unsigned blocks = (unsigned)((L.out_features + 63) / 64);
+    hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks, batch), dim3(256), 0, stream,
                        partial, L.norms, y, y_dtype, batch, L.out_features, a.chunks, L.inv_scale * L.inv_sqrt_bs);
     return hipGetLastError();
 }
