@@ -97,6 +97,16 @@ int tq_linear_mode(tq_linear_t layer);
 int tq_linear_forward(tq_linear_t layer, const void* x_dev, int x_dtype, int batch,
                       void* y_dev, int y_dtype, void* stream);
 
+/**
+ * Two or three layers applied to the SAME activation row (batch 1): y_devs[j][out_j] = x[in] . W_j^T,
+ * e.g. the q, k, v or the gate, up projections of a decoder layer.  Results are identical to n calls of
+ * tq_linear_forward; layers of equal width and mode (shared or dual rotation, blocks <= 512, more
+ * than 2048 columns for shared rotation) share one kernel launch, anything else is run one after the
+ * other.  No counterpart in the reference, whose forward is per layer (include/turboquant/linear.h:21-22).
+ */
+int tq_linear_forward_group(const tq_linear_t* layers, int n, const void* x_dev, int x_dtype,
+                            void* const* y_devs, int y_dtype, void* stream);
+
 /** Same with host buffers (copies in, runs, copies out, synchronises). */
 int tq_linear_forward_host(tq_linear_t layer, const void* x_host, int x_dtype, int batch,
                            void* y_host, int y_dtype);

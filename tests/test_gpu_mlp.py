@@ -76,7 +76,10 @@ def _silu(g):
                                                          (256, 640, 128, 3, "f32"), (512, 1024, 512, 40, "bf16"),
                                                          # wide rows at batch 1: gated store with a cross-wave sum
                                                          # (hidden 4096) and with rows served in pairs (hidden 5120; the 3072-wide down projection)
-                                                         (5120, 1024, 512, 1, "bf16"), (4096, 3072, 512, 1, "f32")])
+                                                         (5120, 1024, 512, 1, "bf16"), (4096, 3072, 512, 1, "f32"),
+                                                         # intermediate rows wider than 16384 columns at batch 1: gate and up in
+                                                         # one launch, silu(gate) * up formed where the row is rotated
+                                                         (3072, 16896, 512, 1, "bf16"), (2560, 16896, 256, 1, "f32")])
 def test_mlp_block_matches_oracle(tq, oracle, shared, hidden, inter, bs, batch, x_dt):
     hip = _Hip()
     o = oracle
@@ -156,3 +159,56 @@ def test_five_bit_dual_rotation_still_dequantise_only(tq, oracle):
     with pytest.raises(RuntimeError):
         layer.forward(np.zeros((1, 128), np.float32))
     layer.close()
+
+
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("outs,in_f,bs,x_dt", [((640, 128, 131), 5120, 512, "bf16"),     # q, k, v: rows served in pairs
+                                                 ((1100, 1000), 4096, 512, "f32"),         # gate, up: two slabs
+                                                 ((300, 40, 7), 3072, 256, "f16"),
+                                                 ((700, 300), 8192, 512, "bf16"),          # four slabs (dual: old tables)
+                                                 ((257, 255), 2048, 512, "bf16"),          # one slab: shared rotation runs them one by one
+                                                 ((96, 64), 18944, 512, "bf16")])          # too wide to share a launch
+def test_forward_group_equals_single_forwards(tq, oracle, shared, outs, in_f, bs, x_dt):
+    """tq_linear_forward_group: two or three layers on the same activation row.  Bit-identical to one
+    tq_linear_forward per layer whether the layers share a launch or not, and within the fp32 tolerance
+    of the oracle."""
+    hip = _Hip()
+    layers, dense = [], []
+    for j, out_f in enumerate(outs):
+        layer, w = _layer(tq, oracle, out_f, in_f, bs, shared, seed=50 + j)
+        layers.append(layer); dense.append(w)
+    x32 = np.random.default_rng(9).standard_normal((1, in_f)).astype(np.float32)
+    if x_dt == "bf16":
+        xbits = oracle.f32_to_bf16_bits(x32); xin = oracle.bf16_bits_to_f32(xbits); xarg, xcode = xbits, tq.BF16
+    elif x_dt == "f16":
+        xarg = x32.astype(np.float16); xin = xarg.astype(np.float32); xcode = tq.F16
+    else:
+        xarg, xin, xcode = x32, x32, tq.F32
+    dx = hip.upload(xarg)
+    ys_group = [hip.alloc(o * 4) for o in outs]
+    ys_single = [hip.alloc(o * 4) for o in outs]
+    for _ in range(2):                                   # twice: nothing stale between calls
+        tq.forward_group_device(layers, dx, xcode, ys_group, tq.F32)
+    for layer, yp in zip(layers, ys_single):
+        layer.forward_device(dx, xcode, 1, yp, tq.F32)
+    for j, o in enumerate(outs):
+        yg = hip.download(ys_group[j], (1, o), np.float32)
+        y1 = hip.download(ys_single[j], (1, o), np.float32)
+        assert np.array_equal(yg, y1)
+        assert _rel(yg, xin @ dense[j].T) < 1e-3
+    hip.free(dx, *ys_group, *ys_single)
+    for layer in layers:
+        layer.close()
+
+
+def test_forward_group_rejects_bad_arguments(tq, oracle):
+    layer, _ = _layer(tq, oracle, 64, 512, 256, True, seed=3)
+    other, _ = _layer(tq, oracle, 64, 1024, 256, True, seed=4)
+    hip = _Hip()
+    dx = hip.upload(np.zeros((1, 1024), np.float32)); dy = hip.alloc(64 * 4)
+    with pytest.raises(RuntimeError):
+        tq.forward_group_device([layer, other], dx, tq.F32, [dy, dy], tq.F32)      # different in_features
+    with pytest.raises(RuntimeError):
+        tq.forward_group_device([layer] * 4, dx, tq.F32, [dy] * 4, tq.F32)         # more than three layers
+    hip.free(dx, dy)
+    layer.close(); other.close()

@@ -53,6 +53,8 @@ def lib():
             getattr(L, name).argtypes = [C.c_void_p]
         L.tq_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
         L.tq_linear_forward_host.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]
+        L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int,
+                                              C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
         L.tq_linear_dequantize.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.tq_linear_dequantize_host.argtypes = [C.c_void_p, _f32p]
         L.tq_linear_free.argtypes = [C.c_void_p]
@@ -187,6 +189,17 @@ class TurboQuantMLP:
             self.close()
         except Exception:
             pass
+
+
+def forward_group_device(layers, x_ptr, x_dtype, y_ptrs, y_dtype, stream=None):
+    """Two or three TurboQuantLinear layers applied to the same activation row on raw device pointers
+    (q, k, v or gate, up of a decoder layer): one kernel launch where the layers allow it, the same
+    results as one forward_device call per layer."""
+    n = len(layers)
+    hs = (C.c_void_p * n)(*[layer._h for layer in layers])
+    ys = (C.c_void_p * n)(*y_ptrs)
+    if lib().tq_linear_forward_group(hs, n, x_ptr, x_dtype, ys, y_dtype, stream) != 0:
+        raise RuntimeError(last_error())
 
 
 def fused_dequant_matmul(qw, primary_codebook, residual_codebook, block_size, x, x_dtype=F32, y_dtype=F32):

@@ -43,8 +43,12 @@ struct LayerView {
 
 // Launchers (tq_gemv.hip, tq_dequant.hip).  All return hipError_t of the launch.
 // gate (optional, fp32 [batch, out]): store silu(gate) * y instead of y.
+// x_gate (optional, fp32 [in], batch 1, x fp32): the layer is applied to silu(x_gate) * x; only where
+// gemv_x_gate_supported() says so (the product is formed by the kernel that rotates the row).
 hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch,
-                       void* y, int y_dtype, int num_cus, hipStream_t stream, const float* gate = nullptr);
+                       void* y, int y_dtype, int num_cus, hipStream_t stream, const float* gate = nullptr,
+                       const float* x_gate = nullptr);
+bool gemv_x_gate_supported(const LayerView& L);
 // out[i] = silu(gate[i]) * up[i] over n fp32 values, written as out_dtype (gated MLP, batched path).
 hipError_t launch_silu_mul(const float* gate, const float* up, void* out, int out_dtype, size_t n, hipStream_t stream);
 hipError_t launch_combine_planes5(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,

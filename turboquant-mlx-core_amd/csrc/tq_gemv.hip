@@ -334,7 +334,10 @@ __global__ __launch_bounds__(MAXT) void tq_gemv_kernel(GemvArgs a) {
 // One wave per 512-column tile (blocks of at most 512 columns).  Rows wider than 16384 columns run one
 // workgroup per CU whose waves would otherwise each rotate a slab of the row on their own, the same
 // work on every CU, which took a quarter of the kernel's time.
+// x_gate (optional, x fp32): the row is silu(x_gate) * x, the activation of a gated MLP block, formed here
+// in fp32 with the expression of apply_gate.
 __global__ __launch_bounds__(256) void tq_rotate_row_kernel(const void* __restrict__ x, int x_dtype,
+                                                            const float* __restrict__ x_gate,
                                                             float* __restrict__ out, int cols, uint32_t seed0,
                                                             uint32_t seed1, uint32_t bs) {
     const int lane = threadIdx.x & (kWave - 1);
@@ -342,7 +345,16 @@ __global__ __launch_bounds__(256) void tq_rotate_row_kernel(const void* __restri
     if (tile0 >= cols) return;
     const int col = tile0 + lane * 8;
     const bool active = col < cols;
-    const TileRaw raw = load_tile_raw(x, x_dtype, 0, active ? col : 0);
+    TileRaw raw = load_tile_raw(x, x_dtype, 0, active ? col : 0);
+    if (x_gate) {                                           // wave-uniform; x is fp32 here
+        const float4* gp = reinterpret_cast<const float4*>(x_gate + (active ? col : 0));
+        const float4 g0 = gp[0], g1 = gp[1];
+        const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        uint32_t* w[8] = {&raw.a.x, &raw.a.y, &raw.a.z, &raw.a.w, &raw.b.x, &raw.b.y, &raw.b.z, &raw.b.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            *w[j] = __builtin_bit_cast(uint32_t, gv[j] / (1.0f + expf(-gv[j])) * __builtin_bit_cast(float, *w[j]));
+    }
     float v[8];
     rotate_tile(raw, x_dtype, col, active, blockIdx.y ? seed1 : seed0, bs, lane, v);
     if (active) {
@@ -397,7 +409,7 @@ static void pre_rotate(GemvArgs& a, hipStream_t stream) {
     if (!L.xrot_work || L.block_size > (uint32_t)kTile || L.in_features % 8 != 0) return;
     const int tiles = (L.in_features + kTile - 1) / kTile;
     hipLaunchKernelGGL(tq_rotate_row_kernel, dim3((tiles + 3) / 4, L.mode == kDual ? 2 : 1), dim3(256), 0, stream,
-                       a.x, a.x_dtype, L.xrot_work, L.in_features, L.seed_primary, L.seed_residual, L.block_size);
+                       a.x, a.x_dtype, a.x_gate, L.xrot_work, L.in_features, L.seed_primary, L.seed_residual, L.block_size);
     a.x = L.xrot_work;
     a.x_dtype = kF32;
     a.pre_rotated = 1;
@@ -442,11 +454,19 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
     return hipSuccess;
 }
 
+// silu(x_gate) * x can be formed on the way where the row goes through tq_rotate_row_kernel.
+bool gemv_x_gate_supported(const LayerView& L) {
+    return L.xrot_work && L.block_size <= (uint32_t)kTile && L.in_features > 8 * kSlab && L.in_features % 8 == 0 &&
+           (L.mode == kSharedLut || L.mode == kDual || L.mode == kPrimaryOnly);
+}
+
 hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch,
-                       void* y, int y_dtype, int num_cus, hipStream_t stream, const float* gate) {
+                       void* y, int y_dtype, int num_cus, hipStream_t stream, const float* gate, const float* x_gate) {
+    if (x_gate && (batch != 1 || x_dtype != kF32 || !gemv_x_gate_supported(L))) return hipErrorInvalidValue;
     GemvArgs a{};
     a.L = L;
     a.gate = gate;
+    a.x_gate = x_gate;
     a.x = x; a.y = y; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
     a.out_scale = L.inv_scale * L.inv_sqrt_bs;
     switch (L.mode) {

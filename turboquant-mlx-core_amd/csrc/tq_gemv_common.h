@@ -20,6 +20,7 @@ struct GemvArgs {
     int rows_q, rows_rem;   // rows per row range, and how many ranges hold one more
     int w_inv;       // (w * w_inv) >> 8 == w / W
     int pre_rotated; // narrow kernel: x holds fp32 rotated activations (second rotation in_features further on)
+    const float* x_gate;  // optional fp32 [in]: the row to multiply is silu(x_gate) * x (x fp32; rows wider than 16384 columns)
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -186,5 +187,8 @@ __device__ __forceinline__ int stage_index(int col_in_slab) {
 // activations built once per CU.  `a` as for the narrow kernel (x, y, gate already at the batch row).
 bool gemv_wide_supported(const LayerView& L, int num_cus, bool pre_rotated = false);
 hipError_t launch_gemv_wide(const GemvArgs& a, int num_cus, hipStream_t stream);
+// Two or three layers of equal width and mode reading the same activation row, one launch.
+bool gemv_wide_group_supported(const LayerView* Ls, int n, int num_cus);
+hipError_t launch_gemv_wide_group(const GemvArgs* as, int n, int num_cus, hipStream_t stream);
 
 }  // namespace tq

@@ -121,8 +121,9 @@ __device__ __forceinline__ void take_from_image(const float* image, int lane, in
 // PT (nibble planes): the table is indexed by a whole byte of the plane and an entry holds the
 // centroids of both its nibbles, rounded to fp16: one table read and two mixed-precision FMAs
 // (v_fma_mix_f32) per byte instead of two reads, two permutes and two FMAs.  64 KB per plane.
+// block: index of the workgroup among those of this layer (a launch may serve several layers).
 template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false>
-__global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
+__device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     static_assert(!PT || MODE != kSharedLut, "pair tables serve the nibble planes");
     constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;   // decode tables
     static_assert(!PRE || (!PAIR && !DYN && MODE != kDual && TILES == 1), "pre-rotated rows: plain slab streams");
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
 
     // Contiguous row range of this stream (DYN: of the workgroup): rows_q rows, one more for the
     // first rows_rem ranges.
-    const int gs = DYN ? (int)blockIdx.x : (int)blockIdx.x * a.S + stream;
+    const int gs = DYN ? block : block * a.S + stream;
     const int r_begin = gs * a.rows_q + (gs < a.rows_rem ? gs : a.rows_rem);
     const int r_end = r_begin + a.rows_q + (gs < a.rows_rem ? 1 : 0);
     const int r_base = r_begin < out ? r_begin : out - 1;
@@ -420,6 +421,25 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
     if (it0 < a.iters) consume(0, r_begin + it0 * V, it0);
 }
 
+template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false>
+__global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
+    wide_body<MODE, R, TILES, PAIR, DYN, PRE, PT>(a, (int)blockIdx.x);
+}
+
+// Two or three layers that read the same activation row (q, k, v or gate, up of a decoder layer),
+// one launch: the workgroups are shared out over the layers by rows, each workgroup serves one
+// layer with that layer's seeds, tables and row ranges.  One start of the kernel instead of three.
+struct GemvGroup {
+    GemvArgs a[3];
+    int first[4];          // layer j owns workgroups first[j] .. first[j + 1] - 1
+};
+template <int MODE, int R, bool PAIR, bool PT>
+__global__ __launch_bounds__(1024) void tq_gemv_wide_group_kernel(GemvGroup g) {
+    const int b = (int)blockIdx.x;
+    const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
+    wide_body<MODE, R, 1, PAIR, false, false, PT>(g.a[j], b - g.first[j]);
+}
+
 template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false, bool PT = false>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
     constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
@@ -502,7 +522,109 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
                                         : launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
 }
 
+template <int MODE, int R, bool PAIR, bool PT>
+hipError_t launch_group_one(const GemvGroup& g, int grid, int threads, size_t lds, hipStream_t stream) {
+    auto* kernel = tq_gemv_wide_group_kernel<MODE, R, PAIR, PT>;
+    static bool asked[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || !asked[dev]) {
+        constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kRegion + kPartialBytes +
+                                    ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float));
+        if (e != hipSuccess) return e;
+        if (dev >= 0 && dev < 64) asked[dev] = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, g);
+    return hipGetLastError();
+}
+
+template <int MODE, bool PAIR, bool PT>
+hipError_t launch_group_mode(GemvGroup& g, int n, int num_cus, hipStream_t stream) {
+    const int in = g.a[0].L.in_features;
+    const int slabs = (in / kChunk + kWave - 1) / kWave;
+    const int W = PAIR ? in / (kSlab / 2) : (MODE == kDual ? 2 * slabs : slabs);
+    const int S = 16 / W;
+    const int threads = W * S * kWave;
+    long long total = 0;
+    for (int j = 0; j < n; ++j) total += g.a[j].L.out_features;
+    // Workgroups per layer in proportion to its rows (the layers have rows of equal width).
+    int blocks[3] = {0, 0, 0}, used = 0;
+    for (int j = 0; j < n; ++j) {
+        blocks[j] = (int)((long long)num_cus * g.a[j].L.out_features / total);
+        if (blocks[j] < 1) blocks[j] = 1;
+        used += blocks[j];
+    }
+    for (int j = 0; used < num_cus; j = (j + 1) % n) { ++blocks[j]; ++used; }
+    for (int j = 0; used > num_cus; j = (j + 1) % n) if (blocks[j] > 1) { --blocks[j]; --used; }
+    const int per_r = PAIR ? 2 : 1;
+    int min_rows = 1 << 30;
+    for (int j = 0; j < n; ++j) {
+        GemvArgs& a = g.a[j];
+        a.chunks = in / kChunk;
+        a.W = W; a.S = S;
+        a.img_cols = slabs * kSlab;
+        a.pre_rotated = 0;
+        const int ts = blocks[j] * S;
+        a.rows_q = a.L.out_features / ts;
+        a.rows_rem = a.L.out_features % ts;
+        a.w_inv = (256 + W - 1) / W;
+        const int max_rows = a.rows_q + (a.rows_rem ? 1 : 0);
+        if (max_rows < min_rows) min_rows = max_rows;
+    }
+    const int R = (MODE != kSharedLut && min_rows >= 4) ? 4 : min_rows >= 2 * per_r ? 2 : 1;
+    g.first[0] = 0;
+    for (int j = 0; j < 3; ++j) g.first[j + 1] = g.first[j] + (j < n ? blocks[j] : 0);
+    for (int j = n; j < 3; ++j) g.first[j + 1] = 1 << 30;        // no workgroup reaches an unused slot
+    for (int j = n; j < 3; ++j) g.first[j] = 1 << 30;
+    for (int j = 0; j < n; ++j) {
+        const int max_rows = g.a[j].rows_q + (g.a[j].rows_rem ? 1 : 0);
+        g.a[j].iters = (max_rows + R * per_r - 1) / (R * per_r);
+    }
+    constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
+    const size_t lds = (size_t)kRegion + kPartialBytes + (size_t)slabs * kSlab * sizeof(float);
+    if constexpr (MODE != kSharedLut) {
+        if (R == 4) return launch_group_one<MODE, 4, PAIR, PT>(g, used, threads, lds, stream);
+    }
+    if (R == 2) return launch_group_one<MODE, 2, PAIR, PT>(g, used, threads, lds, stream);
+    return launch_group_one<MODE, 1, PAIR, PT>(g, used, threads, lds, stream);
+}
+
 }  // namespace
+
+// Layers that can share a launch: two or three, same mode (shared or dual rotation), same width,
+// each fit for the kernel on its own, rows of more than one wave (no group counter) and one
+// activation tile per wave.
+bool gemv_wide_group_supported(const LayerView* Ls, int n, int num_cus) {
+    if (n < 2 || n > 3 || num_cus < n) return false;
+    const LayerView& L0 = Ls[0];
+    if (L0.mode != kSharedLut && L0.mode != kDual) return false;
+    const int slabs = (L0.in_features / kChunk + kWave - 1) / kWave;
+    const int W = wants_pairs(L0) ? L0.in_features / (kSlab / 2) : (L0.mode == kDual ? 2 * slabs : slabs);
+    if (W < 2 || W > 16) return false;
+    const int threads = W * (16 / W) * kWave;
+    if ((L0.in_features + kTile - 1) / kTile > threads / kWave) return false;
+    for (int j = 0; j < n; ++j) {
+        if (Ls[j].mode != L0.mode || Ls[j].in_features != L0.in_features) return false;
+        if (!gemv_wide_supported(Ls[j], 1, false)) return false;      // (1 CU: the strictest bound on a stream's share)
+    }
+    return true;
+}
+
+// as[j]: x, y, types, gate and out_scale of layer j set by the caller (same x for all).
+hipError_t launch_gemv_wide_group(const GemvArgs* as, int n, int num_cus, hipStream_t stream) {
+    GemvGroup g{};
+    for (int j = 0; j < n; ++j) g.a[j] = as[j];
+    const LayerView& L = g.a[0].L;
+    const int slabs = (L.in_features / kChunk + kWave - 1) / kWave;
+    if (L.mode == kSharedLut)
+        return wants_pairs(L) ? launch_group_mode<kSharedLut, true, false>(g, n, num_cus, stream)
+                              : launch_group_mode<kSharedLut, false, false>(g, n, num_cus, stream);
+    return slabs <= kPairDualSlabs ? launch_group_mode<kDual, false, true>(g, n, num_cus, stream)
+                                   : launch_group_mode<kDual, false, false>(g, n, num_cus, stream);
+}
 
 // One batch row, blocks of at most 512 columns, per-stream share of the plane below 2 GB.
 // Shared rotation and primary only: rows of 1 to 8 slabs, or (shared rotation) of an odd number,

@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "tq_device.h"
+#include "tq_gemv_common.h"
 
 namespace {
 thread_local std::string g_last_error;
@@ -326,6 +327,39 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
     } catch (...) { set_error("tq_linear_forward: exception"); return 1; }
 }
 
+int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int x_dtype,
+                            void* const* y_devs, int y_dtype, void* stream) {
+    try {
+        if (!hs || !x_dev || !y_devs || n < 1 || n > 3) { set_error("tq_linear_forward_group: bad arguments (1 to 3 layers)"); return 1; }
+        if (!dtype_valid(x_dtype) || !dtype_valid(y_dtype)) { set_error("tq_linear_forward_group: bad dtype"); return 1; }
+        tq::LayerView views[3];
+        bool plain = true;
+        for (int j = 0; j < n; ++j) {
+            if (!hs[j] || !y_devs[j]) { set_error("tq_linear_forward_group: NULL layer or output"); return 1; }
+            if (hs[j]->view.mode >= tq::kShared5 && !hs[j]->has_fwd_view) plain = false;
+            views[j] = hs[j]->has_fwd_view ? hs[j]->fwd_view : hs[j]->view;
+            if (views[j].in_features != views[0].in_features) {
+                set_error("tq_linear_forward_group: the layers must have the same in_features"); return 1;
+            }
+        }
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        if (plain && tq::gemv_wide_group_supported(views, n, device_cu_count())) {
+            tq::GemvArgs as[3] = {};
+            for (int j = 0; j < n; ++j) {
+                as[j].L = views[j];
+                as[j].x = x_dev; as[j].y = y_devs[j];
+                as[j].x_dtype = x_dtype; as[j].y_dtype = y_dtype;
+                as[j].out_scale = views[j].inv_scale * views[j].inv_sqrt_bs;
+                as[j].gate = nullptr;
+            }
+            return hip_ok(tq::launch_gemv_wide_group(as, n, device_cu_count(), st), "tq_gemv group launch") ? 0 : 1;
+        }
+        for (int j = 0; j < n; ++j)
+            if (forward_impl(hs[j], x_dev, x_dtype, 1, y_devs[j], y_dtype, st, nullptr) != 0) return 1;
+        return 0;
+    } catch (...) { set_error("tq_linear_forward_group: exception"); return 1; }
+}
+
 int tq_linear_forward_host(tq_linear_t h, const void* x_host, int x_dtype, int batch,
                            void* y_host, int y_dtype) {
     try {
@@ -459,6 +493,26 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
         }
         hipStream_t st = static_cast<hipStream_t>(stream);
         const size_t n = (size_t)batch * m->gate->view.out_features;
+        if (batch == 1 && !m->gate->has_fwd_view && !m->up->has_fwd_view && !m->down->has_fwd_view &&
+            m->gate->view.mode < tq::kShared5 && m->up->view.mode < tq::kShared5 && m->down->view.mode < tq::kShared5) {
+            // One row, gate and up of equal width and mode, an intermediate row wider than 16384 columns:
+            // gate and up share a launch, and silu(gate) * up is formed by the kernel that rotates the
+            // row for the down projection: three launches and one kernel start less than below.
+            const tq::LayerView pair[2] = {m->gate->view, m->up->view};
+            if (tq::gemv_wide_group_supported(pair, 2, device_cu_count()) && tq::gemv_x_gate_supported(m->down->view)) {
+                tq::GemvArgs as[2] = {};
+                float* outs[2] = {m->d_gate, m->d_up};
+                for (int j = 0; j < 2; ++j) {
+                    as[j].L = pair[j];
+                    as[j].x = x_dev; as[j].y = outs[j];
+                    as[j].x_dtype = x_dtype; as[j].y_dtype = tq::kF32;
+                    as[j].out_scale = pair[j].inv_scale * pair[j].inv_sqrt_bs;
+                }
+                if (!hip_ok(tq::launch_gemv_wide_group(as, 2, device_cu_count(), st), "tq_gemv group launch")) return 1;
+                return hip_ok(tq::launch_gemv(m->down->view, m->d_up, tq::kF32, 1, y_dev, y_dtype, device_cu_count(), st,
+                                              nullptr, m->d_gate), "tq_gemv launch") ? 0 : 1;
+            }
+        }
         if (batch == 1 || x_dtype == tq::kF32) {
             // decode: three launches, the SiLU gate folded into the store of the up projection
             if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
