@@ -426,28 +426,29 @@ def main():
     import ctypes as C
     by = {n_: h for n_, _, _, h in layers}
     out_of = {n_: o_ for n_, o_, _, _ in layers}
-    x1 = {i_: torch.randn(1, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
-    y1 = {n_: torch.empty(1, out_of[n_], device="cuda", dtype=torch.float32) for n_ in by}
-    L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int,
+    L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
                                           C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
+    for batch in (1, 4, 8):
+        xg = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
+        yg = {n_: torch.empty(batch, out_of[n_], device="cuda", dtype=torch.float32) for n_ in by}
 
-    def group(names, x, s):
-        hs = (C.c_void_p * len(names))(*[by[n_] for n_ in names])
-        yp = (C.c_void_p * len(names))(*[y1[n_].data_ptr() for n_ in names])
-        if L.tq_linear_forward_group(hs, len(names), x.data_ptr(), tq.BF16, yp, tq.F32, s) != 0:
-            raise RuntimeError(tq.last_error())
+        def group(names, x, s):
+            hs = (C.c_void_p * len(names))(*[by[n_] for n_ in names])
+            yp = (C.c_void_p * len(names))(*[yg[n_].data_ptr() for n_ in names])
+            if L.tq_linear_forward_group(hs, len(names), x.data_ptr(), tq.BF16, batch, yp, tq.F32, s) != 0:
+                raise RuntimeError(tq.last_error())
 
-    def grouped_step(s):
-        group(("q", "k", "v"), x1[5120], s)
-        group(("o",), x1[5120], s)
-        group(("gate", "up"), x1[5120], s)
-        group(("down",), x1[27648], s)
-    us_g = time_graph_fn(torch, grouped_step, max(args.steps // 10, 10), 2) * 1e6
-    Bg = sum(algorithmic_bytes(o_, i_, 1, 2, 4) for _, o_, i_, _ in layers)
-    extra["decoder_layer_projections_32b_bs1_grouped_launches"] = {
-        "us_per_layer_all_7_projections": us_g, "algorithmic_bytes": Bg,
-        "hbm_frac": Bg / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBS,
-        "launches": "q+k+v, o, gate+up, rotation of the down projection's row, down"}
+        def grouped_step(s):
+            group(("q", "k", "v"), xg[5120], s)
+            group(("o",), xg[5120], s)
+            group(("gate", "up"), xg[5120], s)
+            group(("down",), xg[27648], s)
+        us_g = time_graph_fn(torch, grouped_step, max(args.steps // 10, 10), 2) * 1e6
+        Bg = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
+        extra[f"decoder_layer_projections_32b_bs{batch}_grouped_launches"] = {
+            "us_per_layer_all_7_projections": us_g, "algorithmic_bytes": Bg,
+            "hbm_frac": Bg / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "calls": "q+k+v, o, gate+up, down through tq_linear_forward_group"}
     for _, _, _, h in layers:
         L.tq_linear_free(h)
     finish(args, torch, extra, result)

@@ -98,13 +98,14 @@ int tq_linear_forward(tq_linear_t layer, const void* x_dev, int x_dtype, int bat
                       void* y_dev, int y_dtype, void* stream);
 
 /**
- * Two or three layers applied to the SAME activation row (batch 1): y_devs[j][out_j] = x[in] . W_j^T,
- * e.g. the q, k, v or the gate, up projections of a decoder layer.  Results are identical to n calls of
- * tq_linear_forward; layers of equal width and mode (shared or dual rotation, blocks <= 512, more
- * than 2048 columns for shared rotation) share one kernel launch, anything else is run one after the
- * other.  No counterpart in the reference, whose forward is per layer (include/turboquant/linear.h:21-22).
+ * One to three layers applied to the SAME activations: y_devs[j][batch, out_j] = x[batch, in] . W_j^T,
+ * e.g. the q, k, v or the gate, up projections of a decoder layer.  Layers of equal width and mode share
+ * their kernel launches where the kernels allow it (batch 1: shared or dual rotation, blocks <= 512, more
+ * than 2048 columns for shared rotation; 2..15 rows of 16-bit activations: shared rotation, blocks <= 512);
+ * anything else is run one layer after the other.  Results are identical to n calls of tq_linear_forward.
+ * No counterpart in the reference, whose forward is per layer (include/turboquant/linear.h:21-22).
  */
-int tq_linear_forward_group(const tq_linear_t* layers, int n, const void* x_dev, int x_dtype,
+int tq_linear_forward_group(const tq_linear_t* layers, int n, const void* x_dev, int x_dtype, int batch,
                             void* const* y_devs, int y_dtype, void* stream);
 
 /** Same with host buffers (copies in, runs, copies out, synchronises). */

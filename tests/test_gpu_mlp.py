@@ -188,7 +188,7 @@ def test_forward_group_equals_single_forwards(tq, oracle, shared, outs, in_f, bs
     ys_group = [hip.alloc(o * 4) for o in outs]
     ys_single = [hip.alloc(o * 4) for o in outs]
     for _ in range(2):                                   # twice: nothing stale between calls
-        tq.forward_group_device(layers, dx, xcode, ys_group, tq.F32)
+        tq.forward_group_device(layers, dx, xcode, 1, ys_group, tq.F32)
     for layer, yp in zip(layers, ys_single):
         layer.forward_device(dx, xcode, 1, yp, tq.F32)
     for j, o in enumerate(outs):
@@ -207,8 +207,43 @@ def test_forward_group_rejects_bad_arguments(tq, oracle):
     hip = _Hip()
     dx = hip.upload(np.zeros((1, 1024), np.float32)); dy = hip.alloc(64 * 4)
     with pytest.raises(RuntimeError):
-        tq.forward_group_device([layer, other], dx, tq.F32, [dy, dy], tq.F32)      # different in_features
+        tq.forward_group_device([layer, other], dx, tq.F32, 1, [dy, dy], tq.F32)   # different in_features
     with pytest.raises(RuntimeError):
-        tq.forward_group_device([layer] * 4, dx, tq.F32, [dy] * 4, tq.F32)         # more than three layers
+        tq.forward_group_device([layer] * 4, dx, tq.F32, 1, [dy] * 4, tq.F32)      # more than three layers
+    with pytest.raises(RuntimeError):
+        tq.forward_group_device([other], dx, tq.F32, 0, [dy], tq.F32)              # no rows
     hip.free(dx, dy)
     layer.close(); other.close()
+
+
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("batch", [2, 5, 8, 15])
+@pytest.mark.parametrize("outs,in_f,bs", [((640, 128, 131), 5120, 512), ((1100, 1000), 4096, 256), ((50, 33), 1024, 512),
+                                          ((40, 24), 2048, 1024)])
+def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):
+    """tq_linear_forward_group with 2..15 rows of bf16 activations: shared-rotation layers with blocks of
+    at most 512 columns share the matrix-core kernel and its reduction, everything else (dual rotation,
+    larger blocks) is run layer by layer.  Bit-identical to separate calls either way; bf16 tolerance
+    against the dense product."""
+    hip = _Hip()
+    layers, dense = [], []
+    for j, out_f in enumerate(outs):
+        layer, w = _layer(tq, oracle, out_f, in_f, bs, shared, seed=70 + j)
+        layers.append(layer); dense.append(w)
+    xbits = oracle.f32_to_bf16_bits(np.random.default_rng(batch).standard_normal((batch, in_f)).astype(np.float32))
+    xin = oracle.bf16_bits_to_f32(xbits)
+    dx = hip.upload(xbits)
+    ys_group = [hip.alloc(batch * o * 4) for o in outs]
+    ys_single = [hip.alloc(batch * o * 4) for o in outs]
+    for _ in range(2):
+        tq.forward_group_device(layers, dx, tq.BF16, batch, ys_group, tq.F32)
+    for layer, yp in zip(layers, ys_single):
+        layer.forward_device(dx, tq.BF16, batch, yp, tq.F32)
+    for j, o in enumerate(outs):
+        yg = hip.download(ys_group[j], (batch, o), np.float32)
+        y1 = hip.download(ys_single[j], (batch, o), np.float32)
+        assert np.array_equal(yg, y1)
+        assert _rel(yg, xin @ dense[j].T) < 5e-3
+    hip.free(dx, *ys_group, *ys_single)
+    for layer in layers:
+        layer.close()

@@ -53,7 +53,7 @@ def lib():
             getattr(L, name).argtypes = [C.c_void_p]
         L.tq_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
         L.tq_linear_forward_host.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]
-        L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int,
+        L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
                                               C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
         L.tq_linear_dequantize.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.tq_linear_dequantize_host.argtypes = [C.c_void_p, _f32p]
@@ -191,14 +191,14 @@ class TurboQuantMLP:
             pass
 
 
-def forward_group_device(layers, x_ptr, x_dtype, y_ptrs, y_dtype, stream=None):
-    """Two or three TurboQuantLinear layers applied to the same activation row on raw device pointers
-    (q, k, v or gate, up of a decoder layer): one kernel launch where the layers allow it, the same
-    results as one forward_device call per layer."""
+def forward_group_device(layers, x_ptr, x_dtype, batch, y_ptrs, y_dtype, stream=None):
+    """One to three TurboQuantLinear layers applied to the same activations on raw device pointers
+    (q, k, v or gate, up of a decoder layer): shared kernel launches where the layers allow it, the
+    same results as one forward_device call per layer."""
     n = len(layers)
     hs = (C.c_void_p * n)(*[layer._h for layer in layers])
     ys = (C.c_void_p * n)(*y_ptrs)
-    if lib().tq_linear_forward_group(hs, n, x_ptr, x_dtype, ys, y_dtype, stream) != 0:
+    if lib().tq_linear_forward_group(hs, n, x_ptr, x_dtype, batch, ys, y_dtype, stream) != 0:
         raise RuntimeError(last_error())
 
 

@@ -67,6 +67,10 @@ bool skinny_supported(const LayerView& L, int x_dtype, int batch);
 size_t skinny_partial_bytes(const LayerView& L);
 hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                          void* xt_workspace, float* partial, int num_cus, hipStream_t stream);
+// Two or three shared-rotation layers of equal width on the same activation rows: both launches shared.
+bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, int num_cus);
+hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
+                               int y_dtype, float* const* partials, int num_cus, hipStream_t stream);
 hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t seed,
                       uint32_t block_size, float inv_sqrt_bs, int inverse, hipStream_t stream);
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream);

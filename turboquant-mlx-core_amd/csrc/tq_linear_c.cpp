@@ -327,11 +327,11 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
     } catch (...) { set_error("tq_linear_forward: exception"); return 1; }
 }
 
-int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int x_dtype,
+int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int x_dtype, int batch,
                             void* const* y_devs, int y_dtype, void* stream) {
     try {
         if (!hs || !x_dev || !y_devs || n < 1 || n > 3) { set_error("tq_linear_forward_group: bad arguments (1 to 3 layers)"); return 1; }
-        if (!dtype_valid(x_dtype) || !dtype_valid(y_dtype)) { set_error("tq_linear_forward_group: bad dtype"); return 1; }
+        if (batch <= 0 || !dtype_valid(x_dtype) || !dtype_valid(y_dtype)) { set_error("tq_linear_forward_group: bad batch or dtype"); return 1; }
         tq::LayerView views[3];
         bool plain = true;
         for (int j = 0; j < n; ++j) {
@@ -343,7 +343,7 @@ int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int
             }
         }
         hipStream_t st = static_cast<hipStream_t>(stream);
-        if (plain && tq::gemv_wide_group_supported(views, n, device_cu_count())) {
+        if (plain && batch == 1 && tq::gemv_wide_group_supported(views, n, device_cu_count())) {
             tq::GemvArgs as[3] = {};
             for (int j = 0; j < n; ++j) {
                 as[j].L = views[j];
@@ -354,8 +354,19 @@ int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int
             }
             return hip_ok(tq::launch_gemv_wide_group(as, n, device_cu_count(), st), "tq_gemv group launch") ? 0 : 1;
         }
+        if (plain && tq::skinny_group_supported(views, n, x_dtype, batch, device_cu_count())) {
+            // 2..15 rows on the matrix cores; the per-chunk partial products are per layer and allocated
+            // on the first such call (not capturable in a graph), as in tq_linear_forward.
+            float* partials[3] = {nullptr, nullptr, nullptr};
+            for (int j = 0; j < n; ++j) {
+                if (!ensure_stage(&hs[j]->d_partial, &hs[j]->partial_bytes, tq::skinny_partial_bytes(views[j]))) return 1;
+                partials[j] = static_cast<float*>(hs[j]->d_partial);
+            }
+            return hip_ok(tq::launch_skinny_group(views, n, x_dev, x_dtype, batch, y_devs, y_dtype, partials,
+                                                  device_cu_count(), st), "tq_skinny group launch") ? 0 : 1;
+        }
         for (int j = 0; j < n; ++j)
-            if (forward_impl(hs[j], x_dev, x_dtype, 1, y_devs[j], y_dtype, st, nullptr) != 0) return 1;
+            if (forward_impl(hs[j], x_dev, x_dtype, batch, y_devs[j], y_dtype, st, nullptr) != 0) return 1;
         return 0;
     } catch (...) { set_error("tq_linear_forward_group: exception"); return 1; }
 }

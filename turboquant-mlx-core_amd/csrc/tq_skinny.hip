@@ -54,8 +54,10 @@ __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t l
 
 // FUSED: the workgroup rotates the 16 x 512 activations of its chunk itself (blocks of at most 512
 // columns: a block never leaves the chunk), instead of reading tile images a separate kernel wrote.
+// chunk, wg_in_chunk: the 512-column chunk of this workgroup and its index among the workgroups that
+// share the chunk for this layer (a launch may serve several layers).
 template <bool FUSED>
-__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_kernel(SkinnyArgs a) {
+__device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk, const int wg_in_chunk) {
     // table | 16 x 512 bf16 rotated activations (FUSED).  One workgroup of 8 waves per CU: 16 waves
     // gained nothing, and 8 have the registers for two row groups in flight.
     __shared__ __align__(16) char smem[kSkLutBytes + kSkStageBytes];
@@ -64,10 +66,8 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t laneoff = (uint32_t)lane << 2;
 
-    // (grid = chunks x workgroups per chunk; no integer division in the kernel: the waves of a CU
-    // share one scalar unit and a division is a few hundred instructions)
-    const int chunk = blockIdx.x;
-    const int wg_in_chunk = blockIdx.y;
+    // (no integer division in the kernel: the waves of a CU share one scalar unit and a division is a
+    // few hundred instructions)
     const int m = lane & 15, g = lane >> 4;               // A operand: batch row, k group; B operand: weight row, k group
 
     // Row groups of this wave: the groups are dealt out evenly over all waves that share the chunk.
@@ -200,6 +200,25 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         if (grp + 2 < g_end) request(rawA, grp + 2);
         multiply(rawB, grp + 1);
     }
+}
+
+// grid = chunks x workgroups per chunk
+template <bool FUSED>
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_kernel(SkinnyArgs a) {
+    skinny_body<FUSED>(a, (int)blockIdx.x, (int)blockIdx.y);
+}
+
+// Two or three layers of equal width on the same activation rows (q, k, v or gate, up), one launch:
+// the workgroups of a chunk are shared out over the layers by rows (layer j owns blockIdx.y in
+// first[j] .. first[j + 1] - 1).
+struct SkinnyGroup {
+    SkinnyArgs a[3];
+    int first[4];
+};
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_group_kernel(SkinnyGroup g) {
+    const int b = (int)blockIdx.y;
+    const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
+    skinny_body<true>(g.a[j], (int)blockIdx.x, b - g.first[j]);
 }
 
 // Nibble planes (dual rotation, primary only): the same scheme on a plane of two weights per
@@ -347,13 +366,13 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 // columns (wave w takes chunks w, w + 4, ..., eight loads in flight at a time) and add up through
 // LDS: a single thread per output walking all chunks four at a time spent one memory latency per
 // four chunks, 4.5 us for a kernel that moves a few hundred KB.
-__global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __restrict__ partial,
-                                                               const float* __restrict__ norms, void* __restrict__ y,
-                                                               int y_dtype, int batch, int N, int chunks, float out_scale) {
+__device__ __forceinline__ void skinny_reduce_body(const float* __restrict__ partial, const float* __restrict__ norms,
+                                                   void* __restrict__ y, int y_dtype, int N, int chunks,
+                                                   float out_scale, const int block) {
     __shared__ float part[4][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int b = blockIdx.y;
-    const int n = blockIdx.x * 64 + lane;
+    const int n = block * 64 + lane;
     const bool live = n < N;
     const float nrm = live ? norms[n] : 0.0f;
     const float* p = partial + (size_t)b * N + (live ? n : 0);
@@ -373,6 +392,27 @@ __global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __re
         const float t = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
         store_scalar(y, y_dtype, (size_t)b * N + n, t * (out_scale * nrm));
     }
+}
+
+__global__ __launch_bounds__(256) void tq_skinny_reduce_kernel(const float* __restrict__ partial,
+                                                               const float* __restrict__ norms, void* __restrict__ y,
+                                                               int y_dtype, int batch, int N, int chunks, float out_scale) {
+    skinny_reduce_body(partial, norms, y, y_dtype, N, chunks, out_scale, (int)blockIdx.x);
+}
+
+struct SkinnyReduceGroup {
+    const float* partial[3];
+    const float* norms[3];
+    void* y[3];
+    int N[3];
+    float out_scale[3];
+    int first[4];              // layer j owns blockIdx.x in first[j] .. first[j + 1] - 1
+    int y_dtype, chunks;
+};
+__global__ __launch_bounds__(256) void tq_skinny_reduce_group_kernel(SkinnyReduceGroup r) {
+    const int b = (int)blockIdx.x;
+    const int j = b >= r.first[2] ? 2 : (b >= r.first[1] ? 1 : 0);
+    skinny_reduce_body(r.partial[j], r.norms[j], r.y[j], r.y_dtype, r.N[j], r.chunks, r.out_scale[j], b - r.first[j]);
 }
 
 static bool skinny_nibble(const LayerView& L) {
@@ -440,6 +480,70 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     const unsigned blocks = (unsigned)((L.out_features + 63) / 64);
     hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks, batch), dim3(256), 0, stream,
                        partial, L.norms, y, y_dtype, batch, L.out_features, a.chunks, L.inv_scale * L.inv_sqrt_bs);
+    return hipGetLastError();
+}
+
+// Layers that can share the two launches: two or three shared-rotation layers of equal width with
+// blocks of at most 512 columns (the workgroup rotates its chunk itself), 2..15 rows of 16-bit
+// activations, and at least one workgroup per chunk and layer.
+bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, int num_cus) {
+    if (n < 2 || n > 3) return false;
+    for (int j = 0; j < n; ++j) {
+        if (Ls[j].mode != kSharedLut || !Ls[j].packed_combined || Ls[j].block_size > (uint32_t)kSkChunk) return false;
+        if (Ls[j].in_features != Ls[0].in_features || !skinny_supported(Ls[j], x_dtype, batch)) return false;
+    }
+    return num_cus / (Ls[0].in_features / kSkChunk) >= n;
+}
+
+hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
+                               int y_dtype, float* const* partials, int num_cus, hipStream_t stream) {
+    const int K = Ls[0].in_features, chunks = K / kSkChunk;
+    const int total_wgs = num_cus / chunks;                       // workgroups per chunk, all layers together
+    long long rows = 0;
+    for (int j = 0; j < n; ++j) rows += Ls[j].out_features;
+    int wgs[3] = {0, 0, 0}, used = 0;
+    for (int j = 0; j < n; ++j) {
+        wgs[j] = (int)((long long)total_wgs * Ls[j].out_features / rows);
+        if (wgs[j] < 1) wgs[j] = 1;
+        used += wgs[j];
+    }
+    for (int j = 0; used < total_wgs; j = (j + 1) % n) { ++wgs[j]; ++used; }
+    for (int j = 0; used > total_wgs; j = (j + 1) % n) if (wgs[j] > 1) { --wgs[j]; --used; }
+    SkinnyGroup g{};
+    SkinnyReduceGroup r{};
+    g.first[0] = 0; r.first[0] = 0;
+    for (int j = 0; j < 3; ++j) {
+        if (j < n) {
+            const LayerView& L = Ls[j];
+            SkinnyArgs& a = g.a[j];
+            a.x = x; a.x_dtype = x_dtype; a.seed = L.seed_primary; a.block_size = L.block_size;
+            a.xt = nullptr;
+            a.plane = L.packed_combined;
+            a.tables = L.tables;
+            a.partial = partials[j];
+            a.batch = batch; a.N = L.out_features; a.K = K;
+            a.chunks = chunks;
+            a.groups = (L.out_features + 15) / 16;
+            a.wgs_per_chunk = wgs[j];
+            const int workers = wgs[j] * (kSkThreads / 64);
+            a.groups_q = a.groups / workers;
+            a.groups_rem = a.groups % workers;
+            r.partial[j] = partials[j]; r.norms[j] = L.norms; r.y[j] = ys[j]; r.N[j] = L.out_features;
+            r.out_scale[j] = L.inv_scale * L.inv_sqrt_bs;
+            g.first[j + 1] = g.first[j] + wgs[j];
+            r.first[j + 1] = r.first[j] + (L.out_features + 63) / 64;
+        } else {
+            g.first[j] = 1 << 30; g.first[j + 1] = 1 << 30;       // no workgroup reaches an unused slot
+            r.first[j] = 1 << 30; r.first[j + 1] = 1 << 30;
+        }
+    }
+    int reduce_blocks = 0;
+    for (int j = 0; j < n; ++j) reduce_blocks += (Ls[j].out_features + 63) / 64;
+    r.y_dtype = y_dtype; r.chunks = chunks;
+    hipLaunchKernelGGL(tq_skinny_group_kernel, dim3(chunks, used), dim3(kSkThreads), 0, stream, g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(tq_skinny_reduce_group_kernel, dim3(reduce_blocks, batch), dim3(256), 0, stream, r);
     return hipGetLastError();
 }
 
