@@ -532,8 +532,20 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
         }
         // two or more rows of 16-bit activations: matrix-core paths for all three layers (small-batch or
         // prefill kernel), one elementwise kernel, activation handed to the down projection as bf16
-        if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
-        if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_up, tq::kF32, st, nullptr) != 0) return 1;
+        const tq::LayerView both[2] = {m->gate->has_fwd_view ? m->gate->fwd_view : m->gate->view,
+                                       m->up->has_fwd_view ? m->up->fwd_view : m->up->view};
+        const bool plain = !(m->gate->view.mode >= tq::kShared5 && !m->gate->has_fwd_view) &&
+                           !(m->up->view.mode >= tq::kShared5 && !m->up->has_fwd_view);
+        if (plain && tq::skinny_group_supported(both, 2, x_dtype, batch, device_cu_count())) {
+            // gate and up share the small-batch kernel and its reduction (workspaces sized by tq_mlp_create)
+            void* outs[2] = {m->d_gate, m->d_up};
+            float* partials[2] = {static_cast<float*>(m->gate->d_partial), static_cast<float*>(m->up->d_partial)};
+            if (!hip_ok(tq::launch_skinny_group(both, 2, x_dev, x_dtype, batch, outs, tq::kF32, partials,
+                                                device_cu_count(), st), "tq_skinny group launch")) return 1;
+        } else {
+            if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
+            if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_up, tq::kF32, st, nullptr) != 0) return 1;
+        }
         if (!hip_ok(tq::launch_silu_mul(m->d_gate, m->d_up, m->d_act, tq::kBF16, n, st), "silu_mul launch")) return 1;
         return forward_impl(m->down, m->d_act, tq::kBF16, batch, y_dev, y_dtype, st, nullptr);
     } catch (...) { set_error("tq_mlp_forward: exception"); return 1; }
