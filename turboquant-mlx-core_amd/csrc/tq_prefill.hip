@@ -129,19 +129,9 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
     using Stage = PrefillStage<combined>;
 
     for (int plane = 0; plane < kPlanes; ++plane) {
-        // Decode table of this plane -> LDS, one private column per lane, values rounded to bf16.
+        // (second plane: nothing of the first is in flight, and its table has been read for the last time)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        {
-            const int entries = combined ? 256 : 16;
-            const float* src = a.tables + (plane == 0 ? 0 : 16);
-            uint4* dst = reinterpret_cast<uint4*>(smem);
-            for (int i = tid; i < entries * 16; i += kGemmThreads) {
-                const uint32_t v = (uint32_t)float_to_bf16_bits(src[i >> 4]) << 16;
-                dst[i] = make_uint4(v, v, v, v);
-            }
-        }
-
         const char* a_tiles = reinterpret_cast<const char*>(a.xt) +
                               ((size_t)plane * a.m_tiles + m_tile) * (size_t)T * kATile;
         const uint8_t* w_plane = combined ? a.plane0 : (plane == 0 ? a.plane0 : a.plane1);
@@ -299,6 +289,21 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
         load_b(S0, 0);
         load_b(S1, 1);
         load_b(S2, 2);
+        // The table is built while those requests travel.  Its values come through scalar loads (the
+        // same for all lanes; the compiler's waits for vector loads would not know about the requests
+        // above): wave w writes entries 32 w .. 32 w + 31, lane l into bytes 4 l .. of each entry's 256.
+        {
+            constexpr int entries = combined ? 256 : 16;
+            typedef const __attribute__((address_space(4))) float cfloat;
+            cfloat* const src = (cfloat*)(a.tables + (plane == 0 ? 0 : 16));
+            uint32_t* const dst = reinterpret_cast<uint32_t*>(smem) + lane;
+            constexpr int per_wave = (entries + 7) / 8;
+#pragma unroll
+            for (int e = 0; e < per_wave; ++e) {
+                const int entry = wave * per_wave + e;
+                if (entry < entries) dst[entry * 64] = (uint32_t)float_to_bf16_bits(src[entry]) << 16;
+            }
+        }
         asm volatile("s_waitcnt vmcnt(0)"
                      : "+v"(S0.b[0]), "+v"(S0.b[1]), "+v"(S1.b[0]), "+v"(S1.b[1]), "+v"(S2.b[0]), "+v"(S2.b[1])
                      :: "memory");
