@@ -166,6 +166,7 @@ def test_five_bit_dual_rotation_still_dequantise_only(tq, oracle):
                                                  ((1100, 1000), 4096, 512, "f32"),         # gate, up: two slabs
                                                  ((300, 40, 7), 3072, 256, "f16"),
                                                  ((700, 300), 8192, 512, "bf16"),          # four slabs (dual: old tables)
+                                                 ((9000, 7001), 4096, 512, "bf16"),        # many rows per stream (dual: groups of four rows)
                                                  ((257, 255), 2048, 512, "bf16"),          # one slab: shared rotation runs them one by one
                                                  ((96, 64), 18944, 512, "bf16")])          # too wide to share a launch
 def test_forward_group_equals_single_forwards(tq, oracle, shared, outs, in_f, bs, x_dt):
