@@ -158,6 +158,23 @@ def test_forward_batch1_one_slab_rows(tq, oracle, mode, out, inf, bs):
     layer.close()
 
 
+@pytest.mark.parametrize("mode", ["primary_only", "dual"])
+def test_forward_batch1_centroids_outside_fp16_range(tq, oracle, mode):
+    """Codebooks whose values do not fit fp16 (1e5 times the usual ones): the one-row kernel must not
+    use its fp16 centroid pairs for such a layer.  Same packed indices, scaled codebooks: the output is
+    the scaled output, finite, and within the fp32 tolerance of the oracle."""
+    out, inf, bs = 300, 4096, 512
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    big_p = oracle.Codebook(cbp.centroids * np.float32(1e5), cbp.bits)
+    big_r = oracle.Codebook(cbr.centroids * np.float32(1e5), cbr.bits)
+    x = np.random.default_rng(3).standard_normal((1, inf)).astype(np.float32)
+    layer = tq.TurboQuantLinear(inf, out, qw, big_p, big_r, bs)
+    y = layer.forward(x)
+    layer.close()
+    want = oracle.linear_forward(qw, big_p, big_r, bs, x)
+    assert np.isfinite(y).all() and _rel(y, want) < 1e-3
+
+
 @pytest.mark.parametrize("mode", ["shared", "primary_only", "dual"])
 @pytest.mark.parametrize("out,inf,bs", [(600, 27648, 512), (515, 18944, 256), (257, 17408, 512), (40, 20480, 2048)])
 def test_forward_batch1_rows_beyond_16384_columns(tq, oracle, mode, out, inf, bs):

@@ -37,6 +37,8 @@ struct LayerView {
     int mode;
     float inv_scale;                 // 1/sqrt(in), computed on the host as the reference does
     float inv_sqrt_bs;               // 1/sqrt(block_size), host computed
+    int fp16_centroids_ok;           // every centroid fits fp16 with room to spare (the byte-pair tables of the
+                                     // batch-1 kernel hold fp16 values); otherwise fp32 tables are used
     float* xrot_work;                // scratch of 2 * in_features floats (rows wider than 16384 columns: the
                                      // batch-1 path rotates the activations once, in a kernel of its own), or NULL
 };

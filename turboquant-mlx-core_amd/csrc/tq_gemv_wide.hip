@@ -517,9 +517,12 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     const int ntiles = (a.L.in_features + kTile - 1) / kTile;
     const bool two = ntiles > threads / kWave;              // at most two tiles per wave: checked by the caller
     if constexpr (MODE == kSharedLut) return launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
-    else if constexpr (MODE == kPrimaryOnly) return launch_wide_shape<MODE, PAIR, true>(a, grid, threads, R, two, out, stream);
-    else return slabs <= kPairDualSlabs ? launch_wide_shape<MODE, PAIR, true>(a, grid, threads, R, two, out, stream)
-                                        : launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
+    else if constexpr (MODE == kPrimaryOnly)
+        return a.L.fp16_centroids_ok ? launch_wide_shape<MODE, PAIR, true>(a, grid, threads, R, two, out, stream)
+                                     : launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
+    else return (slabs <= kPairDualSlabs && a.L.fp16_centroids_ok)
+                    ? launch_wide_shape<MODE, PAIR, true>(a, grid, threads, R, two, out, stream)
+                    : launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
 }
 
 template <int MODE, int R, bool PAIR, bool PT>
@@ -622,8 +625,10 @@ hipError_t launch_gemv_wide_group(const GemvArgs* as, int n, int num_cus, hipStr
     if (L.mode == kSharedLut)
         return wants_pairs(L) ? launch_group_mode<kSharedLut, true, false>(g, n, num_cus, stream)
                               : launch_group_mode<kSharedLut, false, false>(g, n, num_cus, stream);
-    return slabs <= kPairDualSlabs ? launch_group_mode<kDual, false, true>(g, n, num_cus, stream)
-                                   : launch_group_mode<kDual, false, false>(g, n, num_cus, stream);
+    bool fp16_ok = true;
+    for (int j = 0; j < n; ++j) fp16_ok = fp16_ok && g.a[j].L.fp16_centroids_ok;
+    return (slabs <= kPairDualSlabs && fp16_ok) ? launch_group_mode<kDual, false, true>(g, n, num_cus, stream)
+                                                : launch_group_mode<kDual, false, false>(g, n, num_cus, stream);
 }
 
 // One batch row, blocks of at most 512 columns, per-stream share of the plane below 2 GB.

@@ -239,6 +239,12 @@ tq_linear_t create_impl(int in_features, int out_features,
         }
     }
     v.xrot_work = h->d_xrot;
+    {
+        float big = 0.0f;
+        for (int i = 0; i < np; ++i) big = std::fmax(big, std::fabs(cbp[i]));
+        for (int i = 0; i < nr; ++i) big = std::fmax(big, std::fabs(cbr[i]));
+        v.fp16_centroids_ok = (big < 30000.0f) ? 1 : 0;      // NaN compares false
+    }
     if (fused5) {
         h->fwd_view = v;
         h->fwd_view.mode = tq::kSharedLut;
