@@ -308,3 +308,42 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     yf = layer.forward(x32)
     assert _rel(yf, oracle.linear_forward(qw, cbp, cbr, bs, x32)) < 1e-3
     layer.close()
+
+
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < n:
+        inf = int(rng.choice([64, 96, 128, 384, 512, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 7168, 8192,
+                              9216, 11264, 13312, 16384, 17408, 18944, 24576, 27648, 32768]))
+        divisors = [b for b in (16, 32, 64, 128, 256, 512, 1024, 2048) if inf % b == 0]
+        bs = int(rng.choice(divisors))
+        out = int(rng.integers(1, max(2, min(3000, (6 << 20) // inf))))
+        mode = str(rng.choice(["shared", "dual", "primary_only"]))
+        batch = int(rng.choice([1, 1, 1, 2, 3, 5, 8, 15, 16, 17, 33]))
+        xd = str(rng.choice(["f32", "bf16", "f16"]))
+        cases.append((out, inf, bs, mode, batch, xd))
+    return cases
+
+
+@pytest.mark.parametrize("out,inf,bs,mode,batch,xd", _random_cases(160, 20240611))
+def test_forward_random_configurations(tq, oracle, out, inf, bs, mode, batch, xd):
+    """Whatever kernel a call is routed to (one-workgroup-per-CU, pre-rotated, narrow, small-batch or
+    prefill): the output agrees with the oracle's dense product on the same quantised weights, within
+    1e-3 for fp32 activations and single rows, 5e-3 where bf16 weights are used (2+ rows of 16-bit
+    activations)."""
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode, seed=out + inf)
+    x32 = np.random.default_rng(out * 7 + batch).standard_normal((batch, inf)).astype(np.float32)
+    if xd == "bf16":
+        xarg = oracle.f32_to_bf16_bits(x32); xin = oracle.bf16_bits_to_f32(xarg); code = tq.BF16
+    elif xd == "f16":
+        xarg = x32.astype(np.float16); xin = xarg.astype(np.float32); code = tq.F16
+    else:
+        xarg, xin, code = x32, x32, tq.F32
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    y = layer.forward(xarg, code, tq.F32)
+    layer.close()
+    want = oracle.linear_forward(qw, cbp, cbr, bs, xin)
+    tol = 1e-3 if (xd == "f32" or batch == 1) else 5e-3
+    assert y.shape == (batch, out) and np.isfinite(y).all()
+    assert _rel(y, want) < tol
