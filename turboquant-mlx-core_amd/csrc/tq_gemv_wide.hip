@@ -122,13 +122,17 @@ __device__ __forceinline__ void take_from_image(const float* image, int lane, in
 // centroids of both its nibbles, rounded to fp16: one table read and two mixed-precision FMAs
 // (v_fma_mix_f32) per byte instead of two reads, two permutes and two FMAs.  64 KB per plane.
 // block: index of the workgroup among those of this layer (a launch may serve several layers).
-template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false>
+// BOTH (dual rotation, rows of one slab): a wave decodes both planes of its rows (two rotated
+// activation vectors in registers, one row per group), so the waves need no cross-wave sum and take
+// their rows from the LDS counter like the other one-slab layers.
+template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false, bool BOTH = false>
 __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
+    static_assert(!BOTH || (MODE == kDual && PT && DYN && !PAIR && !PRE && R <= 2), "both planes per wave: dual rotation, pair tables");
     static_assert(!PT || MODE != kSharedLut, "pair tables serve the nibble planes");
     constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;   // decode tables
     static_assert(!PRE || (!PAIR && !DYN && MODE != kDual && TILES == 1), "pre-rotated rows: plain slab streams");
     static_assert(!PAIR || MODE == kSharedLut, "row pairs need the one-byte-per-weight plane");
-    static_assert(!DYN || (!PAIR && MODE != kDual), "the group counter serves one-wave row streams");
+    static_assert(!DYN || (!PAIR && (MODE != kDual || BOTH)), "the group counter serves one-wave row streams");
     constexpr int NS = 2;                           // register ring: one group decoded, one in flight
     constexpr int V = PAIR ? 2 * R : R;             // rows, and sums, per row group
     constexpr int NX = PAIR ? 16 : kChunk;          // rotated activations per lane
@@ -143,8 +147,8 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     // scalar unit: the host supplies the quotients)
     const int stream = (wave * a.w_inv) >> 8;               // wave / a.W
     const int unit = wave - stream * a.W;
-    const int slab = (MODE == kDual) ? unit >> 1 : unit;
-    const int plane = (MODE == kDual) ? unit & 1 : 0;       // 0: primary plane / rotation / table
+    const int slab = (MODE == kDual && !BOTH) ? unit >> 1 : unit;
+    const int plane = (MODE == kDual && !BOTH) ? unit & 1 : 0;       // 0: primary plane / rotation / table
     constexpr bool combined = (MODE == kSharedLut);
     const int col_a = PAIR ? slab * (kSlab / 2) + 16 * lane : slab * kSlab + (combined ? 16 * lane : 32 * lane);
     const int col_b = PAIR ? col_a : (combined ? col_a + 1024 : col_a + 16);
@@ -152,7 +156,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     const uint32_t laneoff = (uint32_t)lane << 2;
     const int out = a.L.out_features;
     const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
-    constexpr bool use_res = (MODE == kSharedLut);          // second 16-byte load per row
+    constexpr bool use_res = (MODE == kSharedLut) || BOTH;  // second 16-byte load per row
 
     // Contiguous row range of this stream (DYN: of the workgroup): rows_q rows, one more for the
     // first rows_rem ranges.
@@ -171,6 +175,9 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(pp) + (size_t)r_base * row_bytes, 0, 0x7fffffff, 0x00020000);
     const int row_stride = (int)row_bytes;
+    // (BOTH: the residual plane through a descriptor of its own; same offsets as the primary plane)
+    const __amdgpu_buffer_rsrc_t rs2 = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(BOTH ? a.L.packed_residual : pp) + (size_t)r_base * row_bytes, 0, 0x7fffffff, 0x00020000);
 
     uint4 P[NS][R], Q[NS][R];                 // register ring of row groups
     float nrm[NS];                            // norm of the row this lane will store (lanes < V)
@@ -192,6 +199,8 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
             if constexpr (PAIR) {
                 const int rq = ra + 1 < r_last ? ra + 1 : r_last;
                 Q[buf][i] = load_stream16(rs, off_q, (rq - r_base) * row_stride);
+            } else if constexpr (BOTH) {
+                Q[buf][i] = load_stream16(rs2, off_p, soff);
             } else if constexpr (use_res) {
                 Q[buf][i] = load_stream16(rs, off_q, soff);
             }
@@ -213,6 +222,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     for (int e = 0; e < 16; ++e) tv[e] = PT ? 0.0f : tab[e0 + e];
     TileRaw raw[TILES];
     float xt[NX];       // rotated activations, kept in registers for the whole kernel
+    float xr[BOTH ? NX : 1];   // BOTH: those of the residual rotation
     if constexpr (PRE) {
         const float4* pa = reinterpret_cast<const float4*>(static_cast<const float*>(a.x) + (act_a ? col_a : 0));
         const float4* pb = reinterpret_cast<const float4*>(static_cast<const float*>(a.x) + (act_b ? col_b : 0));
@@ -280,7 +290,8 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
         rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_residual, a.L.block_size, image,
                                          wave, nwaves, lane);
         __syncthreads();
-        if (plane == 1) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xt);
+        if constexpr (BOTH) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xr);
+        else if (plane == 1) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xt);
     }
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
@@ -288,6 +299,32 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
 
     // One row (or with PAIR the same columns of two rows: p -> sum, q -> sum2).
     auto decode_row = [&](const uint4& p, const uint4& q, float& sum, float& sum2) {
+        if constexpr (BOTH) {
+            const uint32_t pw[4] = {p.x, p.y, p.z, p.w}, qw[4] = {q.x, q.y, q.z, q.w};
+            float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                uint32_t pv[4], qv[4];
+                pv[0] = *reinterpret_cast<const uint32_t*>(smem + entry_addr<0>(pw[d], laneoff));
+                pv[1] = *reinterpret_cast<const uint32_t*>(smem + entry_addr<1>(pw[d], laneoff));
+                pv[2] = *reinterpret_cast<const uint32_t*>(smem + entry_addr<2>(pw[d], laneoff));
+                pv[3] = *reinterpret_cast<const uint32_t*>(smem + entry_addr<3>(pw[d], laneoff));
+                qv[0] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<0>(qw[d], laneoff));
+                qv[1] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<1>(qw[d], laneoff));
+                qv[2] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<2>(qw[d], laneoff));
+                qv[3] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<3>(qw[d], laneoff));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {        // byte 4 d + j: columns 8 d + 2 j and 8 d + 2 j + 1
+                    const int c = 8 * d + 2 * j;
+                    s0 = __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(pv[j] & 0xffffu)), xt[c], s0);
+                    s1 = __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(pv[j] >> 16)), xt[c + 1], s1);
+                    s2 = __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(qv[j] & 0xffffu)), xr[c], s2);
+                    s3 = __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(qv[j] >> 16)), xr[c + 1], s3);
+                }
+            }
+            sum = (s0 + s1) + (s2 + s3);
+            return;
+        }
         if constexpr (PT) {
             const char* tabp = smem + plane * kLut256Bytes;
             const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
@@ -421,9 +458,9 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     if (it0 < a.iters) consume(0, r_begin + it0 * V, it0);
 }
 
-template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false>
+template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false, bool BOTH = false>
 __global__ __launch_bounds__(1024) void tq_gemv_wide_kernel(GemvArgs a) {
-    wide_body<MODE, R, TILES, PAIR, DYN, PRE, PT>(a, (int)blockIdx.x);
+    wide_body<MODE, R, TILES, PAIR, DYN, PRE, PT, BOTH>(a, (int)blockIdx.x);
 }
 
 // Two or three layers that read the same activation row (q, k, v or gate, up of a decoder layer),
@@ -440,11 +477,11 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_group_kernel(GemvGroup g) {
     wide_body<MODE, R, 1, PAIR, false, false, PT>(g.a[j], b - g.first[j]);
 }
 
-template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false, bool PT = false>
+template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false, bool PT = false, bool BOTH = false>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
     constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
     const size_t lds = (size_t)kRegion + kPartialBytes + (PRE ? 0 : (size_t)a.img_cols * sizeof(float));
-    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE, PT>;
+    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE, PT, BOTH>;
     // More LDS than the default limit has to be asked for, once per kernel and device.
     static bool asked[64] = {};
     int dev = 0;
@@ -493,7 +530,10 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     const int out = a.L.out_features;
     const int slabs = a.W;
     if (PAIR) a.W = a.L.in_features / (kSlab / 2);           // halves per row
-    if (MODE == kDual) a.W = 2 * slabs;                      // (slab, plane) pairs per row
+    // Dual rotation: (slab, plane) pairs per row; rows of one slab whose centroids fit fp16 keep both
+    // planes in one wave instead.
+    const bool both = MODE == kDual && slabs == 1 && a.L.fp16_centroids_ok;
+    if (MODE == kDual && !both) a.W = 2 * slabs;
     a.S = 16 / a.W;                                          // row streams sharing the CU
     const int threads = a.W * a.S * kWave;
     const int padded = slabs * kSlab;
@@ -503,7 +543,7 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     int grid = (out + a.S - 1) / a.S;
     if (grid > num_cus) grid = num_cus;
     if (grid < 1) grid = 1;
-    const bool shared_range = !PAIR && MODE != kDual && a.W == 1;   // one range per workgroup (group counter)
+    const bool shared_range = !PAIR && (MODE != kDual || both) && a.W == 1;   // one range per workgroup (group counter)
     const int ts = shared_range ? grid : grid * a.S;        // row ranges
     a.rows_q = out / ts;
     a.rows_rem = out % ts;
@@ -514,6 +554,13 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     const int R = (MODE != kSharedLut && !a.pre_rotated && max_rows >= 4) ? 4 : max_rows >= 2 * per_r ? 2 : 1;
     a.iters = (max_rows + R * per_r - 1) / (R * per_r);
 
+    if constexpr (MODE == kDual) {
+        if (both) {
+            const int rows_wg = (out + grid - 1) / grid;
+            if (rows_wg >= 4 * a.S) return launch_wide_one<kDual, 2, 1, false, true, false, true, true>(a, grid, threads, stream);
+            return launch_wide_one<kDual, 1, 1, false, true, false, true, true>(a, grid, threads, stream);
+        }
+    }
     const int ntiles = (a.L.in_features + kTile - 1) / kTile;
     const bool two = ntiles > threads / kWave;              // at most two tiles per wave: checked by the caller
     if constexpr (MODE == kSharedLut) return launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
@@ -607,6 +654,7 @@ bool gemv_wide_group_supported(const LayerView* Ls, int n, int num_cus) {
     const int slabs = (L0.in_features / kChunk + kWave - 1) / kWave;
     const int W = wants_pairs(L0) ? L0.in_features / (kSlab / 2) : (L0.mode == kDual ? 2 * slabs : slabs);
     if (W < 2 || W > 16) return false;
+    if (L0.mode == kDual && slabs == 1) return false;       // one-slab dual rows: one wave per row (both planes), no sharing
     const int threads = W * (16 / W) * kWave;
     if ((L0.in_features + kTile - 1) / kTile > threads / kWave) return false;
     for (int j = 0; j < n; ++j) {
