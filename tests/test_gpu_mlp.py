@@ -56,9 +56,9 @@ def _rel(a, b):
     return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / np.linalg.norm(b.astype(np.float64)))
 
 
-def _layer(tq, o, out_f, in_f, bs, shared, seed, scale=0.05):
+def _layer(tq, o, out_f, in_f, bs, shared, seed, scale=0.05, fit=True):
     w = (np.random.default_rng(seed).standard_normal((out_f, in_f)) * scale).astype(np.float32)
-    if out_f * in_f <= 1 << 21:
+    if fit and out_f * in_f <= 1 << 21:
         cbp, cbr = o.fit_layer_codebooks(w, bs)
     else:                                    # the CPU fit takes seconds per million weights
         cbp = cbr = o.generate_codebook(4)
@@ -245,6 +245,40 @@ def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):
         y1 = hip.download(ys_single[j], (batch, o), np.float32)
         assert np.array_equal(yg, y1)
         assert _rel(yg, xin @ dense[j].T) < 5e-3
+    hip.free(dx, *ys_group, *ys_single)
+    for layer in layers:
+        layer.close()
+
+
+def _random_groups(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        inf = int(rng.choice([512, 1024, 2048, 2560, 3072, 4096, 5120, 6144, 8192, 12288, 17408]))
+        bs = int(rng.choice([b for b in (128, 256, 512, 1024) if inf % b == 0]))
+        k = int(rng.integers(1, 4))
+        outs = tuple(int(rng.integers(1, max(2, min(1500, (2 << 20) // inf)))) for _ in range(k))
+        cases.append((outs, inf, bs, bool(rng.integers(0, 2)), int(rng.choice([1, 1, 2, 4, 9, 15, 20]))))
+    return cases
+
+
+@pytest.mark.parametrize("outs,in_f,bs,shared,batch", _random_groups(40, 77))
+def test_forward_group_random_configurations(tq, oracle, outs, in_f, bs, shared, batch):
+    """tq_linear_forward_group on random layer sets and batch sizes: whichever way the call is served
+    (shared launches or layer by layer), every output equals the one of a separate tq_linear_forward."""
+    hip = _Hip()
+    layers = [_layer(tq, oracle, o, in_f, bs, shared, seed=200 + j, fit=False)[0] for j, o in enumerate(outs)]
+    xbits = oracle.f32_to_bf16_bits(np.random.default_rng(batch + in_f).standard_normal((batch, in_f)).astype(np.float32))
+    dx = hip.upload(xbits)
+    ys_group = [hip.alloc(batch * o * 4) for o in outs]
+    ys_single = [hip.alloc(batch * o * 4) for o in outs]
+    tq.forward_group_device(layers, dx, tq.BF16, batch, ys_group, tq.F32)
+    for layer, yp in zip(layers, ys_single):
+        layer.forward_device(dx, tq.BF16, batch, yp, tq.F32)
+    for j, o in enumerate(outs):
+        yg = hip.download(ys_group[j], (batch, o), np.float32)
+        y1 = hip.download(ys_single[j], (batch, o), np.float32)
+        assert np.isfinite(yg).all() and np.array_equal(yg, y1)
     hip.free(dx, *ys_group, *ys_single)
     for layer in layers:
         layer.close()
