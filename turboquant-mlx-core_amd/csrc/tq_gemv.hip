@@ -436,7 +436,11 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
         if constexpr (MODE == kDual) {
             if (gemv_wide_supported(a.L, num_cus)) e = launch_gemv_wide(a, num_cus, stream);
             else if (W <= 8) e = launch_nb<MODE, 1, 512>(a, num_cus, stream);
-            else { pre_rotate(a, stream); e = launch_nb<MODE, 1, 1024>(a, num_cus, stream); }
+            else {
+                pre_rotate(a, stream);
+                if (a.pre_rotated && gemv_wide_supported(a.L, num_cus, true)) e = launch_gemv_wide(a, num_cus, stream);
+                else e = launch_nb<MODE, 1, 1024>(a, num_cus, stream);
+            }
         } else {
             if (left >= 4 && W <= 8)      { step = 4; e = launch_nb<MODE, 4, 512>(a, num_cus, stream); }
             else if (left >= 2 && W <= 8) { step = 2; e = launch_nb<MODE, 2, 512>(a, num_cus, stream); }

@@ -127,10 +127,10 @@ __device__ __forceinline__ void take_from_image(const float* image, int lane, in
 // their rows from the LDS counter like the other one-slab layers.
 template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false, bool BOTH = false>
 __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
-    static_assert(!BOTH || (MODE == kDual && PT && DYN && !PAIR && !PRE && R <= 2), "both planes per wave: dual rotation, pair tables");
+    static_assert(!BOTH || (MODE == kDual && PT && (DYN != PRE) && !PAIR && R <= 2), "both planes per wave: dual rotation, pair tables");
     static_assert(!PT || MODE != kSharedLut, "pair tables serve the nibble planes");
     constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;   // decode tables
-    static_assert(!PRE || (!PAIR && !DYN && MODE != kDual && TILES == 1), "pre-rotated rows: plain slab streams");
+    static_assert(!PRE || (!PAIR && !DYN && (MODE != kDual || BOTH) && TILES == 1), "pre-rotated rows: plain slab streams");
     static_assert(!PAIR || MODE == kSharedLut, "row pairs need the one-byte-per-weight plane");
     static_assert(!DYN || (!PAIR && (MODE != kDual || BOTH)), "the group counter serves one-wave row streams");
     constexpr int NS = 2;                           // register ring: one group decoded, one in flight
@@ -232,6 +232,16 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
             xt[4 * i] = u.x; xt[4 * i + 1] = u.y; xt[4 * i + 2] = u.z; xt[4 * i + 3] = u.w;
             xt[16 + 4 * i] = w.x; xt[17 + 4 * i] = w.y; xt[18 + 4 * i] = w.z; xt[19 + 4 * i] = w.w;
         }
+        if constexpr (BOTH) {          // the residual rotation follows in_features floats further on
+            const float4* qa = pa + (a.L.in_features >> 2);
+            const float4* qb = pb + (a.L.in_features >> 2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 u = qa[i], w = qb[i];
+                xr[4 * i] = u.x; xr[4 * i + 1] = u.y; xr[4 * i + 2] = u.z; xr[4 * i + 3] = u.w;
+                xr[16 + 4 * i] = w.x; xr[17 + 4 * i] = w.y; xr[18 + 4 * i] = w.z; xr[19 + 4 * i] = w.w;
+            }
+        }
     } else {
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {     // tiles past the row re-read its start and are not used
@@ -276,6 +286,10 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
         fetch(1, r_begin + V);
 #pragma unroll
         for (int k = 0; k < NX; ++k) xt[k] = ((k < 16) ? act_a : act_b) ? xt[k] : 0.0f;   // idle runs contribute 0
+        if constexpr (BOTH) {
+#pragma unroll
+            for (int k = 0; k < NX; ++k) xr[k] = ((k < 16) ? act_a : act_b) ? xr[k] : 0.0f;
+        }
     } else {
     float* const image = reinterpret_cast<float*>(smem + kRegion + kPartialBytes);
     rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_primary, a.L.block_size, image, wave,
@@ -532,7 +546,7 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     if (PAIR) a.W = a.L.in_features / (kSlab / 2);           // halves per row
     // Dual rotation: (slab, plane) pairs per row; rows of one slab whose centroids fit fp16 keep both
     // planes in one wave instead.
-    const bool both = MODE == kDual && slabs == 1 && a.L.fp16_centroids_ok;
+    const bool both = MODE == kDual && (slabs == 1 || a.pre_rotated) && a.L.fp16_centroids_ok;
     if (MODE == kDual && !both) a.W = 2 * slabs;
     a.S = 16 / a.W;                                          // row streams sharing the CU
     const int threads = a.W * a.S * kWave;
@@ -551,10 +565,15 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     const int max_rows = (int)(((long long)out + grid * a.S - 1) / (grid * a.S));   // longest share of a stream
     const int per_r = PAIR ? 2 : 1;                         // rows per unit of R
     // (nibble planes: a row is 16 bytes per lane, so four rows make the group of loads of two byte-plane rows)
-    const int R = (MODE != kSharedLut && !a.pre_rotated && max_rows >= 4) ? 4 : max_rows >= 2 * per_r ? 2 : 1;
+    const int R = (MODE != kSharedLut && !a.pre_rotated && !both && max_rows >= 4) ? 4 : max_rows >= 2 * per_r ? 2 : 1;
     a.iters = (max_rows + R * per_r - 1) / (R * per_r);
 
     if constexpr (MODE == kDual) {
+        if (a.pre_rotated) {          // 9 to 16 slabs, one wave per slab, both planes per wave
+            if (!a.L.fp16_centroids_ok) return hipErrorInvalidValue;     // gemv_wide_supported() rules this out
+            return R == 2 ? launch_wide_one<kDual, 2, 1, false, false, true, true, true>(a, grid, threads, stream)
+                          : launch_wide_one<kDual, 1, 1, false, false, true, true, true>(a, grid, threads, stream);
+        }
         if (both) {
             const int rows_wg = (out + grid - 1) / grid;
             if (rows_wg >= 4 * a.S) return launch_wide_one<kDual, 2, 1, false, true, false, true, true>(a, grid, threads, stream);
@@ -687,7 +706,7 @@ bool gemv_wide_supported(const LayerView& L, int num_cus, bool pre_rotated) {
     if (L.block_size > (uint32_t)kTile) return false;
     const int slabs = (L.in_features / kChunk + kWave - 1) / kWave;
     int W = slabs;
-    if (pre_rotated) { if (L.mode == kDual || slabs < 9 || slabs > 16) return false; }
+    if (pre_rotated) { if ((L.mode == kDual && !L.fp16_centroids_ok) || slabs < 9 || slabs > 16) return false; }
     else if (wants_pairs(L)) W = L.in_features / (kSlab / 2);
     else if (L.mode == kDual) { if (slabs > 8) return false; W = 2 * slabs; }   // two waves per slab
     else if (slabs < 1 || slabs > 8) return false;
