@@ -242,7 +242,9 @@ struct SkinnyNibbleArgs {
 };
 
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
-    constexpr int kTabBytes = 16 * 256;                    // 16 entries, one private column per lane
+    // The table is indexed by a whole byte of the plane: an entry holds the bf16 centroids of both
+    // its nibbles, i.e. one register of the B operand, so two weights cost one table read.
+    constexpr int kTabBytes = kSkLutBytes;                 // 256 entries, one private column per lane
     __shared__ __align__(16) char smem[kTabBytes + kSkStageBytes];   // table | 16 x 512 bf16 rotated activations
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -269,7 +271,12 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 
     // Small loads first (they complete in order), then the first row group, which travels while the
     // activations are rotated.
-    const float tval = a.tables[16 * pl + (tid >> 4 & 15)];        // threads 0..255 fill the 256 table slots
+    // Table slots of this thread: slot i = tid + 512 k is entry i >> 4, whose low nibble is the same
+    // for all k and whose high nibble is (tid >> 8) + 2 k.
+    const float tlo = a.tables[16 * pl + ((tid >> 4) & 15)];
+    float thi[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) thi[k] = a.tables[16 * pl + (tid >> 8) + 2 * k];
     TileRaw xin[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {                          // batch rows w and w + 8 (row 0 again past the batch: not used)
@@ -287,9 +294,13 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     };
     if (g_begin < g_end) request(rawA, g_begin);
 
-    if (tid < 256) {                                        // 16 entries x 16 slots of 16 bytes, values rounded to bf16
-        const uint32_t v = (uint32_t)float_to_bf16_bits(tval) << 16;
-        reinterpret_cast<uint4*>(smem)[tid] = make_uint4(v, v, v, v);
+    {                                                       // 256 entries x 16 slots of 16 bytes, values rounded to bf16
+        const uint32_t lo = (uint32_t)float_to_bf16_bits(tlo);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t v = lo | ((uint32_t)float_to_bf16_bits(thi[k]) << 16);
+            reinterpret_cast<uint4*>(smem)[tid + k * kSkThreads] = make_uint4(v, v, v, v);
+        }
     }
     // Rotate batch rows w and w + 8 of the chunk with this plane's seed -> bf16 [16][512] in LDS.
     constexpr int kPitch = kSkChunk * 2;
@@ -318,18 +329,13 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     for (int s = 0; s < 16; ++s)
         afrag[s] = *reinterpret_cast<const sk_bf16x8*>(stage + m * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
 
-    // One dword = 8 weights of 8 consecutive columns (low nibble first) -> one B operand.
+    // One dword = 8 weights of 8 consecutive columns (low nibble first) -> one B operand: byte j of
+    // the dword selects the register that holds columns 2 j and 2 j + 1.
     auto operand = [&](uint32_t w) {
-        const uint32_t ce = w & 0x0F0F0F0Fu, co = (w >> 4) & 0x0F0F0F0Fu;
-        uint32_t e[4], o[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            e[j] = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(ce, laneoff, j));
-            o[j] = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(co, laneoff, j));
-        }
-        // entries are fp32 patterns with the value in the upper half: {even.hi, odd.hi} per column pair
-        const sk_u32x4 r = {__builtin_amdgcn_perm(o[0], e[0], 0x07060302u), __builtin_amdgcn_perm(o[1], e[1], 0x07060302u),
-                            __builtin_amdgcn_perm(o[2], e[2], 0x07060302u), __builtin_amdgcn_perm(o[3], e[3], 0x07060302u)};
+        const sk_u32x4 r = {*reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 0)),
+                            *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 1)),
+                            *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 2)),
+                            *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 3))};
         return __builtin_bit_cast(sk_bf16x8, r);
     };
     auto multiply = [&](const sk_u32x4 (&raw)[4], int grp) {
