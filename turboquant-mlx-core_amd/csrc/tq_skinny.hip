@@ -241,7 +241,9 @@ struct SkinnyNibbleArgs {
     int groups_q, groups_rem;  // groups / workers and groups % workers (workers = waves sharing a unit)
 };
 
-__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
+// unit, wg_in_unit: the (chunk, plane) unit of this workgroup and its index among the workgroups that
+// share the unit for this layer (a launch may serve several layers).
+__device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, const int unit, const int wg_in_unit) {
     // The table is indexed by a whole byte of the plane: an entry holds the bf16 centroids of both
     // its nibbles, i.e. one register of the B operand, so two weights cost one table read.
     constexpr int kTabBytes = kSkLutBytes;                 // 256 entries, one private column per lane
@@ -251,9 +253,7 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t laneoff = (uint32_t)lane << 2;
 
-    // (grid = units x workgroups per unit; unit = chunk * planes + plane; one workgroup per CU)
-    const int unit = blockIdx.x;
-    const int wg_in_unit = blockIdx.y;
+    // (unit = chunk * planes + plane; one workgroup per CU)
     const int chunk = a.planes == 2 ? unit >> 1 : unit, pl = a.planes == 2 ? unit & 1 : 0;
     const int m = lane & 15, g = lane >> 4;
 
@@ -365,6 +365,22 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         if (grp + 2 < g_end) request(rawA, grp + 2);
         multiply(rawB, grp + 1);
     }
+}
+
+// grid = units x workgroups per unit
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
+    skinny_nibble_body(a, (int)blockIdx.x, (int)blockIdx.y);
+}
+
+// Layers of equal width and mode on the same activation rows, one launch (see SkinnyGroup).
+struct SkinnyNibbleGroup {
+    SkinnyNibbleArgs a[3];
+    int first[4];
+};
+__global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_group_kernel(SkinnyNibbleGroup g) {
+    const int b = (int)blockIdx.y;
+    const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
+    skinny_nibble_body(g.a[j], (int)blockIdx.x, b - g.first[j]);
 }
 
 // y[b, n] = norm[n] * out_scale * sum over chunks of partial[c][b][n]
@@ -489,22 +505,27 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     return hipGetLastError();
 }
 
-// Layers that can share the two launches: two or three shared-rotation layers of equal width with
-// blocks of at most 512 columns (the workgroup rotates its chunk itself), 2..15 rows of 16-bit
-// activations, and at least one workgroup per chunk and layer.
+// Layers that can share the two launches: two or three layers of equal width and mode with blocks
+// of at most 512 columns (the workgroup rotates its chunk itself), 2..15 rows of 16-bit activations,
+// and at least one workgroup per work unit and layer.
 bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, int num_cus) {
     if (n < 2 || n > 3) return false;
+    const bool nibble = Ls[0].mode == kDual || Ls[0].mode == kPrimaryOnly;
     for (int j = 0; j < n; ++j) {
-        if (Ls[j].mode != kSharedLut || !Ls[j].packed_combined || Ls[j].block_size > (uint32_t)kSkChunk) return false;
+        if (Ls[j].mode != Ls[0].mode || Ls[j].block_size > (uint32_t)kSkChunk) return false;
+        if (!nibble && (Ls[j].mode != kSharedLut || !Ls[j].packed_combined)) return false;
         if (Ls[j].in_features != Ls[0].in_features || !skinny_supported(Ls[j], x_dtype, batch)) return false;
     }
-    return num_cus / (Ls[0].in_features / kSkChunk) >= n;
+    const int units = Ls[0].in_features / kSkChunk * (Ls[0].mode == kDual ? 2 : 1);
+    return num_cus / units >= n;
 }
 
 hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
                                int y_dtype, float* const* partials, int num_cus, hipStream_t stream) {
-    const int K = Ls[0].in_features, chunks = K / kSkChunk;
-    const int total_wgs = num_cus / chunks;                       // workgroups per chunk, all layers together
+    const bool nibble = Ls[0].mode == kDual || Ls[0].mode == kPrimaryOnly;
+    const int planes = Ls[0].mode == kDual ? 2 : 1;
+    const int K = Ls[0].in_features, chunks = K / kSkChunk * planes;   // work units: (chunk, plane)
+    const int total_wgs = num_cus / chunks;                       // workgroups per unit, all layers together
     long long rows = 0;
     for (int j = 0; j < n; ++j) rows += Ls[j].out_features;
     int wgs[3] = {0, 0, 0}, used = 0;
@@ -516,11 +537,25 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
     for (int j = 0; used < total_wgs; j = (j + 1) % n) { ++wgs[j]; ++used; }
     for (int j = 0; used > total_wgs; j = (j + 1) % n) if (wgs[j] > 1) { --wgs[j]; --used; }
     SkinnyGroup g{};
+    SkinnyNibbleGroup gn{};
     SkinnyReduceGroup r{};
-    g.first[0] = 0; r.first[0] = 0;
+    g.first[0] = 0; gn.first[0] = 0; r.first[0] = 0;
     for (int j = 0; j < 3; ++j) {
         if (j < n) {
             const LayerView& L = Ls[j];
+            SkinnyNibbleArgs& q = gn.a[j];
+            q.x = x; q.x_dtype = x_dtype; q.seed[0] = L.seed_primary; q.seed[1] = L.seed_residual; q.block_size = L.block_size;
+            q.plane[0] = L.packed_primary; q.plane[1] = L.packed_residual;
+            q.tables = L.tables;
+            q.partial = partials[j];
+            q.batch = batch; q.N = L.out_features; q.K = K;
+            q.planes = planes;
+            q.units = chunks;
+            q.groups = (L.out_features + 15) / 16;
+            q.wgs_per_unit = wgs[j];
+            q.groups_q = q.groups / (wgs[j] * (kSkThreads / 64));
+            q.groups_rem = q.groups % (wgs[j] * (kSkThreads / 64));
+            gn.first[j + 1] = gn.first[j] + wgs[j];
             SkinnyArgs& a = g.a[j];
             a.x = x; a.x_dtype = x_dtype; a.seed = L.seed_primary; a.block_size = L.block_size;
             a.xt = nullptr;
@@ -540,13 +575,15 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
             r.first[j + 1] = r.first[j] + (L.out_features + 63) / 64;
         } else {
             g.first[j] = 1 << 30; g.first[j + 1] = 1 << 30;       // no workgroup reaches an unused slot
+            gn.first[j] = 1 << 30; gn.first[j + 1] = 1 << 30;
             r.first[j] = 1 << 30; r.first[j + 1] = 1 << 30;
         }
     }
     int reduce_blocks = 0;
     for (int j = 0; j < n; ++j) reduce_blocks += (Ls[j].out_features + 63) / 64;
     r.y_dtype = y_dtype; r.chunks = chunks;
-    hipLaunchKernelGGL(tq_skinny_group_kernel, dim3(chunks, used), dim3(kSkThreads), 0, stream, g);
+    if (nibble) hipLaunchKernelGGL(tq_skinny_nibble_group_kernel, dim3(chunks, used), dim3(kSkThreads), 0, stream, gn);
+    else hipLaunchKernelGGL(tq_skinny_group_kernel, dim3(chunks, used), dim3(kSkThreads), 0, stream, g);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(tq_skinny_reduce_group_kernel, dim3(reduce_blocks, batch), dim3(256), 0, stream, r);
