@@ -428,28 +428,36 @@ def main():
     out_of = {n_: o_ for n_, o_, _, _ in layers}
     L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
                                           C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
-    for batch in (1, 4, 8):
-        xg = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
-        yg = {n_: torch.empty(batch, out_of[n_], device="cuda", dtype=torch.float32) for n_ in by}
+    def grouped(by, tag):
+        for batch in (1, 4, 8):
+            xg = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
+            yg = {n_: torch.empty(batch, out_of[n_], device="cuda", dtype=torch.float32) for n_ in by}
 
-        def group(names, x, s):
-            hs = (C.c_void_p * len(names))(*[by[n_] for n_ in names])
-            yp = (C.c_void_p * len(names))(*[yg[n_].data_ptr() for n_ in names])
-            if L.tq_linear_forward_group(hs, len(names), x.data_ptr(), tq.BF16, batch, yp, tq.F32, s) != 0:
-                raise RuntimeError(tq.last_error())
+            def group(names, x, s):
+                hs = (C.c_void_p * len(names))(*[by[n_] for n_ in names])
+                yp = (C.c_void_p * len(names))(*[yg[n_].data_ptr() for n_ in names])
+                if L.tq_linear_forward_group(hs, len(names), x.data_ptr(), tq.BF16, batch, yp, tq.F32, s) != 0:
+                    raise RuntimeError(tq.last_error())
 
-        def grouped_step(s):
-            group(("q", "k", "v"), xg[5120], s)
-            group(("o",), xg[5120], s)
-            group(("gate", "up"), xg[5120], s)
-            group(("down",), xg[27648], s)
-        us_g = time_graph_fn(torch, grouped_step, max(args.steps // 10, 10), 2) * 1e6
-        Bg = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
-        extra[f"decoder_layer_projections_32b_bs{batch}_grouped_launches"] = {
-            "us_per_layer_all_7_projections": us_g, "algorithmic_bytes": Bg,
-            "hbm_frac": Bg / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBS,
-            "calls": "q+k+v, o, gate+up, down through tq_linear_forward_group"}
+            def grouped_step(s):
+                group(("q", "k", "v"), xg[5120], s)
+                group(("o",), xg[5120], s)
+                group(("gate", "up"), xg[5120], s)
+                group(("down",), xg[27648], s)
+            us_g = time_graph_fn(torch, grouped_step, max(args.steps // 10, 10), 2) * 1e6
+            Bg = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
+            extra[f"decoder_layer_projections_32b_bs{batch}{tag}_grouped_launches"] = {
+                "us_per_layer_all_7_projections": us_g, "algorithmic_bytes": Bg,
+                "hbm_frac": Bg / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                "calls": "q+k+v, o, gate+up, down through tq_linear_forward_group"}
+    grouped(by, "")
     for _, _, _, h in layers:
+        L.tq_linear_free(h)
+    # the same layer in the converter's default format: dual rotation (include/turboquant/quantizer.h:15)
+    dual = {n_: make_layer(tq, torch, o_, i_, bs, seed=950 + k, sigma=0.01, shared=False, per_layer_codebooks=True)[0]
+            for k, (n_, o_, i_) in enumerate(shapes)}
+    grouped(dual, "_dual_rotation")
+    for h in dual.values():
         L.tq_linear_free(h)
     finish(args, torch, extra, result)
 
