@@ -107,7 +107,7 @@ def test_mlp_block_matches_oracle(tq, oracle, shared, hidden, inter, bs, batch, 
     if batch >= 2 and x_dt == "bf16":
         act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))   # handed to the matrix-core paths as bf16
     want = o.matmul_xwT(act.astype(np.float32), wd, acc_double=True)
-    tol = 1e-3 if (x_dt == "f32" or batch == 1) else 8e-3   # three bf16-weight layers in a row
+    tol = 1e-3 if (x_dt == "f32" or batch == 1) else 5e-3   # three bf16-weight layers in a row
     assert _rel(y, want) < tol
     with pytest.raises(RuntimeError):
         mlp.forward_device(x_dev, code, batch + 1, y_dev, tq.F32)

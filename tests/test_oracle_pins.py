@@ -364,3 +364,91 @@ def test_layer_codebook_recipe(oracle):
     sc = oracle.wht_forward(wn.astype(np.float32), oracle.derive_seed(w, 0), 512) * np.float32(np.sqrt(np.float32(512)))
     by_hand = oracle.generate_codebook_from_data(sc, 4, 100)
     assert np.abs(by_hand.centroids - cbp.centroids).max() < 1e-5
+
+
+def test_layer_codebook_recipe_residual_leg_uses_global_primary(oracle):
+    """src/converter.cpp:345-357: the residual codebook is fitted on
+    scaled - global_cb[quantize(scaled, global_cb)], the *global analytic* primary codebook,
+    not the per-layer one fitted a few lines earlier.  Heavy-tailed rows make the two differ."""
+    rng = np.random.default_rng(11)
+    w = (rng.standard_normal((48, 512)) * 0.02).astype(np.float32)
+    tail = rng.random(w.shape) < 0.05
+    w[tail] = (rng.standard_t(2, size=int(tail.sum())) * 0.08).astype(np.float32)
+    bs = 128
+    cbp, cbr = oracle.fit_layer_codebooks(w, bs)
+    g = oracle.generate_codebook(4)
+    # by hand, in numpy: normalise, rotate, scale, bin against the global codebook, subtract
+    nrm = np.sqrt((w.astype(np.float64) ** 2).sum(axis=1)).astype(np.float32)
+    wn = (w / np.maximum(nrm, np.float32(1e-10))[:, None]).astype(np.float32)
+    sc = (oracle.wht_forward(wn, oracle.derive_seed(w, 0), bs) * np.float32(np.sqrt(np.float32(512)))).ravel()
+    gb = ((g.centroids[:-1] + g.centroids[1:]) * np.float32(0.5)).astype(np.float32)
+    idx_g = np.searchsorted(gb, sc, side="left")                     # lower_bound, src/codebook.cpp:284-302
+    resid_g = (sc - g.centroids[idx_g]).astype(np.float32)
+    want = oracle.generate_codebook_from_data(resid_g, 4, 100)
+    assert np.abs(want.centroids - cbr.centroids).max() < 1e-6
+    # the wrong reading (residuals against the fitted primary) lands elsewhere on this data,
+    # so the check above does discriminate
+    fb = ((cbp.centroids[:-1] + cbp.centroids[1:]) * np.float32(0.5)).astype(np.float32)
+    idx_f = np.searchsorted(fb, sc, side="left")
+    resid_f = (sc - cbp.centroids[idx_f]).astype(np.float32)
+    wrong = oracle.generate_codebook_from_data(resid_f, 4, 100)
+    assert np.abs(wrong.centroids - cbr.centroids).max() > 1e-3
+    assert np.abs(cbp.centroids - g.centroids).max() > 1e-2          # fitted != global here
+
+
+def _dense_from_values(vals, seed, bs, norms):
+    """diag(norm) . blockdiag(diag(s) H / sqrt(bs)) . (vals / sqrt(in)) in float64."""
+    out, inf = vals.shape
+    s = np.array([_sign_bigint(int(seed), j) for j in range(bs)])
+    T = (np.diag(s) @ scipy.linalg.hadamard(bs).astype(np.float64)) / math.sqrt(bs)
+    M = vals.astype(np.float64) / math.sqrt(inf)
+    Wn = np.concatenate([M[:, b:b + bs] @ T.T for b in range(0, inf, bs)], axis=1)
+    return Wn * norms.astype(np.float64)[:, None]
+
+
+def test_short_primary_codebook_zero_fill_shared_and_clamp_dual(oracle):
+    """A 3-bit primary codebook (8 centroids) under 4-bit planes that hold indices up to 15.
+    Shared rotation goes through the 256-entry table, whose entries with p >= n_primary are never
+    written and stay 0: the residual centroid is dropped too (src/dequantizer.cpp:144-150).  The
+    dual-rotation and primary-only paths clamp the index to the last centroid (:94,103)."""
+    rng = np.random.default_rng(3)
+    out, inf, bs = 6, 256, 64
+    p = rng.integers(0, 16, size=(out, inf)).astype(np.uint8)
+    r = rng.integers(0, 16, size=(out, inf)).astype(np.uint8)
+    assert (p >= 8).any() and r.any()
+    pp = oracle.pack4(p).reshape(out, inf // 2)
+    pr = oracle.pack4(r).reshape(out, inf // 2)
+    norms = (rng.random(out) + 0.5).astype(np.float32)
+    cb3, cb4 = oracle.generate_codebook(3), oracle.generate_codebook(4)
+    cP, cR = cb3.centroids.astype(np.float64), cb4.centroids.astype(np.float64)
+
+    # shared rotation: zero-fill
+    qs = oracle.QuantizedWeight(pp, pr, norms, np.array([1234, 0, bs], np.uint32))
+    W = oracle.dequantize_weight_cpu(qs, cb3, cb4, bs)
+    vals = np.where(p < 8, cP[np.minimum(p, 7)] + cR[r], 0.0)
+    want = _dense_from_values(vals, 1234, bs, norms)
+    assert np.abs(W - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+    clamp = _dense_from_values(cP[np.minimum(p, 7)] + cR[r], 1234, bs, norms)
+    assert np.abs(W - clamp).max() > 1e-2                      # a clamping oracle would fail above
+
+    # dual rotation: clamp, two inverse rotations
+    qd = oracle.QuantizedWeight(pp, pr, norms, np.array([1234, 777, bs], np.uint32))
+    W = oracle.dequantize_weight_cpu(qd, cb3, cb4, bs)
+    want = _dense_from_values(cP[np.minimum(p, 7)], 1234, bs, norms) + _dense_from_values(cR[r], 777, bs, norms)
+    assert np.abs(W - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+    zero = _dense_from_values(np.where(p < 8, cP[np.minimum(p, 7)], 0.0), 1234, bs, norms) + \
+        _dense_from_values(cR[r], 777, bs, norms)
+    assert np.abs(W - zero).max() > 1e-2
+
+    # primary only (all residual bytes zero): clamp as well
+    qp = oracle.QuantizedWeight(pp, np.zeros_like(pr), norms, np.array([1234, 777, bs], np.uint32))
+    W = oracle.dequantize_weight_cpu(qp, cb3, cb4, bs)
+    want = _dense_from_values(cP[np.minimum(p, 7)], 1234, bs, norms)
+    assert np.abs(W - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+
+    # a short residual codebook under dual rotation clamps too (:229)
+    qd2 = oracle.QuantizedWeight(pp, pr, norms, np.array([1234, 777, bs], np.uint32))
+    W = oracle.dequantize_weight_cpu(qd2, cb4, cb3, bs)
+    c4 = cb4.centroids.astype(np.float64)
+    want = _dense_from_values(c4[p], 1234, bs, norms) + _dense_from_values(cP[np.minimum(r, 7)], 777, bs, norms)
+    assert np.abs(W - want).max() < 1e-5 * max(1.0, np.abs(want).max())
