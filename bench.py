@@ -23,15 +23,23 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152421.1 KiB + 648.9 KiB.
+# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152512.1 KiB + 606.0 KiB.
 MEASURED_TRAFFIC_BYTES = 312965325
+# Average duration of the headline kernel in the rocprofv3 kernel trace of `python bench.py --skip-extra`
+# (same file), in microseconds, and the kernel's name there.
+PROFILED_KERNEL_US = 49.76
+HEADLINE_KERNEL = "tq_gemv_wide_kernel<shared, R=2, TILES=1, rows from an LDS counter>"
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
 
-# Untimed replays of a captured graph before the timed one.  The first replay uploads the graph; the
-# replay after it still runs 4-5 % slower than all later ones (power management settling under the
-# load), so the timed replay is the fourth.
-UNTIMED_REPLAYS = 3
+# A captured graph is replayed untimed until this much GPU time has passed (at least three replays:
+# the first uploads the graph, and the replays right after it still run a few per cent slower while
+# clocks and memory settle under the load), so the timed region starts on a machine in steady state
+# whatever --steps is.
+UNTIMED_WARM_SECONDS = 0.05
+# One event pair then brackets as many back-to-back replays as it takes to time at least this many
+# kernel launches; the time per step is the bracket divided by the steps it holds.
+MIN_TIMED_LAUNCHES = 200
 
 
 def algorithmic_bytes(out, inf, batch, x_bytes, y_bytes):
@@ -75,58 +83,30 @@ def make_layer(tq, torch, out, inf, bs, seed, sigma, shared=True, per_layer_code
                             seeds.ctypes.data_as(u32p)) != 0:
         raise RuntimeError(tq.last_error())
     del w
-    h = L.tq_linear_create_from_device(inf, out, pp.data_ptr(), inf // 2, pr.data_ptr(), inf // 2, norms.data_ptr(),
-                                       seeds.ctypes.data_as(u32p), cbp.ctypes.data_as(f32p), 16,
-                                       cbr.ctypes.data_as(f32p), 16, bs)
+    tensors = dict(pp=pp, pr=pr, norms=norms, cbp=cbp[:16].copy(), cbr=cbr[:16].copy(), seeds=seeds)
+    h = layer_from_tensors(tq, tensors, out, inf, bs)
+    torch.cuda.synchronize()
+    return h, tensors
+
+
+def layer_from_tensors(tq, t, out, inf, bs):
+    """A layer handle with its own device copy of the quantized tensors `t` (as make_layer returns them)."""
+    import ctypes as C
+    f32p, u32p = C.POINTER(C.c_float), C.POINTER(C.c_uint32)
+    h = tq.lib().tq_linear_create_from_device(inf, out, t["pp"].data_ptr(), inf // 2, t["pr"].data_ptr(), inf // 2,
+                                              t["norms"].data_ptr(), t["seeds"].ctypes.data_as(u32p),
+                                              t["cbp"].ctypes.data_as(f32p), 16, t["cbr"].ctypes.data_as(f32p), 16, bs)
     if not h:
         raise RuntimeError(tq.last_error())
-    torch.cuda.synchronize()
-    return h, dict(pp=pp, pr=pr, norms=norms, cbp=cbp[:16].copy(), cbr=cbr[:16].copy(), seeds=seeds)
+    return h
 
 
-def time_graph(tq, torch, handles, x, y, xcode, batch, steps, warmup, spread=None):
-    """Capture `steps` forwards (cycling over `handles`) in one HIP graph; return seconds of one replay.
-    With `spread` (a list), replay the graph 20 more times afterwards and append each replay's seconds."""
-    L = tq.lib()
-    stream = torch.cuda.Stream()
-    n = len(handles)
-
-    def enqueue(count, s):
-        for i in range(count):
-            rc = L.tq_linear_forward(handles[i % n], x.data_ptr(), xcode, batch, y.data_ptr(), 0, s.cuda_stream)
-            if rc != 0:
-                raise RuntimeError(tq.last_error())
-
-    with torch.cuda.stream(stream):
-        enqueue(max(warmup, 1), stream)
-    stream.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=stream):
-        enqueue(steps, stream)
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with torch.cuda.stream(stream):
-        for _ in range(UNTIMED_REPLAYS):   # untimed: graph upload, then clocks and memory settle under load
-            graph.replay()
-        stream.synchronize()
-        torch.cuda.synchronize()
-        start.record(stream)
-        graph.replay()
-        end.record(stream)
-    torch.cuda.synchronize()
-    secs = start.elapsed_time(end) * 1e-3
-    if spread is not None:
-        for _ in range(20):
-            with torch.cuda.stream(stream):
-                start.record(stream)
-                graph.replay()
-                end.record(stream)
-            torch.cuda.synchronize()
-            spread.append(start.elapsed_time(end) * 1e-3)
-    return secs
-
-
-def time_graph_fn(torch, enqueue_step, steps, warmup):
-    """Capture `steps` calls of enqueue_step(stream_handle) in one HIP graph; return seconds per step."""
+def time_graph_fn(torch, enqueue_step, steps, warmup, launches_per_step=1, spread=None):
+    """Capture `steps` calls of enqueue_step(stream_handle) in one HIP graph and time it with HIP events
+    on the launching stream.  Returns (seconds per step, timed steps).  `warmup` eager steps run first;
+    the graph is then replayed untimed for UNTIMED_WARM_SECONDS, and one event pair brackets enough
+    back-to-back replays to hold MIN_TIMED_LAUNCHES kernel launches.  With `spread` (a list): 20 more
+    single replays are timed one by one and their seconds per step appended."""
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for _ in range(max(warmup, 1)):
@@ -137,16 +117,43 @@ def time_graph_fn(torch, enqueue_step, steps, warmup):
         for _ in range(steps):
             enqueue_step(stream.cuda_stream)
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    replays = max(1, -(-MIN_TIMED_LAUNCHES // (steps * launches_per_step)))
     with torch.cuda.stream(stream):
-        for _ in range(UNTIMED_REPLAYS):   # untimed: graph upload, then clocks and memory settle under load
+        t0 = time.perf_counter()
+        done = 0
+        while done < 3 or time.perf_counter() - t0 < UNTIMED_WARM_SECONDS:
             graph.replay()
-        stream.synchronize()
+            stream.synchronize()
+            done += 1
         torch.cuda.synchronize()
         start.record(stream)
-        graph.replay()
+        for _ in range(replays):
+            graph.replay()
         end.record(stream)
     torch.cuda.synchronize()
-    return start.elapsed_time(end) * 1e-3 / steps
+    secs = start.elapsed_time(end) * 1e-3 / (steps * replays)
+    if spread is not None:
+        for _ in range(20):
+            with torch.cuda.stream(stream):
+                start.record(stream)
+                graph.replay()
+                end.record(stream)
+            torch.cuda.synchronize()
+            spread.append(start.elapsed_time(end) * 1e-3 / steps)
+    return secs, steps * replays
+
+
+def time_graph(tq, torch, handles, x, y, xcode, batch, steps, warmup, spread=None):
+    """Seconds per forward and timed forwards, cycling over `handles` (see time_graph_fn)."""
+    L = tq.lib()
+    n = len(handles)
+    turn = [0]
+
+    def step(s):
+        if L.tq_linear_forward(handles[turn[0] % n], x.data_ptr(), xcode, batch, y.data_ptr(), 0, s) != 0:
+            raise RuntimeError(tq.last_error())
+        turn[0] += 1
+    return time_graph_fn(torch, step, steps, warmup, 1, spread)
 
 
 def cpu_baseline(torch, tensors, out, inf, bs, x_f32):
@@ -209,10 +216,16 @@ def main():
     g = torch.Generator(device="cuda"); g.manual_seed(0xCAFEBABE + 3)
     x = torch.randn(1, inf, device="cuda", generator=g).to(torch.bfloat16)
     y = torch.empty(1, out, device="cuda", dtype=torch.float32)
+    # Two copies of the layer (2 x 311 MB) are cycled, so no launch can find its weights in the 256 MB
+    # last-level cache left there by the launch before it: `value` is the HBM-resident rate.  The same
+    # graph over one copy is reported beside it.
+    handle2 = layer_from_tensors(tq, tensors, out, inf, bs)
     spread = []
-    secs = time_graph(tq, torch, [handle], x, y, tq.BF16, 1, args.steps, args.warmup, spread)
-    us = secs / args.steps * 1e6
-    spread_us = np.sort(np.array(spread)) / args.steps * 1e6
+    secs, timed = time_graph(tq, torch, [handle, handle2], x, y, tq.BF16, 1, args.steps, args.warmup, spread)
+    us = secs * 1e6
+    secs_one, _ = time_graph(tq, torch, [handle], x, y, tq.BF16, 1, args.steps, args.warmup)
+    tq.lib().tq_linear_free(handle2)
+    spread_us = np.sort(np.array(spread)) * 1e6
     B = algorithmic_bytes(out, inf, 1, 2, 4)
     achieved = B / (us * 1e-6) / 1e9
 
@@ -223,7 +236,10 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "untimed_graph_replays_before_timing": UNTIMED_REPLAYS,
+        "timed_launches": timed,
+        "timing": f"{args.steps} steps per HIP graph; untimed replays for {UNTIMED_WARM_SECONDS * 1e3:.0f} ms, then "
+                  f"{timed // args.steps} back-to-back replays inside one HIP event pair ({timed} kernel launches); "
+                  "ms_per_step = bracket / steps in it",
         "ms_per_step": us * 1e-3,
         "higher_is_better": True,
         "scaling": "weak",
@@ -233,15 +249,21 @@ def main():
                 "library's TQ8 quantizer with per-layer Lloyd-Max codebooks (shared rotation, block 512); "
                 "bf16 N(0,1) activations",
         "config": {"workload": "Qwen2.5-0.5B lm_head as TQ8 linear 151936x2048, shared rotation, block 512, "
-                               "x bf16 [1,2048], y f32 [1,151936]",
+                               "x bf16 [1,2048], y f32 [1,151936]; two weight copies cycled (HBM-resident)",
                    "baseline_note": "vs_baseline divides by the reference's published 47.3 tok/s (Apple Silicon)"},
         "us_per_layer": us,
+        "us_per_layer_one_weight_copy": secs_one * 1e6,
         "us_per_layer_over_20_more_replays": {"median": float(np.median(spread_us)),
                                               "p10": float(np.percentile(spread_us, 10)),
                                               "p90": float(np.percentile(spread_us, 90))},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "tq_gemv_wide_kernel<shared, R=2, TILES=1, rows from an LDS counter>", "algorithmic_bytes": B},
+                     "kernel": HEADLINE_KERNEL, "algorithmic_bytes": B,
+                     "us_per_launch_hip_events": us,
+                     "us_per_launch_kernel_trace": PROFILED_KERNEL_US,
+                     "kernel_trace_source": "profiles/gemv_lm_head_151936x2048_bs1.txt (rocprofv3 --kernel-trace "
+                                            "--stats of this command; average kernel duration, launch gaps excluded)",
+                     "frac_one_weight_copy": B / secs_one / 1e9 / HBM_PEAK_GBS},
     }
 
     # ---- CPU baseline on this host ---------------------------------------------------
@@ -286,8 +308,8 @@ def main():
         x1 = torch.randn(1, in1, device="cuda", generator=g)
         y1 = torch.empty(1, out1, device="cuda", dtype=torch.float32)
         steps1 = max(args.steps, copies) // copies * copies
-        us_hbm = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
-        us_hot = time_graph(tq, torch, handles[:1], x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
+        us_hbm = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup)[0] * 1e6
+        us_hot = time_graph(tq, torch, handles[:1], x1, y1, tq.F32, 1, steps1, args.warmup)[0] * 1e6
         B1 = algorithmic_bytes(out1, in1, 1, 4, 4)
         extra["gemv_4096x4096_f32_bs1"] = {"us_per_layer_hbm_resident": us_hbm, "us_per_layer_cache_resident": us_hot,
                                            "weight_copies_cycled": copies, "algorithmic_bytes": B1,
@@ -315,7 +337,7 @@ def main():
         tq.lib().tq_linear_free(href)
         # the library default of the reference is dual rotation (include/turboquant/quantizer.h:15)
         handles = [make_layer(tq, torch, out1, in1, bs, seed=300 + 2 * i, sigma=0.02, shared=False)[0] for i in range(copies)]
-        us_dual = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup) / steps1 * 1e6
+        us_dual = time_graph(tq, torch, handles, x1, y1, tq.F32, 1, steps1, args.warmup)[0] * 1e6
         extra["gemv_4096x4096_f32_bs1_dual_rotation"] = {"us_per_layer_hbm_resident": us_dual,
                                                          "hbm_frac": B1 / (us_dual * 1e-6) / 1e9 / HBM_PEAK_GBS}
         for h in handles:
@@ -389,7 +411,7 @@ def main():
                     raise RuntimeError(tq.last_error())
                 turn[0] += 1
             steps_m = max(2, args.steps // 2 * 2)
-            us_m = time_graph_fn(torch, mlp_step, steps_m, 2) * 1e6
+            us_m = time_graph_fn(torch, mlp_step, steps_m, 2, 3)[0] * 1e6
             Bm = 2 * algorithmic_bytes(inter, hid, 1, 2, 4) + algorithmic_bytes(hid, inter, 1, 4, 4)
             extra["mlp_block_7b_bs1_" + ("shared_rotation" if shared else "dual_rotation")] = {
                 "us_per_block": us_m, "algorithmic_bytes": Bm, "hbm_frac": Bm / (us_m * 1e-6) / 1e9 / HBM_PEAK_GBS,
@@ -416,7 +438,7 @@ def main():
             for n_, o_, i_, h in layers:
                 if L.tq_linear_forward(h, xs[i_].data_ptr(), tq.BF16, batch, ys[o_].data_ptr(), tq.F32, s) != 0:
                     raise RuntimeError(tq.last_error())
-        us_l = time_graph_fn(torch, layer_step, max(args.steps // 10, 10), 2) * 1e6
+        us_l = time_graph_fn(torch, layer_step, max(args.steps // 10, 10), 2, 7)[0] * 1e6
         Bl = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
         extra[f"decoder_layer_projections_32b_bs{batch}"] = {
             "us_per_layer_all_7_projections": us_l, "algorithmic_bytes": Bl,
@@ -444,7 +466,7 @@ def main():
                 group(("o",), xg[5120], s)
                 group(("gate", "up"), xg[5120], s)
                 group(("down",), xg[27648], s)
-            us_g = time_graph_fn(torch, grouped_step, max(args.steps // 10, 10), 2) * 1e6
+            us_g = time_graph_fn(torch, grouped_step, max(args.steps // 10, 10), 2, 4)[0] * 1e6
             Bg = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
             extra[f"decoder_layer_projections_32b_bs{batch}{tag}_grouped_launches"] = {
                 "us_per_layer_all_7_projections": us_g, "algorithmic_bytes": Bg,

@@ -98,6 +98,16 @@ int tq_linear_forward(tq_linear_t layer, const void* x_dev, int x_dtype, int bat
                       void* y_dev, int y_dtype, void* stream);
 
 /**
+ * Size the layer's workspaces for calls of up to max_batch rows now, so that no later
+ * tq_linear_forward / tq_linear_forward_group call with at most that many rows allocates (the
+ * matrix-core paths for 2 or more rows of 16-bit activations otherwise allocate on first use, which
+ * synchronises the device and cannot be captured in a HIP graph; a call that would have to grow a
+ * workspace while its stream is being captured fails instead).  The reference allocates its output
+ * per call (src/dequantizer.cpp:516) and has no such entry.
+ */
+int tq_linear_reserve(tq_linear_t layer, int max_batch);
+
+/**
  * One to three layers applied to the SAME activations: y_devs[j][batch, out_j] = x[batch, in] . W_j^T,
  * e.g. the q, k, v or the gate, up projections of a decoder layer.  Layers of equal width and mode share
  * their kernel launches where the kernels allow it (batch 1: shared or dual rotation, blocks <= 512, more

@@ -52,6 +52,7 @@ def lib():
         for name in ("tq_linear_in_features", "tq_linear_out_features", "tq_linear_mode"):
             getattr(L, name).argtypes = [C.c_void_p]
         L.tq_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
+        L.tq_linear_reserve.argtypes = [C.c_void_p, C.c_int]
         L.tq_linear_forward_host.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]
         L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
                                               C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
@@ -139,6 +140,11 @@ class TurboQuantLinear:
         """Asynchronous forward on raw device pointers (e.g. torch ``data_ptr()``)."""
         rc = lib().tq_linear_forward(self._h, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream)
         if rc != 0:
+            raise RuntimeError(last_error())
+
+    def reserve(self, max_batch):
+        """Size the workspaces now so that forward_device with up to max_batch rows never allocates."""
+        if lib().tq_linear_reserve(self._h, max_batch) != 0:
             raise RuntimeError(last_error())
 
     def dequantize(self):

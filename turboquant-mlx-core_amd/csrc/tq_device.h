@@ -64,9 +64,10 @@ hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int ba
 hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
                                hipStream_t stream);
 // Small batches (tq_skinny.hip): 2..15 rows of 16-bit activations on shared-rotation layers, batch rows as
-// the M side of 16x16x32 MFMAs.  xt_workspace as for launch_prefill; partial: skinny_partial_bytes().
+// the M side of 16x16x32 MFMAs.  xt_workspace as for launch_prefill; partial: skinny_partial_bytes() for this batch.
 bool skinny_supported(const LayerView& L, int x_dtype, int batch);
-size_t skinny_partial_bytes(const LayerView& L);
+size_t skinny_partial_bytes(const LayerView& L, int batch);
+size_t skinny_workspace_bytes(const LayerView& L, int batch);
 hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                          void* xt_workspace, float* partial, int num_cus, hipStream_t stream);
 // Two or three shared-rotation layers of equal width on the same activation rows: both launches shared.

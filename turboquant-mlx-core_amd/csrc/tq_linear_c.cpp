@@ -112,8 +112,15 @@ void build_tables(int mode, const float* cbp, int np, const float* cbr, int nr, 
     for (int i = 0; i < 16; ++i) t[pn + i] = cbr[i < nr ? i : nr - 1];
 }
 
-bool ensure_stage(void** buf, size_t* have, size_t need) {
+// Grows a workspace of a handle.  A buffer that a captured graph may still reference is never
+// replaced while the stream is being captured: growth during capture is an error.
+bool ensure_stage(void** buf, size_t* have, size_t need, hipStream_t stream = nullptr) {
     if (*have >= need) return true;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (stream && hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
+        set_error("workspace too small while the stream is being captured: call tq_linear_reserve first");
+        return false;
+    }
     if (*buf) { (void)hipFree(*buf); *buf = nullptr; *have = 0; }
     if (!hip_ok(hipMalloc(buf, need), "hipMalloc(staging)")) return false;
     *have = need;
@@ -256,8 +263,8 @@ tq_linear_t create_impl(int in_features, int out_features,
 
 }  // namespace
 
-// Shared by tq_linear_forward and the MLP block (tq_mlp_c.cpp).  gate: optional fp32 [batch, out];
-// the batch-1..15 kernel then stores silu(gate) * y.  Returns 0 on success.
+// Shared by tq_linear_forward and the MLP block.  gate: optional fp32 [batch, out]; the batch-1..15
+// kernel then stores silu(gate) * y.  Returns 0 on success.
 int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void* y_dev, int y_dtype,
                  hipStream_t stream, const float* gate) {
     if (h->view.mode >= tq::kShared5 && !h->has_fwd_view) {
@@ -265,21 +272,29 @@ int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void
                   "supported by the fused kernels"); return 1;
     }
     const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
-    if (tq::prefill_supported(V, x_dtype, batch)) {
+    const bool prefill = tq::prefill_supported(V, x_dtype, batch);
+    const bool skinny = !prefill && !gate && tq::skinny_supported(V, x_dtype, batch);
+    void* work = nullptr;
+    float* partial = nullptr;
+    if (prefill || skinny) {
+        const size_t work_need = prefill ? tq::prefill_workspace_bytes(V, batch) : tq::skinny_workspace_bytes(V, batch);
+        const size_t partial_need = skinny ? tq::skinny_partial_bytes(V, batch) : 0;
+        // The first call with a larger batch allocates (not capturable in a graph); tq_linear_reserve
+        // sizes the workspaces ahead of time.
+        if (!ensure_stage(&h->d_work, &h->work_bytes, work_need, stream)) return 1;
+        if (skinny && !ensure_stage(&h->d_partial, &h->partial_bytes, partial_need, stream)) return 1;
+        work = h->d_work;
+        partial = static_cast<float*>(h->d_partial);
+    }
+    if (prefill) {
         if (gate) { set_error("tq_linear_forward: gated store is a batch < 16 feature"); return 1; }
-        // Dense contraction: rotate once, dequantise tiles to bf16 in LDS, MFMA.  The first call
-        // with a larger batch allocates the rotated-activation workspace (not capturable in a graph).
-        if (!ensure_stage(&h->d_work, &h->work_bytes, tq::prefill_workspace_bytes(V, batch))) return 1;
-        return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, h->d_work, stream),
+        // Dense contraction: rotate once, dequantise tiles to bf16 in LDS, MFMA.
+        return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, stream),
                       "tq_prefill launch") ? 0 : 1;
     }
-    if (!gate && tq::skinny_supported(V, x_dtype, batch)) {
-        // 2..15 rows of 16-bit activations: batch rows on the matrix cores, bf16 weights.  Workspaces are
-        // allocated on the first such call (not capturable in a graph), then reused.
-        if (!ensure_stage(&h->d_work, &h->work_bytes, tq::prefill_workspace_bytes(V, batch)) ||
-            !ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V))) return 1;
-        return hip_ok(tq::launch_skinny(V, x_dev, x_dtype, batch, y_dev, y_dtype, h->d_work,
-                                        static_cast<float*>(h->d_partial), device_cu_count(), stream),
+    if (skinny) {
+        // 2..15 rows of 16-bit activations: batch rows on the matrix cores, bf16 weights.
+        return hip_ok(tq::launch_skinny(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, partial, device_cu_count(), stream),
                       "tq_skinny launch") ? 0 : 1;
     }
     return hip_ok(tq::launch_gemv(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream, gate),
@@ -333,6 +348,19 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
     } catch (...) { set_error("tq_linear_forward: exception"); return 1; }
 }
 
+int tq_linear_reserve(tq_linear_t h, int max_batch) {
+    try {
+        if (!h || max_batch <= 0) { set_error("tq_linear_reserve: bad argument"); return 1; }
+        const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
+        if (max_batch < 2) return 0;                       // one row uses no workspace
+        const size_t small = tq::skinny_workspace_bytes(V, max_batch < 15 ? max_batch : 15);
+        const size_t big = max_batch >= 16 ? tq::prefill_workspace_bytes(V, max_batch) : 0;
+        if (!ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big)) return 1;
+        if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < 15 ? max_batch : 15))) return 1;
+        return 0;
+    } catch (...) { set_error("tq_linear_reserve: exception"); return 1; }
+}
+
 int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int x_dtype, int batch,
                             void* const* y_devs, int y_dtype, void* stream) {
     try {
@@ -365,7 +393,7 @@ int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int
             // on the first such call (not capturable in a graph), as in tq_linear_forward.
             float* partials[3] = {nullptr, nullptr, nullptr};
             for (int j = 0; j < n; ++j) {
-                if (!ensure_stage(&hs[j]->d_partial, &hs[j]->partial_bytes, tq::skinny_partial_bytes(views[j]))) return 1;
+                if (!ensure_stage(&hs[j]->d_partial, &hs[j]->partial_bytes, tq::skinny_partial_bytes(views[j], batch), st)) return 1;
                 partials[j] = static_cast<float*>(hs[j]->d_partial);
             }
             return hip_ok(tq::launch_skinny_group(views, n, x_dev, x_dtype, batch, y_devs, y_dtype, partials,
@@ -491,12 +519,8 @@ tq_mlp_t tq_mlp_create(tq_linear_t gate, tq_linear_t up, tq_linear_t down, int m
                   hip_ok(hipMalloc(&m->d_act, n * sizeof(float)), "hipMalloc(act)");
         // The batched path of the three layers needs rotated-activation workspaces: size them now so
         // that tq_mlp_forward never allocates.
-        for (tq_linear_t l : {gate, up, down}) {
-            const tq::LayerView& V = l->has_fwd_view ? l->fwd_view : l->view;
-            if (ok && max_batch >= 2)
-                ok = ensure_stage(&l->d_work, &l->work_bytes, tq::prefill_workspace_bytes(V, max_batch)) &&
-                     ensure_stage(&l->d_partial, &l->partial_bytes, tq::skinny_partial_bytes(V));
-        }
+        for (tq_linear_t l : {gate, up, down})
+            if (ok) ok = tq_linear_reserve(l, max_batch) == 0;
         if (!ok) { delete m; return nullptr; }
         return m;
     } catch (...) { set_error("tq_mlp_create: exception"); return nullptr; }

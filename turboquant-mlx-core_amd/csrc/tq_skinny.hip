@@ -35,7 +35,7 @@ struct SkinnyArgs {
     const uint16_t* xt;        // otherwise: rotated activations, bf16 tile images [K/32][256 rows x 64 B] (rows >= batch unset)
     const uint8_t* plane;      // combined bytes [N, K]
     const float* tables;       // 256-entry sum table
-    float* partial;            // [chunks][16][N] fp32
+    float* partial;            // [chunks][batch][N] fp32
     int batch, N, K;
     int chunks;                // K / 512
     int groups;                // ceil(N / 16)
@@ -187,7 +187,7 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int b = 4 * g + r;
-                if (b < a.batch) a.partial[((size_t)chunk * 16 + b) * a.N + n] = acc[r];
+                if (b < a.batch) a.partial[((size_t)chunk * a.batch + b) * a.N + n] = acc[r];
             }
         }
     };
@@ -232,7 +232,7 @@ struct SkinnyNibbleArgs {
     uint32_t seed[2], block_size;
     const uint8_t* plane[2];   // [N, K/2] each; plane[1] unused for primary-only layers
     const float* tables;       // 16 primary centroids, then 16 residual ones
-    float* partial;            // [units][16][N] fp32
+    float* partial;            // [units][batch][N] fp32
     int batch, N, K;
     int units;                 // (K / 512) * planes
     int planes;                // 1 or 2
@@ -353,7 +353,7 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int b = 4 * g + r;
-                if (b < a.batch) a.partial[((size_t)unit * 16 + b) * a.N + n] = acc[r];
+                if (b < a.batch) a.partial[((size_t)unit * a.batch + b) * a.N + n] = acc[r];
             }
         }
     };
@@ -398,7 +398,7 @@ __device__ __forceinline__ void skinny_reduce_body(const float* __restrict__ par
     const bool live = n < N;
     const float nrm = live ? norms[n] : 0.0f;
     const float* p = partial + (size_t)b * N + (live ? n : 0);
-    const size_t step = (size_t)16 * N;
+    const size_t step = (size_t)gridDim.y * N;          // one chunk: [batch][N]
     float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     int c = wave;
     for (; c + 28 < chunks; c += 32) {
@@ -446,12 +446,19 @@ bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
     return (L.mode == kSharedLut && L.packed_combined) || skinny_nibble(L);
 }
 
-size_t skinny_partial_bytes(const LayerView& L) {
+size_t skinny_partial_bytes(const LayerView& L, int batch) {
     const size_t units = (size_t)(L.in_features / kSkChunk) * (L.mode == kDual ? 2 : 1);
-    return units * 16 * L.out_features * sizeof(float);
+    return units * (size_t)batch * L.out_features * sizeof(float);
 }
 
-// xt_workspace: as for launch_prefill (prefill_workspace_bytes); partial: skinny_partial_bytes.
+// Rotated-activation workspace of launch_skinny: only layers with blocks wider than a chunk go
+// through the separate rotation kernel; everything else rotates inside the kernel.
+size_t skinny_workspace_bytes(const LayerView& L, int batch) {
+    if (skinny_nibble(L) || L.block_size <= (uint32_t)kSkChunk) return 0;
+    return prefill_workspace_bytes(L, batch);
+}
+
+// xt_workspace: skinny_workspace_bytes (may be NULL when that is 0); partial: skinny_partial_bytes.
 hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                          void* xt_workspace, float* partial, int num_cus, hipStream_t stream) {
     if (skinny_nibble(L)) {
