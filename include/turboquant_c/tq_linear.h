@@ -108,6 +108,21 @@ int tq_linear_forward(tq_linear_t layer, const void* x_dev, int x_dtype, int bat
 int tq_linear_reserve(tq_linear_t layer, int max_batch);
 
 /**
+ * tq_linear_forward for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * kernels and the same results as tq_linear_forward, but the workspaces of the matrix-core paths
+ * (2 or more rows of 16-bit activations: rotated activations and per-chunk partial products) live in
+ * a fixed array of TQ_STATIC_SCRATCH_BYTES inside the library instead of buffers the handle allocates
+ * on first use; the call allocates and frees nothing.  It fails (non-zero, tq_last_error says how many
+ * bytes were needed) when layer and batch need more than that.  Each GPU has one such array, shared
+ * by every call on it and keeping the previous call's contents: calls that overlap on one GPU
+ * (different streams or threads) race.  One row, and fp32 activations, use no workspace.
+ */
+#define TQ_STATIC_SCRATCH_BYTES (32u << 20)
+int tq_linear_forward_static(tq_linear_t layer, const void* x_dev, int x_dtype, int batch,
+                             void* y_dev, int y_dtype, void* stream);
+
+/**
  * One to three layers applied to the SAME activations: y_devs[j][batch, out_j] = x[batch, in] . W_j^T,
  * e.g. the q, k, v or the gate, up projections of a decoder layer.  Layers of equal width and mode share
  * their kernel launches where the kernels allow it (batch 1: shared or dual rotation, blocks <= 512, more

@@ -52,6 +52,7 @@ def lib():
         for name in ("tq_linear_in_features", "tq_linear_out_features", "tq_linear_mode"):
             getattr(L, name).argtypes = [C.c_void_p]
         L.tq_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
+        L.tq_linear_forward_static.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
         L.tq_linear_reserve.argtypes = [C.c_void_p, C.c_int]
         L.tq_linear_forward_host.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]
         L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
@@ -139,6 +140,12 @@ class TurboQuantLinear:
     def forward_device(self, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream=None):
         """Asynchronous forward on raw device pointers (e.g. torch ``data_ptr()``)."""
         rc = lib().tq_linear_forward(self._h, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream)
+        if rc != 0:
+            raise RuntimeError(last_error())
+
+    def forward_static_device(self, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream=None):
+        """forward_device without any allocation: workspaces in the library's fixed scratch array."""
+        rc = lib().tq_linear_forward_static(self._h, x_ptr, x_dtype, batch, y_ptr, y_dtype, stream)
         if rc != 0:
             raise RuntimeError(last_error())
 

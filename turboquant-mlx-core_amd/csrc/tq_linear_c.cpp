@@ -9,6 +9,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -263,10 +264,41 @@ tq_linear_t create_impl(int in_features, int out_features,
 
 }  // namespace
 
-// Shared by tq_linear_forward and the MLP block.  gate: optional fp32 [batch, out]; the batch-1..15
-// kernel then stores silu(gate) * y.  Returns 0 on success.
+// Workspace of the matrix-core paths for callers that cannot allocate (tq_linear_forward_static):
+// rotated activations (tile images) followed by the per-chunk partial products of the small-batch
+// kernels.  One copy per GPU, held until the process ends; every call on a GPU shares it, so calls
+// that overlap on one GPU race.  Nothing in it has to start at zero: the kernels write every element
+// they later read (rows past the batch are computed from whatever is there and never stored).
+__device__ __align__(256) unsigned char scratch[TQ_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+// Device address of `scratch` on the current device (the array's name is only a host-side stand-in).
+void* static_scratch_ptr() {
+    static std::mutex mu;
+    static void* ptrs[64] = {};
+    int dev = 0;
+    if (!hip_ok(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+    if (dev < 0 || dev >= 64) { set_error("tq_linear_forward_static: device index out of range"); return nullptr; }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        if (!hip_ok(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+        ptrs[dev] = p;
+    }
+    return ptrs[dev];
+}
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+}  // namespace
+
+// Shared by tq_linear_forward, tq_linear_forward_static and the MLP block.  gate: optional fp32
+// [batch, out]; the batch-1..15 kernel then stores silu(gate) * y.  static_ws: the workspaces of the
+// matrix-core paths come from there (TQ_STATIC_SCRATCH_BYTES) instead of the handle's own buffers,
+// and nothing is allocated.  Returns 0 on success.
 int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void* y_dev, int y_dtype,
-                 hipStream_t stream, const float* gate) {
+                 hipStream_t stream, const float* gate, void* static_ws = nullptr) {
     if (h->view.mode >= tq::kShared5 && !h->has_fwd_view) {
         set_error("tq_linear_forward: 5-bit primary with its own residual rotation or a 4-bit residual is not "
                   "supported by the fused kernels"); return 1;
@@ -279,12 +311,22 @@ int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void
     if (prefill || skinny) {
         const size_t work_need = prefill ? tq::prefill_workspace_bytes(V, batch) : tq::skinny_workspace_bytes(V, batch);
         const size_t partial_need = skinny ? tq::skinny_partial_bytes(V, batch) : 0;
-        // The first call with a larger batch allocates (not capturable in a graph); tq_linear_reserve
-        // sizes the workspaces ahead of time.
-        if (!ensure_stage(&h->d_work, &h->work_bytes, work_need, stream)) return 1;
-        if (skinny && !ensure_stage(&h->d_partial, &h->partial_bytes, partial_need, stream)) return 1;
-        work = h->d_work;
-        partial = static_cast<float*>(h->d_partial);
+        if (static_ws) {
+            if (align256(work_need) + partial_need > (size_t)TQ_STATIC_SCRATCH_BYTES) {
+                set_error("tq_linear_forward_static: this layer and batch need a workspace of " +
+                          std::to_string(align256(work_need) + partial_need) + " bytes, more than the static " +
+                          std::to_string((size_t)TQ_STATIC_SCRATCH_BYTES)); return 1;
+            }
+            work = static_ws;
+            partial = reinterpret_cast<float*>(static_cast<unsigned char*>(static_ws) + align256(work_need));
+        } else {
+            // The first call with a larger batch allocates (not capturable in a graph); tq_linear_reserve
+            // sizes the workspaces ahead of time.
+            if (!ensure_stage(&h->d_work, &h->work_bytes, work_need, stream)) return 1;
+            if (skinny && !ensure_stage(&h->d_partial, &h->partial_bytes, partial_need, stream)) return 1;
+            work = h->d_work;
+            partial = static_cast<float*>(h->d_partial);
+        }
     }
     if (prefill) {
         if (gate) { set_error("tq_linear_forward: gated store is a batch < 16 feature"); return 1; }
@@ -359,6 +401,19 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
         if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < 15 ? max_batch : 15))) return 1;
         return 0;
     } catch (...) { set_error("tq_linear_reserve: exception"); return 1; }
+}
+
+int tq_linear_forward_static(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
+                             void* y_dev, int y_dtype, void* stream) {
+    try {
+        if (!h || !x_dev || !y_dev) { set_error("tq_linear_forward_static: NULL argument"); return 1; }
+        if (batch <= 0 || !dtype_valid(x_dtype) || !dtype_valid(y_dtype)) {
+            set_error("tq_linear_forward_static: bad batch or dtype"); return 1;
+        }
+        void* ws = static_scratch_ptr();
+        if (!ws) return 1;
+        return forward_impl(h, x_dev, x_dtype, batch, y_dev, y_dtype, static_cast<hipStream_t>(stream), nullptr, ws);
+    } catch (...) { set_error("tq_linear_forward_static: exception"); return 1; }
 }
 
 int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int x_dtype, int batch,
