@@ -241,10 +241,11 @@ def test_error_conventions(tq, oracle):
         tq.TurboQuantLinear(256, 8, qw, cbp, cbr, 128)       # shape mismatch
     with pytest.raises(ValueError):
         tq.TurboQuantLinear(128, 8, qw, cbp, cbr, 96)        # block size does not divide
-    q5, c5, c3 = _make(oracle, 8, 128, 128, "5+3dual")
-    layer = tq.TurboQuantLinear(128, 8, q5, c5, c3, 128)
+    with pytest.raises(ValueError):
+        tq.TurboQuantLinear(128, 8, qw, cbp, cbr, 4096)      # block wider than the row
+    layer = tq.TurboQuantLinear(128, 8, qw, cbp, cbr, 128)
     with pytest.raises(RuntimeError):
-        layer.forward(np.zeros((1, 128), np.float32))        # 5-bit with its own residual rotation: dequantise only
+        layer.forward_device(None, tq.F32, 1, None, tq.F32)
     layer.close()
 
 
@@ -347,3 +348,42 @@ def test_forward_random_configurations(tq, oracle, out, inf, bs, mode, batch, xd
     tol = 1e-3 if (xd == "f32" or batch == 1) else 5e-3
     assert y.shape == (batch, out) and np.isfinite(y).all()
     assert _rel(y, want) < tol
+
+
+# ------------------------------------------------------------------ every shape the reference accepts
+def _packed_layer(o, out, inf, bs, mode, seed):
+    """Random packed planes (no quantizer involved: the oracle's dequantiser defines the layer)."""
+    rng = np.random.default_rng(seed)
+    cb = o.generate_codebook(4)
+    pp = rng.integers(0, 256, size=(out, inf // 2)).astype(np.uint8)
+    pr = rng.integers(0, 256, size=(out, inf // 2)).astype(np.uint8)
+    if mode == "primary_only":
+        pr[:] = 0
+    norms = (rng.random(out) + 0.5).astype(np.float32)
+    seeds = np.array([rng.integers(1, 2 ** 32), 0 if mode == "shared" else rng.integers(1, 2 ** 32), bs], np.uint32)
+    return o.QuantizedWeight(pp, pr, norms, seeds), cb
+
+
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("out,inf,bs", [(5, 48, 16), (9, 24, 8), (7, 6, 2), (3, 80, 16), (4, 36, 4), (6, 64, 1),
+                                        (2, 10, 1), (5, 96, 32), (3, 34816, 512), (2, 53248, 512), (3, 36864, 2048)])
+def test_shapes_beyond_the_tuned_kernels(tq, oracle, mode, out, inf, bs):
+    """The reference only requires in % block_size == 0 (src/rotation.cpp:374,396): widths that are not a
+    multiple of 32 (blocks of 1 to 16 columns) and rows wider than 32768 columns load, dequantise bit-exactly,
+    rotate bit-exactly and run forward."""
+    qw, cb = _packed_layer(oracle, out, inf, bs, mode, out * 1000 + inf + bs)
+    w_ref = oracle.dequantize_weight_cpu(qw, cb, cb, bs)
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    assert np.array_equal(layer.dequantize(), w_ref)
+    for batch in (1, 3):
+        x = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
+        y = layer.forward(x)
+        assert y.shape == (batch, out)
+        assert _rel(y, oracle.matmul_xwT(x, w_ref, acc_double=True)) < 1e-3
+        xb = oracle.f32_to_bf16_bits(x)
+        yb = layer.forward(xb, tq.BF16, tq.F32)
+        assert _rel(yb, oracle.matmul_xwT(oracle.bf16_bits_to_f32(xb), w_ref, acc_double=True)) < 5e-3
+    layer.close()
+    x = np.random.default_rng(9).standard_normal((2, inf)).astype(np.float32)
+    assert np.array_equal(tq.apply_wht_rotation(x, 77, bs), oracle.wht_forward(x, 77, bs))
+    assert np.array_equal(tq.apply_inverse_wht_rotation(x, 77, bs), oracle.wht_inverse(x, 77, bs))

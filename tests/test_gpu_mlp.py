@@ -148,16 +148,32 @@ def test_five_bit_primary_fused_forward(tq, oracle, rbits, shared, out_f, in_f, 
     layer.close()
 
 
-def test_five_bit_dual_rotation_still_dequantise_only(tq, oracle):
+@pytest.mark.parametrize("rbits,shared", [(3, False), (4, False), (4, True), (0, False)],
+                         ids=["5+3dual", "5+4dual", "5+4shared", "5+0_long_residual_codebook"])
+@pytest.mark.parametrize("out_f,in_f,bs,batch", [(16, 128, 64, 1), (96, 512, 256, 3), (70, 2048, 512, 1),
+                                                 (33, 5120, 512, 2), (24, 1024, 1024, 20)])
+def test_five_bit_two_plane_forward(tq, oracle, rbits, shared, out_f, in_f, bs, batch):
+    """5-bit primary with its own residual rotation, or with a 4-bit residual (what `--bits 5` of the
+    converter writes by default): byte primary plane + nibble residual plane, two rotations, the case of
+    metal/turboquant_dequant_mm.metal:240-248, 277-292."""
     o = oracle
-    w = o.lcg_matrix(16, 128, 3)
-    cbp, cbr = o.generate_codebook(5), o.generate_codebook(3)
-    qw = o.quantize_weight(w, cbp, cbr, 5, 3, 64, False)
-    layer = tq.TurboQuantLinear(128, 16, qw, cbp, cbr, 64)
-    assert layer.mode() == "dual_5bit"
-    assert np.array_equal(layer.dequantize(), o.dequantize_weight_cpu(qw, cbp, cbr, 64))
-    with pytest.raises(RuntimeError):
-        layer.forward(np.zeros((1, 128), np.float32))
+    w = (np.random.default_rng(5 + out_f).standard_normal((out_f, in_f)) * 0.03).astype(np.float32)
+    cbp = o.generate_codebook(5)
+    cbr = o.generate_codebook(rbits) if rbits else o.generate_codebook(4)   # 16 residual centroids nobody reads
+    qw = o.quantize_weight(w, cbp, cbr, 5, rbits, bs, shared)
+    w_ref = o.dequantize_weight_cpu(qw, cbp, cbr, bs)
+    layer = tq.TurboQuantLinear(in_f, out_f, qw, cbp, cbr, bs)
+    assert layer.mode() == ("primary_only_5bit" if rbits == 0 else "shared_5bit" if shared else "dual_5bit")
+    assert np.array_equal(layer.dequantize(), w_ref)
+    x = np.random.default_rng(batch).standard_normal((batch, in_f)).astype(np.float32)
+    y = layer.forward(x)
+    assert y.shape == (batch, out_f)
+    assert _rel(y, o.matmul_xwT(x, w_ref, acc_double=True)) < 1e-3
+    xb = o.f32_to_bf16_bits(x)
+    yb = layer.forward(xb, tq.BF16, tq.F32)
+    assert _rel(yb, o.matmul_xwT(o.bf16_bits_to_f32(xb), w_ref, acc_double=True)) < 5e-3
+    y16 = o.bf16_bits_to_f32(layer.forward(x.astype(np.float16), tq.F16, tq.BF16))
+    assert _rel(y16, o.matmul_xwT(x.astype(np.float16).astype(np.float32), w_ref, acc_double=True)) < 5e-3
     layer.close()
 
 

@@ -108,13 +108,33 @@ hipError_t launch_codebook_quantize(const float* values, size_t n, const float* 
 hipError_t launch_codebook_lookup(const uint8_t* indices, size_t n, const float* centroids_dev, int nc, float* values,
                                   hipStream_t stream);
 
-// True when the fast wave-per-slab kernels can handle this shape.
+// Generic kernels (tq_generic.hip): any even width that is a multiple of a power-of-two block of 1 to 2048
+// columns, all six modes.  Forward through the layer's fp32 scratch row (xrot_work); dequantiser and
+// rotation for blocks of at most 16 columns (widths that are not a multiple of 32).
+bool generic_supported(const LayerView& L);
+hipError_t launch_gemv_generic(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
+                               int num_cus, hipStream_t stream, const float* gate);
+hipError_t launch_dequant_small(const LayerView& L, void* w, int w_dtype, hipStream_t stream);
+hipError_t launch_wht_small(const float* in, float* out, int rows, int cols, uint32_t seed, uint32_t block_size,
+                            float inv_sqrt_bs, int inverse, hipStream_t stream);
+
+// What the layout itself requires (the reference's only rule is in % block_size == 0,
+// src/rotation.cpp:374,396; its butterfly needs a power of two): blocks of 1 to 2048 columns, an even width.
+inline bool layout_valid(int in_features, uint32_t block_size) {
+    if (in_features <= 0 || (in_features & 1)) return false;
+    if (block_size < 1 || block_size > 2048 || (block_size & (block_size - 1))) return false;
+    return in_features % (int)block_size == 0;
+}
+
+// True when the wave-per-slab kernels (a lane owns 32 consecutive columns) can handle this shape:
+// dequantiser, rotation, quantizer, prefill and small-batch kernels.
+inline bool lanes_supported(int in_features, uint32_t block_size) {
+    return layout_valid(in_features, block_size) && block_size >= 2 && in_features % kChunk == 0;
+}
+
+// True when the batch-1..4 kernels can: additionally at most 16 slabs of 2048 columns per row.
 inline bool shape_supported(int in_features, uint32_t block_size) {
-    if (in_features <= 0 || in_features % kChunk != 0) return false;
-    if (block_size < 2 || block_size > 2048 || (block_size & (block_size - 1))) return false;
-    if (in_features % (int)block_size != 0) return false;
-    if (in_features > 16 * kSlab) return false;
-    return true;
+    return lanes_supported(in_features, block_size) && in_features <= 16 * kSlab;
 }
 
 // ---------------------------------------------------------------------------

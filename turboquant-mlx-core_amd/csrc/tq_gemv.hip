@@ -406,7 +406,7 @@ static hipError_t launch_nb(GemvArgs a, int num_cus, hipStream_t stream) {
 // has the scratch for it and blocks of at most 512 columns) and hand the kernel the result.
 static void pre_rotate(GemvArgs& a, hipStream_t stream) {
     const LayerView& L = a.L;
-    if (!L.xrot_work || L.block_size > (uint32_t)kTile || L.in_features % 8 != 0) return;
+    if (!L.xrot_work || L.block_size > (uint32_t)kTile || L.in_features <= 8 * kSlab) return;
     const int tiles = (L.in_features + kTile - 1) / kTile;
     hipLaunchKernelGGL(tq_rotate_row_kernel, dim3((tiles + 3) / 4, L.mode == kDual ? 2 : 1), dim3(256), 0, stream,
                        a.x, a.x_dtype, a.x_gate, L.xrot_work, L.in_features, L.seed_primary, L.seed_residual, L.block_size);
@@ -460,7 +460,8 @@ static hipError_t launch_mode(const GemvArgs& base, int batch, int num_cus, hipS
 
 // silu(x_gate) * x can be formed on the way where the row goes through tq_rotate_row_kernel.
 bool gemv_x_gate_supported(const LayerView& L) {
-    return L.xrot_work && L.block_size <= (uint32_t)kTile && L.in_features > 8 * kSlab && L.in_features % 8 == 0 &&
+    return L.xrot_work && shape_supported(L.in_features, L.block_size) && L.block_size <= (uint32_t)kTile &&
+           L.in_features > 8 * kSlab &&
            (L.mode == kSharedLut || L.mode == kDual || L.mode == kPrimaryOnly);
 }
 

@@ -33,6 +33,7 @@
 // group by group from a counter in LDS.
 #include "tq_device.h"
 #include "tq_gemv_common.h"
+#include <atomic>
 
 namespace tq {
 
@@ -496,17 +497,18 @@ hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t
     constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
     const size_t lds = (size_t)kRegion + kPartialBytes + (PRE ? 0 : (size_t)a.img_cols * sizeof(float));
     auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE, PT, BOTH>;
-    // More LDS than the default limit has to be asked for, once per kernel and device.
-    static bool asked[64] = {};
+    // More LDS than the default limit has to be asked for, once per kernel and device (any host
+    // thread may get here first; asking twice is harmless).
+    static std::atomic<bool> asked[64];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64 || !asked[dev]) {
+    if (dev < 0 || dev >= 64 || !asked[dev].load(std::memory_order_acquire)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 kRegion + kPartialBytes +
                                     ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float));
         if (e != hipSuccess) return e;
-        if (dev >= 0 && dev < 64) asked[dev] = true;
+        if (dev >= 0 && dev < 64) asked[dev].store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a);
     return hipGetLastError();
@@ -594,17 +596,17 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
 template <int MODE, int R, bool PAIR, bool PT>
 hipError_t launch_group_one(const GemvGroup& g, int grid, int threads, size_t lds, hipStream_t stream) {
     auto* kernel = tq_gemv_wide_group_kernel<MODE, R, PAIR, PT>;
-    static bool asked[64] = {};
+    static std::atomic<bool> asked[64];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64 || !asked[dev]) {
+    if (dev < 0 || dev >= 64 || !asked[dev].load(std::memory_order_acquire)) {
         constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 kRegion + kPartialBytes +
                                     ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float));
         if (e != hipSuccess) return e;
-        if (dev >= 0 && dev < 64) asked[dev] = true;
+        if (dev >= 0 && dev < 64) asked[dev].store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, g);
     return hipGetLastError();
@@ -703,6 +705,7 @@ hipError_t launch_gemv_wide_group(const GemvArgs* as, int n, int num_cus, hipStr
 // 3 to 15, of 1024-column halves.  Dual rotation: rows of 1 to 8 slabs.
 bool gemv_wide_supported(const LayerView& L, int num_cus, bool pre_rotated) {
     if (L.mode != kSharedLut && L.mode != kPrimaryOnly && L.mode != kDual) return false;
+    if (!shape_supported(L.in_features, L.block_size)) return false;
     if (L.block_size > (uint32_t)kTile) return false;
     const int slabs = (L.in_features / kChunk + kWave - 1) / kWave;
     int W = slabs;

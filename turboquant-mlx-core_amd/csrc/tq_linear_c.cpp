@@ -6,6 +6,7 @@
 #include "turboquant_c/tq_linear.h"
 #include "turboquant_c/tq_mlp.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -36,13 +37,15 @@ using tq::set_error;
 using tq::hip_ok;
 
 int device_cu_count() {
-    static int cus = 0;
+    static std::atomic<int> cached{0};          // any host thread may be the first to ask
+    int cus = cached.load(std::memory_order_relaxed);
     if (cus == 0) {
         int dev = 0;
         hipDeviceProp_t prop;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
             cus = prop.multiProcessorCount;
         if (cus <= 0) cus = 256;
+        cached.store(cus, std::memory_order_relaxed);
     }
     return cus;
 }
@@ -147,9 +150,9 @@ tq_linear_t create_impl(int in_features, int out_features,
     if (block_size == 0 || in_features % (int)block_size != 0) {
         set_error("tq_linear_create: in_features must be divisible by block_size"); return nullptr;
     }
-    if (!tq::shape_supported(in_features, block_size)) {
-        set_error("tq_linear_create: unsupported shape (need in_features % 32 == 0, in_features <= 32768, "
-                  "power-of-two block_size in [2, 2048])");
+    if (!tq::layout_valid(in_features, block_size)) {
+        set_error("tq_linear_create: unsupported shape (need an even in_features and a power-of-two block_size "
+                  "in [1, 2048])");
         return nullptr;
     }
 
@@ -204,7 +207,8 @@ tq_linear_t create_impl(int in_features, int out_features,
         (void)hipFree(h->d_residual); h->d_residual = nullptr;
     }
 
-    const bool fused5 = (mode == tq::kShared5 || mode == tq::kPrimaryOnly5) && nr <= 8;
+    // (a primary-only layer never reads its residual codebook, whatever its length)
+    const bool fused5 = (mode == tq::kShared5 && nr <= 8) || mode == tq::kPrimaryOnly5;
     if (fused5) {
         const size_t cbytes = (size_t)out_features * in_features;
         float lut[256];
@@ -241,10 +245,11 @@ tq_linear_t create_impl(int in_features, int out_features,
     v.mode = mode;
     v.inv_scale = 1.0f / std::sqrt(static_cast<float>(in_features));      // src/dequantizer.cpp:76
     v.inv_sqrt_bs = 1.0f / std::sqrt(static_cast<float>(block_size));     // src/rotation.cpp:333
-    if (in_features > 16384) {     // allocated here so that a forward call never allocates on the batch-1 path
-        if (!hip_ok(hipMalloc((void**)&h->d_xrot, (size_t)2 * in_features * sizeof(float)), "hipMalloc(rotated row)")) {
-            delete h; return nullptr;
-        }
+    // Scratch row for the rotated activations of one batch row (both rotations): rows wider than 16384
+    // columns and the generic kernels rotate in a kernel of their own.  Allocated here so that a forward
+    // call never allocates on the batch-1 path.
+    if (!hip_ok(hipMalloc((void**)&h->d_xrot, (size_t)2 * in_features * sizeof(float)), "hipMalloc(rotated row)")) {
+        delete h; return nullptr;
     }
     v.xrot_work = h->d_xrot;
     {
@@ -299,13 +304,18 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 // and nothing is allocated.  Returns 0 on success.
 int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void* y_dev, int y_dtype,
                  hipStream_t stream, const float* gate, void* static_ws = nullptr) {
-    if (h->view.mode >= tq::kShared5 && !h->has_fwd_view) {
-        set_error("tq_linear_forward: 5-bit primary with its own residual rotation or a 4-bit residual is not "
-                  "supported by the fused kernels"); return 1;
-    }
+    // 5-bit primaries with their own residual rotation or a 4-bit residual keep their two planes and run
+    // on the generic kernels, as does every shape the tuned kernels do not take.
+    const bool two_plane5 = h->view.mode >= tq::kShared5 && !h->has_fwd_view;
     const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
-    const bool prefill = tq::prefill_supported(V, x_dtype, batch);
-    const bool skinny = !prefill && !gate && tq::skinny_supported(V, x_dtype, batch);
+    const bool lanes = !two_plane5 && tq::lanes_supported(V.in_features, V.block_size);
+    const bool prefill = lanes && tq::prefill_supported(V, x_dtype, batch);
+    const bool skinny = lanes && !prefill && !gate && tq::skinny_supported(V, x_dtype, batch);
+    if (!prefill && !skinny && (two_plane5 || !tq::shape_supported(V.in_features, V.block_size))) {
+        if (!tq::generic_supported(V)) { set_error("tq_linear_forward: unsupported layer shape"); return 1; }
+        return hip_ok(tq::launch_gemv_generic(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream, gate),
+                      "tq_gemv_generic launch") ? 0 : 1;
+    }
     void* work = nullptr;
     float* partial = nullptr;
     if (prefill || skinny) {
@@ -482,6 +492,9 @@ int tq_linear_dequantize_as(tq_linear_t h, void* w_dev, int w_dtype, void* strea
     try {
         if (!h || !w_dev) { set_error("tq_linear_dequantize: NULL argument"); return 1; }
         if (w_dtype < tq::kF32 || w_dtype > tq::kBF16) { set_error("tq_linear_dequantize: bad dtype"); return 1; }
+        if (!tq::lanes_supported(h->view.in_features, h->view.block_size))     // blocks of 1 to 16 columns
+            return hip_ok(tq::launch_dequant_small(h->view, w_dev, w_dtype, static_cast<hipStream_t>(stream)),
+                          "tq_dequant launch") ? 0 : 1;
         return hip_ok(tq::launch_dequant(h->view, w_dev, w_dtype, static_cast<hipStream_t>(stream)),
                       "tq_dequant launch") ? 0 : 1;
     } catch (...) { set_error("tq_linear_dequantize: exception"); return 1; }
@@ -520,8 +533,15 @@ int tq_wht_rotate(const float* in_dev, float* out_dev, int rows, int cols,
         if (block_size == 0 || cols % (int)block_size != 0) {
             set_error("tq_wht_rotate: in_features must be divisible by block_size"); return 1;
         }
-        if (!tq::shape_supported(cols, block_size)) { set_error("tq_wht_rotate: unsupported shape"); return 1; }
+        if (block_size > 2048 || (block_size & (block_size - 1))) {
+            set_error("tq_wht_rotate: block_size must be a power of two of at most 2048"); return 1;
+        }
         const float inv_sqrt_bs = 1.0f / std::sqrt(static_cast<float>(block_size));
+        if (block_size < 2 || cols % tq::kChunk != 0) {
+            if (block_size > 16) { set_error("tq_wht_rotate: unsupported shape"); return 1; }   // cannot happen: bs divides cols
+            return hip_ok(tq::launch_wht_small(in_dev, out_dev, rows, cols, seed, block_size, inv_sqrt_bs, inverse,
+                                               static_cast<hipStream_t>(stream)), "tq_wht launch") ? 0 : 1;
+        }
         return hip_ok(tq::launch_wht(in_dev, out_dev, rows, cols, seed, block_size, inv_sqrt_bs, inverse,
                                      static_cast<hipStream_t>(stream)), "tq_wht launch") ? 0 : 1;
     } catch (...) { set_error("tq_wht_rotate: exception"); return 1; }

@@ -451,6 +451,9 @@ size_t prefill_workspace_bytes(const LayerView& L, int batch) {
 bool prefill_supported(const LayerView& L, int x_dtype, int batch) {
     if (x_dtype == kF32 || batch < 16) return false;          // fp32 activations keep the exact fp32 GEMV path
     if (L.mode != kSharedLut && L.mode != kDual && L.mode != kPrimaryOnly) return false;
+    if (!lanes_supported(L.in_features, L.block_size)) return false;
+    // (the kernel addresses the index plane with 32-bit byte offsets)
+    if ((unsigned long long)L.out_features * (unsigned long long)L.in_features >= (1ull << 32)) return false;
     return L.in_features % kKLoad == 0;
 }
 

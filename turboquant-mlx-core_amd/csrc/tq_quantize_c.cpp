@@ -42,8 +42,8 @@ bool check_shape(int out, int in, uint32_t bs, const char* who) {
     if (bs == 0 || in % (int)bs != 0) {
         set_error(std::string(who) + ": in_features must be divisible by block_size"); return false;
     }
-    if (!tq::shape_supported(in, bs)) {
-        set_error(std::string(who) + ": unsupported shape (need in_features % 32 == 0, in_features <= 32768, "
+    if (!tq::lanes_supported(in, bs)) {
+        set_error(std::string(who) + ": unsupported shape (the quantizer needs in_features % 32 == 0 and a "
                   "power-of-two block_size in [2, 2048])");
         return false;
     }

@@ -443,6 +443,7 @@ static bool skinny_nibble(const LayerView& L) {
 
 bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
     if (x_dtype == kF32 || batch < 2 || batch >= 16 || L.in_features % kSkChunk != 0) return false;
+    if (!lanes_supported(L.in_features, L.block_size)) return false;
     return (L.mode == kSharedLut && L.packed_combined) || skinny_nibble(L);
 }
 
