@@ -120,7 +120,25 @@ def test_reader_survives_corrupted_headers(tmp_path):
              mutate(lambda h: h["a.weight"].__setitem__("dtype", "F77")),
              mutate(lambda h: h["a.weight"].pop("shape")),
              mutate(lambda h: h.__setitem__("a.weight", "x")),
-             mutate(lambda h: h.__setitem__("__metadata__", {"a": 1}))]
+             mutate(lambda h: h.__setitem__("__metadata__", {"a": 1})),
+             # three dimensions whose product wraps a 64-bit size; dimensions and offsets that are not
+             # whole numbers, not numbers at all, or beyond every integer type
+             mutate(lambda h: h["a.weight"].__setitem__("shape", [2 ** 31 - 1, 2 ** 31 - 1, 2 ** 31 - 1])),
+             mutate(lambda h: h["a.weight"].__setitem__("shape", [8.5, 16])),
+             mutate(lambda h: h["a.weight"].__setitem__("shape", ["8", 16])),
+             mutate(lambda h: h["a.weight"].__setitem__("shape", [1e300, 1])),
+             mutate(lambda h: h["a.weight"].__setitem__("data_offsets", [0, 1e300])),
+             mutate(lambda h: h["a.weight"].__setitem__("data_offsets", [-512, 0])),
+             mutate(lambda h: h["a.weight"].__setitem__("data_offsets", [None, 512]))]
+
+    def raw_header(text, d=data):
+        hb = text.encode()
+        return struct.pack("<Q", len(hb)) + hb + d
+    # numbers std::stod cannot take, and nesting far beyond a header's three levels
+    cases += [raw_header('{"t":{"dtype":"F32","shape":[-],"data_offsets":[0,4]}}'),
+              raw_header('{"t":{"dtype":"F32","shape":[1e99999],"data_offsets":[0,4]}}'),
+              raw_header('{"t":{"dtype":"F32","shape":[+.e],"data_offsets":[0,4]}}'),
+              raw_header("[" * 200000), raw_header('{"a":' * 50000)]
     rnd = random.Random(1)
     for _ in range(200):
         b = bytearray(raw)

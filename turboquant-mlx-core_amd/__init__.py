@@ -111,6 +111,13 @@ class TurboQuantLinear:
         cr = np.ascontiguousarray(residual_codebook.centroids, dtype=np.float32)
         if pp.ndim != 2 or pr.ndim != 2 or pp.shape[0] != out_features or pr.shape[0] != out_features:
             raise ValueError("packed tensors must be [out_features, cols]")
+        # (the C call reads out_features norms and two seeds through raw pointers)
+        if norms.size != out_features:
+            raise ValueError("norms must hold out_features values")
+        if seeds.size < 2:
+            raise ValueError("seeds must hold {seed_primary, seed_residual[, block_size]}")
+        if cp.size < 1 or cr.size < 1:
+            raise ValueError("codebooks must not be empty")
         self._h = lib().tq_linear_create(in_features, out_features, _p(pp, _u8p), pp.shape[1], _p(pr, _u8p),
                                          pr.shape[1], _p(norms, _f32p), _p(seeds, _u32p), _p(cp, _f32p), len(cp),
                                          _p(cr, _f32p), len(cr), block_size)

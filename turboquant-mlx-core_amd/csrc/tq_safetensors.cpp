@@ -6,6 +6,7 @@
 #include "turboquant/serialization.h"
 
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <fstream>
 #include <map>
@@ -37,7 +38,7 @@ public:
     JsonReader(const char* p, size_t n) : p_(p), end_(p + n) {}
 
     Json parse_document() {
-        Json v = value();
+        Json v = value(0);
         skip_ws();
         if (p_ != end_) bad("trailing characters");
         return v;
@@ -112,7 +113,12 @@ private:
         return s;
     }
 
-    Json value() {
+    // A safetensors header nests three levels deep (entry -> shape / data_offsets); anything much deeper
+    // is not a header, and unbounded recursion on "[[[[..." would overflow the stack.
+    static constexpr int kMaxDepth = 8;
+
+    Json value(int depth) {
+        if (depth > kMaxDepth) bad("nested too deeply");
         skip_ws();
         if (p_ >= end_) bad("unexpected end");
         Json v;
@@ -125,14 +131,14 @@ private:
                 skip_ws();
                 std::string key = string();
                 expect(':');
-                v.members.emplace_back(std::move(key), value());
+                v.members.emplace_back(std::move(key), value(depth + 1));
             } while (eat(','));
             expect('}');
         } else if (c == '[') {
             ++p_;
             v.kind = Json::ArrayK;
             if (eat(']')) return v;
-            do { v.items.push_back(value()); } while (eat(','));
+            do { v.items.push_back(value(depth + 1)); } while (eat(','));
             expect(']');
         } else if (c == '"') {
             v.kind = Json::String;
@@ -150,7 +156,8 @@ private:
                 ++p_;
             if (s == p_) bad("unexpected token");
             v.kind = Json::Number;
-            v.num = std::stod(std::string(s, p_));
+            try { v.num = std::stod(std::string(s, p_)); }
+            catch (const std::exception&) { bad("bad number"); }           // "-", "1e99999", ...
         }
         return v;
     }
@@ -198,7 +205,7 @@ Json read_header(std::ifstream& in, const std::string& path, uint64_t* header_le
     if (!in.read(reinterpret_cast<char*>(len8), 8)) throw std::runtime_error("safetensors: cannot read " + path);
     uint64_t n = 0;
     for (int i = 7; i >= 0; --i) n = (n << 8) | len8[i];
-    if (n < 2 || n > (uint64_t(1) << 30)) throw std::runtime_error("safetensors: bad header length in " + path);
+    if (n < 2 || n > 100000000ull) throw std::runtime_error("safetensors: bad header length in " + path);   // 100 MB, the format's own cap
     std::string text((size_t)n, '\0');
     if (!in.read(&text[0], (std::streamsize)n)) throw std::runtime_error("safetensors: truncated header in " + path);
     *header_len = n;
@@ -245,7 +252,9 @@ std::pair<TensorMap, MetadataMap> load_safetensors(const std::string& path) {
     uint64_t header_len = 0;
     const Json root = read_header(in, path, &header_len);
     in.seekg(0, std::ios::end);
-    const uint64_t data_bytes = (uint64_t)in.tellg() - 8 - header_len;
+    const std::streamoff file_end = in.tellg();
+    if (file_end < 0 || (uint64_t)file_end < 8 + header_len) throw std::runtime_error("safetensors: truncated file " + path);
+    const uint64_t data_bytes = (uint64_t)file_end - 8 - header_len;
 
     TensorMap tensors;
     for (const auto& kv : root.members) {
@@ -257,12 +266,26 @@ std::pair<TensorMap, MetadataMap> load_safetensors(const std::string& path) {
         if (e.kind != Json::Object || !dt || !sh || !off || dt->kind != Json::String || sh->kind != Json::ArrayK ||
             off->kind != Json::ArrayK || off->items.size() != 2)
             throw std::runtime_error("safetensors: malformed entry " + kv.first);
+        // Every number is checked before it is converted (a cast of a huge or negative double is undefined),
+        // and the byte count is checked against the offsets and the file before anything is allocated.
+        auto integral = [&](const Json& j, double max) {
+            if (j.kind != Json::Number || !(j.num >= 0.0) || j.num > max || j.num != std::floor(j.num))
+                throw std::runtime_error("safetensors: bad number in entry " + kv.first);
+            return (uint64_t)j.num;
+        };
+        const Dtype dtype = dtype_from_name(dt->str);
         std::vector<int> shape;
-        for (const Json& d : sh->items) shape.push_back((int)d.num);
-        Array a(shape, dtype_from_name(dt->str));
-        const uint64_t b = (uint64_t)off->items[0].num, e2 = (uint64_t)off->items[1].num;
-        if (e2 < b || e2 > data_bytes || e2 - b != a.nbytes())
+        uint64_t count = 1;
+        for (const Json& d : sh->items) {
+            const uint64_t dim = integral(d, 2147483647.0);
+            if (dim != 0 && count > (uint64_t(1) << 62) / dim) throw std::runtime_error("safetensors: shape too large for " + kv.first);
+            count *= dim;
+            shape.push_back((int)dim);
+        }
+        const uint64_t b = integral(off->items[0], 9007199254740992.0), e2 = integral(off->items[1], 9007199254740992.0);
+        if (count > (uint64_t(1) << 62) / 8 || e2 < b || e2 > data_bytes || e2 - b != count * dtype_size(dtype))
             throw std::runtime_error("safetensors: bad data_offsets for " + kv.first);
+        Array a(shape, dtype);
         in.seekg((std::streamoff)(8 + header_len + b));
         if (a.nbytes() && !in.read(a.data<char>(), (std::streamsize)a.nbytes()))
             throw std::runtime_error("safetensors: truncated data for " + kv.first);
