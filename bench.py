@@ -156,6 +156,60 @@ def time_graph(tq, torch, handles, x, y, xcode, batch, steps, warmup, spread=Non
     return time_graph_fn(torch, step, steps, warmup, 1, spread)
 
 
+TIMELINE_MARKS = ["wave started", "first weight rows requested", "decode table written", "before the barrier",
+                  "behind the barrier", "loop entered", "row group 1 stored", "row group 2 (3)", "row group 3 (5)",
+                  "row group 4 (7)", "row group 5 (9)", "row group 6 (11)", "row group 7 (13)", "row group 8 (15)",
+                  "last row group stored", "memory operations complete"]
+
+
+def timeline(tq, torch):
+    """Where the time of a batch-1 launch goes: the timeline build of the library (same sources, wall-clock
+    marks per wave) on three shapes, 300 back-to-back launches, marks of the last one; microseconds from
+    the start of the launch's first wave."""
+    import ctypes as C
+    import numpy as np
+    tq.LIB_PATH = os.path.join(os.path.dirname(tq.LIB_PATH), "libturboquant_amd_timeline.so")
+    L = tq.lib()
+    L.tq_timeline_read.argtypes = [C.c_void_p]
+    for out, inf, dt, code, copies in ((151936, 2048, torch.bfloat16, tq.BF16, 2), (4096, 4096, torch.float32, tq.F32, 16),
+                                       (27648, 5120, torch.bfloat16, tq.BF16, 4)):
+        hs = [make_layer(tq, torch, out, inf, 512, seed=40 + i, sigma=0.02, shared=True)[0] for i in range(copies)]
+        x = torch.randn(1, inf, device="cuda").to(dt)
+        y = torch.empty(1, out, device="cuda", dtype=torch.float32)
+        for i in range(12):
+            if L.tq_linear_forward(hs[i % copies], x.data_ptr(), code, 1, y.data_ptr(), 0, None) != 0:
+                raise RuntimeError(tq.last_error())
+        torch.cuda.synchronize()
+        L.tq_timeline_clear()
+        for i in range(300):
+            L.tq_linear_forward(hs[i % copies], x.data_ptr(), code, 1, y.data_ptr(), 0, None)
+        torch.cuda.synchronize()
+        buf = np.zeros(256 * 16 * 16, np.uint64)
+        if L.tq_timeline_read(buf.ctypes.data) != 0:
+            raise RuntimeError("tq_timeline_read failed")
+        t = buf.reshape(256, 16, 16).astype(np.int64)
+        live = t[:, :, 0] > 0
+        t0 = t[:, :, 0][live].min()
+        print(f"--- {out} x {inf}, shared rotation, batch 1: {int(live.sum())} waves; us from the first wave's start")
+        print(f"  {'mark':34s} {'min':>7s} {'mean':>7s} {'p90':>7s} {'max':>7s}")
+        for k in range(16):
+            col = t[:, :, k][live]
+            col = col[col > 0]
+            if len(col) == 0:
+                continue
+            r = (col - t0) / 100.0
+            print(f"  {k:2d} {TIMELINE_MARKS[k]:31s} {r.min():7.2f} {r.mean():7.2f} {np.percentile(r, 90):7.2f} {r.max():7.2f}")
+        end = np.where(live, (t[:, :, 14] - t0) / 100.0, 0.0).max(axis=1)
+        end = end[end > 0]
+        print(f"  last row group stored, per CU: min {end.min():.2f} mean {end.mean():.2f} max {end.max():.2f}")
+        per_xcd = [float(np.mean([e for b, e in enumerate(np.where(live, (t[:, :, 14] - t0) / 100.0, 0.0).max(axis=1))
+                                  if b % 8 == xc and e > 0])) for xc in range(8)]
+        print("  the same, mean over the CUs of each XCD (workgroup id % 8):", " ".join(f"{v:.2f}" for v in per_xcd))
+        for h in hs:
+            L.tq_linear_free(h)
+        torch.cuda.empty_cache()
+
+
 def cpu_baseline(torch, tensors, out, inf, bs, x_f32):
     """Reference CPU path (dequantize_weight_cpu + fp32 matmul, restated in oracle/) on the
     host cores of this box, whole layer, single thread as the reference's serial loops."""
@@ -191,6 +245,9 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure the headline configuration only")
     ap.add_argument("--decoder-layer-only", action="store_true",
                     help="of the extra measurements, run only the decoder-layer projections (for kernel profiles)")
+    ap.add_argument("--timeline", action="store_true",
+                    help="instead of the benchmark: per-wave wall-clock marks inside the batch-1 kernel (the "
+                         "timeline build of the library), last of 300 back-to-back launches, as a text table")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy three times (reference reading for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -208,6 +265,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.timeline:
+        timeline(tq, torch)
+        return
 
     # ---- headline: lm_head 151936 x 2048, bf16 x, fp32 y, batch 1 -------------------
     out, inf, bs = 151936, 2048, 512
@@ -294,6 +354,10 @@ def main():
         probes["hbm_stream_read_gbs"] = val.value
     for name, rnd in (("mfma_bf16_tflops_ones", 0), ("mfma_bf16_tflops_random_operands", 1)):
         if Lp.tq_probe_mfma_bf16(rnd, 20000, C.byref(val)) == 0:
+            probes[name] = val.value
+    Lp.tq_probe_device_atomics.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+    for name, addresses in (("device_scope_fetch_adds_per_us_one_word", 1), ("device_scope_fetch_adds_per_us_eight_words", 8)):
+        if Lp.tq_probe_device_atomics(addresses, 20, C.byref(val)) == 0:
             probes[name] = val.value
     extra["machine_probes"] = probes
     if "hbm_stream_read_gbs" in probes:

@@ -25,6 +25,14 @@ int tq_probe_hbm_read(size_t bytes, int repeats, double* gb_per_s);
  * it the rate, depends on how many bits toggle.  Returns 0 on success. */
 int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops);
 
+/* One workgroup of 16 waves per CU; every wave does `per_wave` device-scope relaxed fetch-adds on one of
+ * `addresses` (1..64) words, chosen by workgroup; writes the achieved rate in fetch-adds per microsecond
+ * over the whole chip.  What a device-wide work counter could hand out: on MI355X about 90 per
+ * microsecond on one word (11 ns each, whoever asks), which is why the batch-1 kernel hands its row
+ * groups out from counters in LDS and not from one in memory (an lm_head launch has 76 000 of them in
+ * 45 us).  Returns 0 on success. */
+int tq_probe_device_atomics(int addresses, int per_wave, double* per_microsecond);
+
 #ifdef __cplusplus
 }
 #endif

@@ -387,3 +387,29 @@ def test_shapes_beyond_the_tuned_kernels(tq, oracle, mode, out, inf, bs):
     x = np.random.default_rng(9).standard_normal((2, inf)).astype(np.float32)
     assert np.array_equal(tq.apply_wht_rotation(x, 77, bs), oracle.wht_forward(x, 77, bs))
     assert np.array_equal(tq.apply_inverse_wht_rotation(x, 77, bs), oracle.wht_inverse(x, 77, bs))
+
+
+# ------------------------------------------------------------------ many rows of one slab
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("out,inf,bs", [(70001, 512, 512), (66000, 2048, 256), (131074, 1024, 128)])
+def test_one_slab_layers_with_many_rows(tq, oracle, mode, out, inf, bs):
+    """Rows of one slab (the waves of a CU take their row groups from a counter in LDS) on layers of 65536
+    rows and more, odd row counts included: every output against the float64 product with the oracle's
+    weight (no row missing, doubled or misplaced), and the same bits on every call."""
+    qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf)
+    oracle.set_threads(8)
+    w_ref = oracle.dequantize_weight_cpu(qw, cb, cb, bs)
+    oracle.set_threads(1)
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    x = np.random.default_rng(1).standard_normal((1, inf)).astype(np.float32)
+    want = (w_ref.astype(np.float64) @ x[0].astype(np.float64)).astype(np.float32)
+    ys = [layer.forward(x) for _ in range(3)]
+    assert _rel(ys[0][0], want) < 1e-3
+    assert np.abs(ys[0][0] - want).max() < 1e-3 * np.abs(want).max()
+    for y in ys[1:]:
+        assert np.array_equal(y, ys[0])
+    xb = oracle.f32_to_bf16_bits(x)
+    yb = layer.forward(xb, tq.BF16, tq.F32)
+    wantb = (w_ref.astype(np.float64) @ oracle.bf16_bits_to_f32(xb)[0].astype(np.float64)).astype(np.float32)
+    assert _rel(yb[0], wantb) < 1e-3
+    layer.close()

@@ -37,6 +37,20 @@
 
 namespace tq {
 
+// Timeline build (make timeline: libturboquant_amd_timeline.so, used by bench.py --timeline): lane 0 of
+// every wave of the first 256 workgroups notes the 100 MHz wall clock at fixed points of the kernel.
+//   0 wave started            1 first weight rows requested      2 decode table written
+//   3 before the barrier      4 behind the barrier               5 rotated activations in registers (loop entered)
+//   6 .. 13 after the 1st, 2nd, .. 8th row group (rows from the LDS counter: every other group)
+//   14 last row group stored  15 all memory operations of the wave complete
+// In the regular build the marks are nothing.
+#ifdef TQ_TIMELINE
+__device__ unsigned long long g_timeline[256 * 16 * 16];
+#define TQ_MARK(k) do { if (lane == 0 && blockIdx.x < 256) g_timeline[(blockIdx.x * 16 + wave) * 16 + (k)] = wall_clock64(); } while (0)
+#else
+#define TQ_MARK(k) do { } while (0)
+#endif
+
 namespace {
 
 constexpr int kMaxImageCols = 16384;             // widest rotated-activation image in LDS (64 KB)
@@ -143,6 +157,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TQ_MARK(0);
     const int nwaves = blockDim.x >> 6;
     // (divisions cost a few hundred scalar instructions per wave, and all waves of a CU share one
     // scalar unit: the host supplies the quotients)
@@ -255,6 +270,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     __builtin_amdgcn_sched_barrier(0);
     fetch(0, DYN ? r_begin + wave * V : r_begin);
 
+    TQ_MARK(1);
     // Decode tables -> LDS, one private column per lane.
     int* const next_group = reinterpret_cast<int*>(partial);    // DYN: first group nobody has taken yet
     if (DYN && tid == 0) *next_group = 2 * nwaves;              // (groups w and w + nwaves are wave w's first two)
@@ -282,6 +298,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
         }
     }
 
+    TQ_MARK(2);
     if constexpr (PRE) {
         __syncthreads();              // tables visible to every wave
         fetch(1, r_begin + V);
@@ -295,7 +312,9 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     float* const image = reinterpret_cast<float*>(smem + kRegion + kPartialBytes);
     rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_primary, a.L.block_size, image, wave,
                                      nwaves, lane);
+    TQ_MARK(3);
     __syncthreads();                  // image and tables (and the group counter) visible to every wave
+    TQ_MARK(4);
     // The second stage of the ring is requested behind the barrier: a wave whose requests queue up
     // in the memory pipeline would otherwise keep the whole workgroup waiting there.
     fetch(1, DYN ? r_begin + (wave + nwaves) * V : r_begin + V);
@@ -311,6 +330,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
     }
+    TQ_MARK(5);
 
     // One row (or with PAIR the same columns of two rows: p -> sum, q -> sum2).
     auto decode_row = [&](const uint4& p, const uint4& q, float& sum, float& sum2) {
@@ -449,8 +469,11 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
         auto take = [&]() { return __hip_atomic_fetch_add(slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); };
         auto taken = [&](int t) { asm volatile("" : "+v"(t)); return __builtin_amdgcn_readfirstlane(t); };
         int t = take();
+        [[maybe_unused]] int rounds = 0;
         while (g0 < groups) {
             consume(0, r_begin + g0 * V, 0);
+            if (rounds < 8) TQ_MARK(6 + rounds);
+            ++rounds;
             g0 = taken(t);
             t = take();
             fetch(0, r_begin + g0 * V);
@@ -460,6 +483,11 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
             t = take();
             fetch(1, r_begin + g1 * V);
         }
+        TQ_MARK(14);
+#ifdef TQ_TIMELINE
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+        TQ_MARK(15);
         return;
     }
     int it0 = 0;
@@ -467,10 +495,16 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
             consume(u, r_begin + (it0 + u) * V, it0 + u);
+            if (it0 + u < 8) TQ_MARK(6 + it0 + u);
             fetch(u, r_begin + (it0 + u + NS) * V);
         }
     }
     if (it0 < a.iters) consume(0, r_begin + it0 * V, it0);
+    TQ_MARK(14);
+#ifdef TQ_TIMELINE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+    TQ_MARK(15);
 }
 
 template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false, bool BOTH = false>
@@ -735,3 +769,14 @@ hipError_t launch_gemv_wide(const GemvArgs& base, int num_cus, hipStream_t strea
 }
 
 }  // namespace tq
+
+#ifdef TQ_TIMELINE
+// Timeline build only: copies the marks of the last launches to the host / clears them.
+extern "C" int tq_timeline_read(unsigned long long* host) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tq::g_timeline), sizeof(tq::g_timeline));
+}
+extern "C" int tq_timeline_clear(void) {
+    static unsigned long long zeros[256 * 16 * 16];
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(tq::g_timeline), zeros, sizeof(zeros));
+}
+#endif

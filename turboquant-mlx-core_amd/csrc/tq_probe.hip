@@ -1,5 +1,6 @@
-// Two machine probes for the roofline denominators: what this GPU sustains on a pure streaming
-// read and on a pure bf16 MFMA loop.  Measurement support only: nothing in the layer path calls them.
+// Machine probes for the roofline denominators and for design decisions: what this GPU sustains on a pure
+// streaming read, on a pure bf16 MFMA loop, and on device-scope fetch-adds from every wave of the chip.
+// Measurement support only: nothing in the layer path calls them.
 #include "turboquant_c/tq_probe.h"
 
 #include "tq_device.h"
@@ -47,6 +48,20 @@ __global__ __launch_bounds__(512) void tq_probe_mfma_kernel(float* __restrict__ 
     float s = 0.0f;
     for (int i = 0; i < 8; ++i) s += acc[i][0];
     if (s == 123.456f) sink[0] = s;
+}
+
+// Every wave of a one-workgroup-per-CU launch does `per_wave` device-scope relaxed fetch-adds (lane 0) on
+// one of `addresses` words, 256 bytes apart, chosen by workgroup.
+__global__ __launch_bounds__(1024) void tq_probe_atomic_kernel(unsigned* ctr, int per_wave, int addresses, unsigned* sink) {
+    const int lane = threadIdx.x & 63;
+    unsigned* const c = ctr + (blockIdx.x % addresses) * 64;
+    unsigned acc = 0;
+    for (int i = 0; i < per_wave; ++i) {
+        unsigned t = 0;
+        if (lane == 0) t = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        acc += __builtin_amdgcn_readfirstlane(t);
+    }
+    if (acc == 0xdeadbeefu) sink[0] = acc;
 }
 
 }  // namespace tq
@@ -108,6 +123,37 @@ int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops) {
         if (sink) (void)hipFree(sink);
         return ok ? 0 : 1;
     } catch (...) { tq::set_error("tq_probe_mfma_bf16: exception"); return 1; }
+}
+
+int tq_probe_device_atomics(int addresses, int per_wave, double* per_microsecond) {
+    try {
+        if (!per_microsecond || addresses < 1 || addresses > 64 || per_wave < 1) { tq::set_error("tq_probe_device_atomics: bad argument"); return 1; }
+        int dev = 0; hipDeviceProp_t prop;
+        if (!tq::hip_ok(hipGetDevice(&dev), "hipGetDevice") || !tq::hip_ok(hipGetDeviceProperties(&prop, dev), "properties")) return 1;
+        const int cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        unsigned* ctr = nullptr; unsigned* sink = nullptr;
+        hipEvent_t t0 = nullptr, t1 = nullptr;
+        bool ok = tq::hip_ok(hipMalloc((void**)&ctr, 64 * 64 * sizeof(unsigned)), "hipMalloc(counters)") &&
+                  tq::hip_ok(hipMalloc((void**)&sink, 4), "hipMalloc(sink)") &&
+                  tq::hip_ok(hipMemset(ctr, 0, 64 * 64 * sizeof(unsigned)), "hipMemset(counters)") &&
+                  tq::hip_ok(hipEventCreate(&t0), "event") && tq::hip_ok(hipEventCreate(&t1), "event");
+        float ms = 0.0f;
+        const int reps = 5;
+        if (ok) {
+            hipLaunchKernelGGL(tq::tq_probe_atomic_kernel, dim3(cus), dim3(1024), 0, nullptr, ctr, per_wave, addresses, sink);
+            (void)hipEventRecord(t0, nullptr);
+            for (int r = 0; r < reps; ++r)
+                hipLaunchKernelGGL(tq::tq_probe_atomic_kernel, dim3(cus), dim3(1024), 0, nullptr, ctr, per_wave, addresses, sink);
+            (void)hipEventRecord(t1, nullptr);
+            ok = tq::hip_ok(hipEventSynchronize(t1), "probe sync") && tq::hip_ok(hipEventElapsedTime(&ms, t0, t1), "elapsed");
+        }
+        if (ok) *per_microsecond = (double)cus * 16.0 * per_wave * reps / (ms * 1e3);
+        if (t0) (void)hipEventDestroy(t0);
+        if (t1) (void)hipEventDestroy(t1);
+        if (ctr) (void)hipFree(ctr);
+        if (sink) (void)hipFree(sink);
+        return ok ? 0 : 1;
+    } catch (...) { tq::set_error("tq_probe_device_atomics: exception"); return 1; }
 }
 
 }  // extern "C"
