@@ -48,7 +48,6 @@ struct PrefillArgs {
     int M, N, K;
     int mode;
     int m_tiles, n_tiles;
-    int m_major;               // tile order, see the kernel
     float out_scale;
 };
 
@@ -90,24 +89,13 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t laneoff = (uint32_t)lane << 2;
 
-    // XCD-aware tile order: consecutive workgroup ids land on different XCDs (id % 8), each with an L2
-    // of its own.  With few M tiles, the M tiles that share one N tile of weights are given to the same
-    // XCD back to back (the weights are fetched once, every XCD re-reads the few activation images).
-    // From 8 M tiles on (m_major) an XCD keeps ONE activation image (K x 512 bytes: it stays in its L2)
-    // and sweeps the N tiles: every XCD then streams the weights once, which is less traffic than every
-    // XCD re-reading all the activation images for each of its N tiles (2048 tokens: 714 -> 660 us).
+    // XCD-aware tile order: consecutive workgroup ids land on different XCDs (id % 8), so the
+    // M tiles that share one N tile of weights are given to the same XCD back to back.
     const int id = blockIdx.x;
     const int xcd = id & 7, slot = id >> 3;
-    int n_tile, m_tile;
-    if (a.m_major) {
-        m_tile = (slot / a.n_tiles) * 8 + xcd;
-        n_tile = slot % a.n_tiles;
-        if (m_tile >= a.m_tiles) return;                   // whole workgroup leaves together
-    } else {
-        n_tile = (slot / a.m_tiles) * 8 + xcd;
-        m_tile = slot % a.m_tiles;
-        if (n_tile >= a.n_tiles) return;
-    }
+    const int n_tile = (slot / a.m_tiles) * 8 + xcd;
+    const int m_tile = slot % a.m_tiles;
+    if (n_tile >= a.n_tiles) return;                       // whole workgroup leaves together
     const int m0 = m_tile * kBM, n0 = n_tile * kBN;
 
     constexpr bool combined = (MODE == kSharedLut);
@@ -504,9 +492,8 @@ hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int ba
     a.m_tiles = (M + kBM - 1) / kBM;
     a.n_tiles = (N + kBN - 1) / kBN;
     a.out_scale = L.inv_scale * L.inv_sqrt_bs;
-    a.m_major = a.m_tiles >= 8 ? 1 : 0;
-    const unsigned grid = a.m_major ? (unsigned)(((a.m_tiles + 7) / 8) * 8 * a.n_tiles)
-                                    : (unsigned)(((a.n_tiles + 7) / 8) * 8 * a.m_tiles);
+    const int n_groups = (a.n_tiles + 7) / 8;
+    const unsigned grid = (unsigned)(n_groups * 8 * a.m_tiles);
     switch (L.mode) {
         case kSharedLut:
             hipLaunchKernelGGL(tq_prefill_gemm_kernel<kSharedLut>, dim3(grid), dim3(kGemmThreads), 0, stream, a); break;
