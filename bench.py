@@ -23,11 +23,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152512.1 KiB + 606.0 KiB.
-MEASURED_TRAFFIC_BYTES = 312965325
-# Average duration of the headline kernel in the rocprofv3 kernel trace of `python bench.py --skip-extra`
-# (same file), in microseconds, and the kernel's name there.
-PROFILED_KERNEL_US = 49.76
+# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152507.9 KiB + 605.5 KiB.
+MEASURED_TRAFFIC_BYTES = 312956211
+# Average duration of the headline kernel in the rocprofv3 kernel trace of
+# `python bench.py --steps 20 --warmup 5 --no-cpu-baseline --skip-extra` (same file), in microseconds, and the
+# kernel's name there.
+PROFILED_KERNEL_US = 50.28
 HEADLINE_KERNEL = "tq_gemv_wide_kernel<shared, R=2, TILES=1, rows from an LDS counter>"
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
@@ -193,8 +194,7 @@ def timeline(tq, torch):
         print(f"--- {out} x {inf}, shared rotation, batch 1: {int(live.sum())} waves; us from the first wave's start")
         print(f"  {'mark':34s} {'min':>7s} {'mean':>7s} {'p90':>7s} {'max':>7s}")
         for k in range(16):
-            col = t[:, :, k][live]
-            col = col[col > 0]
+            col = t[:, :, k][live & (t[:, :, k] >= t[:, :, 0])]     # a mark older than the wave's start is a previous launch's
             if len(col) == 0:
                 continue
             r = (col - t0) / 100.0
