@@ -78,6 +78,9 @@ struct tq_linear_s {
     void* d_partial = nullptr; size_t partial_bytes = 0;
     // Rotated activation row (both rotations) of the batch-1 path, layers wider than 16384 columns only.
     float* d_xrot = nullptr;
+    // Workspaces that were outgrown: a captured graph may still hold their addresses, so they live as long
+    // as the handle does (each growth at least doubles the size: their sum stays below the current one).
+    std::vector<void*> retired;
 
     ~tq_linear_s() {
         if (d_primary) (void)hipFree(d_primary);
@@ -91,6 +94,7 @@ struct tq_linear_s {
         if (d_work) (void)hipFree(d_work);
         if (d_partial) (void)hipFree(d_partial);
         if (d_xrot) (void)hipFree(d_xrot);
+        for (void* p : retired) (void)hipFree(p);
     }
 };
 
@@ -118,16 +122,26 @@ void build_tables(int mode, const float* cbp, int np, const float* cbr, int nr, 
 
 // Grows a workspace of a handle.  A buffer that a captured graph may still reference is never
 // replaced while the stream is being captured: growth during capture is an error.
-bool ensure_stage(void** buf, size_t* have, size_t need, hipStream_t stream = nullptr) {
+// Grows *buf to at least `need` bytes.  Refused while `stream` is being captured (an allocation cannot be
+// captured).  With `retired`, an outgrown buffer is kept until the handle is freed instead of being freed
+// here, and the new one is at least twice as large.
+bool ensure_stage(void** buf, size_t* have, size_t need, hipStream_t stream = nullptr,
+                  std::vector<void*>* retired = nullptr) {
     if (*have >= need) return true;
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
     if (stream && hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
         set_error("workspace too small while the stream is being captured: call tq_linear_reserve first");
         return false;
     }
-    if (*buf) { (void)hipFree(*buf); *buf = nullptr; *have = 0; }
-    if (!hip_ok(hipMalloc(buf, need), "hipMalloc(staging)")) return false;
-    *have = need;
+    void* fresh = nullptr;
+    const size_t want = (retired && *buf && need < 2 * *have) ? 2 * *have : need;
+    if (!hip_ok(hipMalloc(&fresh, want), "hipMalloc(staging)")) return false;
+    if (*buf) {
+        if (retired) retired->push_back(*buf);
+        else (void)hipFree(*buf);
+    }
+    *buf = fresh;
+    *have = want;
     return true;
 }
 
@@ -332,8 +346,8 @@ int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void
         } else {
             // The first call with a larger batch allocates (not capturable in a graph); tq_linear_reserve
             // sizes the workspaces ahead of time.
-            if (!ensure_stage(&h->d_work, &h->work_bytes, work_need, stream)) return 1;
-            if (skinny && !ensure_stage(&h->d_partial, &h->partial_bytes, partial_need, stream)) return 1;
+            if (!ensure_stage(&h->d_work, &h->work_bytes, work_need, stream, &h->retired)) return 1;
+            if (skinny && !ensure_stage(&h->d_partial, &h->partial_bytes, partial_need, stream, &h->retired)) return 1;
             work = h->d_work;
             partial = static_cast<float*>(h->d_partial);
         }
@@ -407,8 +421,8 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
         if (max_batch < 2) return 0;                       // one row uses no workspace
         const size_t small = tq::skinny_workspace_bytes(V, max_batch < 15 ? max_batch : 15);
         const size_t big = max_batch >= 16 ? tq::prefill_workspace_bytes(V, max_batch) : 0;
-        if (!ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big)) return 1;
-        if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < 15 ? max_batch : 15))) return 1;
+        if (!ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big, nullptr, &h->retired)) return 1;
+        if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < 15 ? max_batch : 15), nullptr, &h->retired)) return 1;
         return 0;
     } catch (...) { set_error("tq_linear_reserve: exception"); return 1; }
 }
@@ -458,7 +472,7 @@ int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int
             // on the first such call (not capturable in a graph), as in tq_linear_forward.
             float* partials[3] = {nullptr, nullptr, nullptr};
             for (int j = 0; j < n; ++j) {
-                if (!ensure_stage(&hs[j]->d_partial, &hs[j]->partial_bytes, tq::skinny_partial_bytes(views[j], batch), st)) return 1;
+                if (!ensure_stage(&hs[j]->d_partial, &hs[j]->partial_bytes, tq::skinny_partial_bytes(views[j], batch), st, &hs[j]->retired)) return 1;
                 partials[j] = static_cast<float*>(hs[j]->d_partial);
             }
             return hip_ok(tq::launch_skinny_group(views, n, x_dev, x_dtype, batch, y_devs, y_dtype, partials,
