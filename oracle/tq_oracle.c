@@ -466,14 +466,17 @@ int tqo_dequantize_weight(const uint8_t* pp, int primary_cols,
     const int shared = (seed_r == 0 && has_residual);                /* :133 */
 
     if (shared && !primary_5bit) {
-        /* path A (:136-184): 256-entry table, zero where p >= n_cbp.  The
+        /* path A (:136-184): 256-entry table, zero where p >= n_cbp, filled by the
+         * reference's loop as written (:144-150): the index is cast to uint8_t, so a
+         * primary codebook of more than 16 entries on nibble planes writes entry
+         * p >= 16 over ((r | 1) << 4) | (p & 15), later writes winning.  The
          * reference reads r_centroids[r] for all r < 16 without a bound check;
          * a shorter residual codebook is clamped here. */
         float lut[256];
         memset(lut, 0, sizeof lut);
         for (int r = 0; r < 16; ++r)
-            for (int p = 0; p < n_cbp && p < 16; ++p)
-                lut[(r << 4) | p] = cbp[p] + cbr[r < n_cbr ? r : n_cbr - 1];
+            for (int p = 0; p < n_cbp; ++p)
+                lut[(uint8_t)((r << 4) | p)] = cbp[p] + cbr[r < n_cbr ? r : n_cbr - 1];
 #pragma omp parallel for num_threads(g_threads) schedule(static)
         for (int row = 0; row < out; ++row) {
             for (int b = 0; b < primary_cols; ++b) {

@@ -87,6 +87,34 @@ def test_dequantize_fitted_codebooks_and_index_clamp(tq, oracle):
         assert np.array_equal(tq.dequantize_weight_gpu(q, cb3, cb3, 128), oracle.dequantize_weight_cpu(q, cb3, cb3, 128))
 
 
+def test_oversized_primary_codebook_on_nibble_planes(tq, oracle):
+    """32 primary centroids under 4-bit planes, shared rotation: the reference's table loop wraps the index
+    at 8 bits (src/dequantizer.cpp:144-150), so odd residual indices select centroids 16..31.  Dequantised
+    weights equal the oracle's bit for bit and every forward path uses the same table."""
+    cb5, cb4 = oracle.generate_codebook(5), oracle.generate_codebook(4)
+    rng = np.random.default_rng(4)
+    out, inf, bs = 40, 1024, 256
+    q = oracle.QuantizedWeight(rng.integers(0, 256, (out, inf // 2), dtype=np.uint8),
+                               rng.integers(0, 256, (out, inf // 2), dtype=np.uint8),
+                               rng.random(out, dtype=np.float32) + 0.5, np.array([99, 0, bs], np.uint32))
+    want = oracle.dequantize_weight_cpu(q, cb5, cb4, bs)
+    capped = oracle.dequantize_weight_cpu(q, oracle.Codebook(cb5.centroids[:16], 4), cb4, bs)
+    assert not np.array_equal(want, capped)                              # the wrap matters on this input
+    assert np.array_equal(tq.dequantize_weight_gpu(q, cb5, cb4, bs), want)
+    layer = tq.TurboQuantLinear(inf, out, q, cb5, cb4, bs)
+    for batch, xd in ((1, "f32"), (3, "f32"), (6, "bf16"), (40, "bf16")):
+        x32 = rng.standard_normal((batch, inf)).astype(np.float32)
+        if xd == "bf16":
+            xbits = oracle.f32_to_bf16_bits(x32)
+            y = layer.forward(xbits, tq.BF16, tq.F32)
+            ref = oracle.matmul_xwT(oracle.bf16_bits_to_f32(xbits), want, acc_double=True)
+        else:
+            y = layer.forward(x32, tq.F32, tq.F32)
+            ref = oracle.matmul_xwT(x32, want, acc_double=True)
+        assert _rel(y, ref) < (1e-3 if xd == "f32" else 5e-3), (batch, xd)
+    layer.close()
+
+
 # ------------------------------------------------------------------ forward
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only", "shared_3bit_res"])
 @pytest.mark.parametrize("out,inf,bs", [(64, 128, 128), (32, 128, 128), (16, 512, 256), (24, 384, 128), (16, 896, 128),

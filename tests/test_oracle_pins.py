@@ -452,3 +452,28 @@ def test_short_primary_codebook_zero_fill_shared_and_clamp_dual(oracle):
     c4 = cb4.centroids.astype(np.float64)
     want = _dense_from_values(c4[p], 1234, bs, norms) + _dense_from_values(cP[np.minimum(r, 7)], 777, bs, norms)
     assert np.abs(W - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+
+
+def test_oversized_primary_codebook_on_nibble_planes_wraps_in_the_shared_table(oracle):
+    """A 32-entry primary codebook under 4-bit planes with shared rotation.  The reference fills its
+    256-entry table with `lut[uint8_t((r << 4) | p)]` for every p below the codebook size
+    (src/dequantizer.cpp:144-150): for p >= 16 bit 4 of p lands in the residual half of the index, and
+    since r ascends in the outer loop and p in the inner one, what remains is, in closed form,
+    entry (r, p) = cP[p] + cR[r] for even r and cP[p + 16] + cR[r] for odd r."""
+    rng = np.random.default_rng(8)
+    out, inf, bs = 5, 128, 32
+    p = rng.integers(0, 16, size=(out, inf)).astype(np.uint8)
+    r = rng.integers(0, 16, size=(out, inf)).astype(np.uint8)
+    pp = oracle.pack4(p).reshape(out, inf // 2)
+    pr = oracle.pack4(r).reshape(out, inf // 2)
+    norms = (rng.random(out) + 0.5).astype(np.float32)
+    cb5, cb4 = oracle.generate_codebook(5), oracle.generate_codebook(4)
+    cP, cR = cb5.centroids.astype(np.float64), cb4.centroids.astype(np.float64)
+    assert len(cP) == 32
+    qs = oracle.QuantizedWeight(pp, pr, norms, np.array([4321, 0, bs], np.uint32))
+    W = oracle.dequantize_weight_cpu(qs, cb5, cb4, bs)
+    vals = np.where(r % 2 == 1, cP[p.astype(int) + 16], cP[p]) + cR[r]
+    want = _dense_from_values(vals, 4321, bs, norms)
+    assert np.abs(W - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+    capped = _dense_from_values(cP[p] + cR[r], 4321, bs, norms)        # a table that stops at p < 16
+    assert np.abs(W - capped).max() > 1e-2

@@ -109,9 +109,11 @@ namespace {
 void build_tables(int mode, const float* cbp, int np, const float* cbr, int nr, float* t) {
     std::memset(t, 0, 256 * sizeof(float));
     if (mode == tq::kSharedLut) {
+        // (the reference's loop as written: the index wraps at 8 bits, so entries p >= 16 of an oversized
+        // primary codebook land on ((r | 1) << 4) | (p & 15) and later writes win)
         for (int r = 0; r < 16; ++r)
-            for (int p = 0; p < np && p < 16; ++p)
-                t[(r << 4) | p] = cbp[p] + cbr[r < nr ? r : nr - 1];
+            for (int p = 0; p < np; ++p)
+                t[(uint8_t)((r << 4) | p)] = cbp[p] + cbr[r < nr ? r : nr - 1];
         return;
     }
     const bool five = mode >= tq::kShared5;
