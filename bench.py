@@ -181,30 +181,31 @@ def timeline(tq, torch):
             if L.tq_linear_forward(hs[i % copies], x.data_ptr(), code, 1, y.data_ptr(), 0, None) != 0:
                 raise RuntimeError(tq.last_error())
         torch.cuda.synchronize()
-        L.tq_timeline_clear()
-        for i in range(300):
-            L.tq_linear_forward(hs[i % copies], x.data_ptr(), code, 1, y.data_ptr(), 0, None)
-        torch.cuda.synchronize()
-        buf = np.zeros(256 * 16 * 16, np.uint64)
-        if L.tq_timeline_read(buf.ctypes.data) != 0:
-            raise RuntimeError("tq_timeline_read failed")
-        t = buf.reshape(256, 16, 16).astype(np.int64)
-        live = t[:, :, 0] > 0
-        t0 = t[:, :, 0][live].min()
-        print(f"--- {out} x {inf}, shared rotation, batch 1: {int(live.sum())} waves; us from the first wave's start")
-        print(f"  {'mark':34s} {'min':>7s} {'mean':>7s} {'p90':>7s} {'max':>7s}")
-        for k in range(16):
-            col = t[:, :, k][live & (t[:, :, k] >= t[:, :, 0])]     # a mark older than the wave's start is a previous launch's
-            if len(col) == 0:
-                continue
-            r = (col - t0) / 100.0
-            print(f"  {k:2d} {TIMELINE_MARKS[k]:31s} {r.min():7.2f} {r.mean():7.2f} {np.percentile(r, 90):7.2f} {r.max():7.2f}")
-        end = np.where(live, (t[:, :, 14] - t0) / 100.0, 0.0).max(axis=1)
-        end = end[end > 0]
-        print(f"  last row group stored, per CU: min {end.min():.2f} mean {end.mean():.2f} max {end.max():.2f}")
-        per_xcd = [float(np.mean([e for b, e in enumerate(np.where(live, (t[:, :, 14] - t0) / 100.0, 0.0).max(axis=1))
-                                  if b % 8 == xc and e > 0])) for xc in range(8)]
-        print("  the same, mean over the CUs of each XCD (workgroup id % 8):", " ".join(f"{v:.2f}" for v in per_xcd))
+        for pass_ in (1, 2):                               # two passes: what persists from launch to launch
+            L.tq_timeline_clear()
+            for i in range(300):
+                L.tq_linear_forward(hs[i % copies], x.data_ptr(), code, 1, y.data_ptr(), 0, None)
+            torch.cuda.synchronize()
+            buf = np.zeros(256 * 16 * 16, np.uint64)
+            if L.tq_timeline_read(buf.ctypes.data) != 0:
+                raise RuntimeError("tq_timeline_read failed")
+            t = buf.reshape(256, 16, 16).astype(np.int64)
+            live = t[:, :, 0] > 0
+            t0 = t[:, :, 0][live].min()
+            print(f"--- {out} x {inf}, shared rotation, batch 1, pass {pass_}: {int(live.sum())} waves; us from the first wave's start")
+            print(f"  {'mark':34s} {'min':>7s} {'mean':>7s} {'p90':>7s} {'max':>7s}")
+            for k in range(16):
+                col = t[:, :, k][live & (t[:, :, k] >= t[:, :, 0])]     # a mark older than the wave's start is a previous launch's
+                if len(col) == 0:
+                    continue
+                r = (col - t0) / 100.0
+                print(f"  {k:2d} {TIMELINE_MARKS[k]:31s} {r.min():7.2f} {r.mean():7.2f} {np.percentile(r, 90):7.2f} {r.max():7.2f}")
+            end = np.where(live, (t[:, :, 14] - t0) / 100.0, 0.0).max(axis=1)
+            end = end[end > 0]
+            print(f"  last row group stored, per CU: min {end.min():.2f} mean {end.mean():.2f} max {end.max():.2f}")
+            per_xcd = [float(np.mean([e for b, e in enumerate(np.where(live, (t[:, :, 14] - t0) / 100.0, 0.0).max(axis=1))
+                                      if b % 8 == xc and e > 0])) for xc in range(8)]
+            print("  the same, mean over the CUs of each XCD (workgroup id % 8):", " ".join(f"{v:.2f}" for v in per_xcd))
         for h in hs:
             L.tq_linear_free(h)
         torch.cuda.empty_cache()
