@@ -97,6 +97,10 @@ class _Hip:
 def _layer(tq, o, out, inf, bs, mode, seed=11):
     w = (np.random.default_rng(seed).standard_normal((out, inf)) * 0.05).astype(np.float32)
     cb = o.generate_codebook(4)
+    if mode == "dual_5bit":                                    # byte primary plane + nibble residual plane
+        cb5 = o.generate_codebook(5)
+        qw = o.quantize_weight(w, cb5, cb, 5, 4, bs, False)
+        return tq.TurboQuantLinear(inf, out, qw, cb5, cb, bs), qw, (cb5, cb)
     if mode == "shared":
         qw = o.quantize_weight(w, cb, cb, 4, 4, bs, True)
     elif mode == "dual":
@@ -117,7 +121,7 @@ def _bits(o, rng, batch, inf):
 BATCHES = (1, 4, 15, 40)          # batch-1 kernel, small-batch kernels (two sizes), prefill kernel
 
 
-@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only", "dual_5bit"])
 def test_reserved_layer_is_captured_and_replayed(tq, oracle, mode):
     o, hip = oracle, _Hip()
     out, inf, bs = 640, 2048, 512
@@ -132,7 +136,8 @@ def test_reserved_layer_is_captured_and_replayed(tq, oracle, mode):
         layer.forward_device(xs[b], tq.BF16, b, eager[b], tq.F32, hip.stream)
     want = {b: hip.download(eager[b], (b, out)) for b in BATCHES}
     # the eager results are right (CPU oracle), so bit-equality below is equality with a checked result
-    w_ref = o.dequantize_weight_cpu(qw, cb, cb, bs)
+    cbs = cb if isinstance(cb, tuple) else (cb, cb)
+    w_ref = o.dequantize_weight_cpu(qw, cbs[0], cbs[1], bs)
     for b in BATCHES:
         ref = o.matmul_xwT(o.bf16_bits_to_f32(xbits[b]), w_ref, acc_double=True)
         assert _rel(want[b], ref) < (1e-3 if b == 1 else 5e-3)

@@ -151,11 +151,14 @@ def test_five_bit_primary_fused_forward(tq, oracle, rbits, shared, out_f, in_f, 
 @pytest.mark.parametrize("rbits,shared", [(3, False), (4, False), (4, True), (0, False)],
                          ids=["5+3dual", "5+4dual", "5+4shared", "5+0_long_residual_codebook"])
 @pytest.mark.parametrize("out_f,in_f,bs,batch", [(16, 128, 64, 1), (96, 512, 256, 3), (70, 2048, 512, 1),
-                                                 (33, 5120, 512, 2), (24, 1024, 1024, 20)])
+                                                 (33, 5120, 512, 2), (24, 1024, 1024, 20), (200, 5120, 512, 6),
+                                                 (96, 2048, 512, 40), (50, 1024, 1024, 2), (300, 3584, 512, 15),
+                                                 (12, 48, 16, 3)])
 def test_five_bit_two_plane_forward(tq, oracle, rbits, shared, out_f, in_f, bs, batch):
     """5-bit primary with its own residual rotation, or with a 4-bit residual (what `--bits 5` of the
     converter writes by default): byte primary plane + nibble residual plane, two rotations, the case of
-    metal/turboquant_dequant_mm.metal:240-248, 277-292."""
+    metal/turboquant_dequant_mm.metal:240-248, 277-292.  One row runs both planes in one generic pass; two
+    or more rows run each plane through the tuned kernels as a layer of its own and add the results."""
     o = oracle
     w = (np.random.default_rng(5 + out_f).standard_normal((out_f, in_f)) * 0.03).astype(np.float32)
     cbp = o.generate_codebook(5)

@@ -99,6 +99,37 @@ def test_static_forward_equals_forward_two_calls_in_a_row(tq, oracle, mode, out,
     layer.close()
 
 
+def test_static_forward_two_plane_five_bit_layer(tq, oracle):
+    """A 5-bit primary with its own residual rotation: at two or more rows the static entry point also
+    keeps the fp32 results of the two planes in the array."""
+    hip = _Hip()
+    o = oracle
+    out, inf, bs = 200, 2048, 512
+    w = (np.random.default_rng(3).standard_normal((out, inf)) * 0.05).astype(np.float32)
+    cbp, cbr = o.generate_codebook(5), o.generate_codebook(4)
+    qw = o.quantize_weight(w, cbp, cbr, 5, 4, bs, False)
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    assert layer.mode() == "dual_5bit"
+    w_ref = o.dequantize_weight_cpu(qw, cbp, cbr, bs)
+    bufs = []
+    for k, (batch, ydt, ynp) in enumerate(((40, tq.F32, np.float32), (6, tq.BF16, np.uint16), (1, tq.F32, np.float32))):
+        xbits = o.f32_to_bf16_bits(np.random.default_rng(60 + k).standard_normal((batch, inf)).astype(np.float32))
+        x_dev = hip.upload(xbits)
+        nb = batch * out * np.dtype(ynp).itemsize
+        y_ref_dev, y_dev = hip.alloc(nb), hip.alloc(nb)
+        layer.forward_device(x_dev, tq.BF16, batch, y_ref_dev, ydt)
+        want = hip.download(y_ref_dev, (batch, out), ynp)
+        layer.forward_static_device(x_dev, tq.BF16, batch, y_dev, ydt)
+        got = hip.download(y_dev, (batch, out), ynp)
+        assert np.array_equal(got, want), f"call {k}, batch {batch}"
+        gf = got if ydt == tq.F32 else o.bf16_bits_to_f32(got)
+        ref = o.matmul_xwT(o.bf16_bits_to_f32(xbits), w_ref, acc_double=True)
+        assert _rel(gf, ref) < (1e-3 if batch == 1 else 5e-3)
+        bufs += [x_dev, y_ref_dev, y_dev]
+    hip.free(*bufs)
+    layer.close()
+
+
 def test_static_forward_refuses_a_workspace_beyond_the_array(tq, oracle):
     hip = _Hip()
     o = oracle

@@ -291,6 +291,20 @@ hipError_t launch_silu_mul(const float* gate, const float* up, void* out, int ou
     return hipGetLastError();
 }
 
+// out[i] = a[i] + b[i] over n fp32 values, written as out_dtype; out may be a itself.
+__global__ void tq_add_kernel(const float* a, const float* __restrict__ b, void* out, int out_dtype, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        store_scalar(out, out_dtype, i, a[i] + b[i]);
+}
+
+hipError_t launch_add(const float* a, const float* b, void* out, int out_dtype, size_t n, hipStream_t stream) {
+    const size_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(tq_add_kernel, dim3((unsigned)(blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks))), dim3(256), 0,
+                       stream, a, b, out, out_dtype, n);
+    return hipGetLastError();
+}
+
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream) {
     hipLaunchKernelGGL(tq_any_nonzero_kernel, dim3(1024), dim3(256), 0, stream, data, n, flag_dev);
     return hipGetLastError();

@@ -53,6 +53,8 @@ hipError_t launch_gemv(const LayerView& L, const void* x, int x_dtype, int batch
 bool gemv_x_gate_supported(const LayerView& L);
 // out[i] = silu(gate[i]) * up[i] over n fp32 values, written as out_dtype (gated MLP, batched path).
 hipError_t launch_silu_mul(const float* gate, const float* up, void* out, int out_dtype, size_t n, hipStream_t stream);
+// out[i] = a[i] + b[i] over n fp32 values, written as out_dtype (out may be a).
+hipError_t launch_add(const float* a, const float* b, void* out, int out_dtype, size_t n, hipStream_t stream);
 hipError_t launch_combine_planes5(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,
                                   size_t residual_bytes, int n_primary, int n_residual, hipStream_t stream);
 hipError_t launch_dequant(const LayerView& L, void* w, int w_dtype, hipStream_t stream);

@@ -114,9 +114,53 @@ __global__ __launch_bounds__(256) void tq_gemv_generic_kernel(GenericArgs a) {
     constexpr int roff = five ? 32 : 16;
     const float* xp = a.xrot;
     const float* xr = a.xrot + in;
+    const bool by_eight = (in & 7) == 0;                     // uniform: widths that allow 8-byte loads of a row
     for (int row = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6); row < out; row += (int)gridDim.x * 4) {
         float sp = 0.0f, sr = 0.0f;
-        for (int u = lane; u < pairs; u += kWave) {
+        // Eight consecutive columns per lane and step: one 8- or 4-byte load per plane, two 16-byte loads per
+        // rotated activation vector (the byte-wise loop below is left for widths that are not a multiple of 8).
+        for (int c = 8 * lane; by_eight && c < in; c += 8 * kWave) {
+            uint32_t p[8], r[8];
+            if constexpr (combined || five) {
+                const uint2 w = *reinterpret_cast<const uint2*>((combined ? a.L.packed_combined : a.L.packed_primary) + (size_t)row * in + c);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { p[j] = (w.x >> (8 * j)) & 255u; p[4 + j] = (w.y >> (8 * j)) & 255u; }
+                if constexpr (five) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) p[j] = p[j] > 31u ? 31u : p[j];
+                }
+            } else {
+                const uint32_t w = *reinterpret_cast<const uint32_t*>(a.L.packed_primary + (size_t)row * pairs + (c >> 1));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { p[2 * j] = (w >> (8 * j)) & 15u; p[2 * j + 1] = (w >> (8 * j + 4)) & 15u; }
+            }
+            if constexpr (has_res && !combined) {
+                const uint32_t w = *reinterpret_cast<const uint32_t*>(a.L.packed_residual + (size_t)row * pairs + (c >> 1));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { r[2 * j] = (w >> (8 * j)) & 15u; r[2 * j + 1] = (w >> (8 * j + 4)) & 15u; }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) r[j] = 0;
+            }
+            const float4 xa = *reinterpret_cast<const float4*>(xp + c), xb = *reinterpret_cast<const float4*>(xp + c + 4);
+            const float x[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+            if constexpr (combined || !has_res) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sp = __builtin_fmaf(tab[p[j]], x[j], sp);
+            } else if constexpr (dual) {
+                const float4 ya = *reinterpret_cast<const float4*>(xr + c), yb = *reinterpret_cast<const float4*>(xr + c + 4);
+                const float y[8] = {ya.x, ya.y, ya.z, ya.w, yb.x, yb.y, yb.z, yb.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    sp = __builtin_fmaf(tab[p[j]], x[j], sp);
+                    sr = __builtin_fmaf(tab[roff + r[j]], y[j], sr);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sp = __builtin_fmaf(tab[p[j]] + tab[roff + r[j]], x[j], sp);
+            }
+        }
+        for (int u = lane; !by_eight && u < pairs; u += kWave) {
             const int c = 2 * u;
             uint32_t p0, p1, r0 = 0, r1 = 0;
             if constexpr (combined) {

@@ -6,6 +6,7 @@
 #include "turboquant_c/tq_linear.h"
 #include "turboquant_c/tq_mlp.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdio>
@@ -67,6 +68,15 @@ struct tq_linear_s {
     float* d_tables_fwd = nullptr;
     tq::LayerView fwd_view{};
     bool has_fwd_view = false;
+    // 5-bit primary that keeps its two planes (own residual rotation, or a 4-bit residual): each plane by
+    // itself is a layer the tuned kernels take, plane_view[0] the byte plane as a one-byte-per-weight
+    // layer with the table cP[min(b, nP - 1)], plane_view[1] the residual nibbles as a primary-only layer
+    // with the residual codebook and the residual's rotation; the layer is their sum (two or more rows).
+    tq::LayerView plane_view[2]{};
+    bool has_plane_views = false;
+    float* d_tables_plane[2] = {nullptr, nullptr};
+    // fp32 [batch, out] partial results of the two planes.
+    void* d_sum = nullptr; size_t sum_bytes = 0;
     int primary_cols = 0;
     int residual_cols = 0;
     // Staging for the *_host entry points, grown on demand.
@@ -94,6 +104,9 @@ struct tq_linear_s {
         if (d_work) (void)hipFree(d_work);
         if (d_partial) (void)hipFree(d_partial);
         if (d_xrot) (void)hipFree(d_xrot);
+        if (d_tables_plane[0]) (void)hipFree(d_tables_plane[0]);
+        if (d_tables_plane[1]) (void)hipFree(d_tables_plane[1]);
+        if (d_sum) (void)hipFree(d_sum);
         for (void* p : retired) (void)hipFree(p);
     }
 };
@@ -279,6 +292,34 @@ tq_linear_t create_impl(int in_features, int out_features,
         h->fwd_view.mode = tq::kSharedLut;
         h->fwd_view.tables = h->d_tables_fwd;
         h->has_fwd_view = true;
+    } else if (mode >= tq::kShared5 && tq::lanes_supported(in_features, block_size)) {
+        float ta[256], tb[256];
+        std::memset(tb, 0, sizeof(tb));
+        for (int b = 0; b < 256; ++b) ta[b] = cbp[b < np ? b : np - 1];          // index clamp of src/dequantizer.cpp:94
+        for (int i = 0; i < 16; ++i) tb[i] = cbr[i < nr ? i : nr - 1];            // :103
+        ok = hip_ok(hipMalloc((void**)&h->d_tables_plane[0], sizeof(ta)), "hipMalloc(tables)") &&
+             hip_ok(hipMalloc((void**)&h->d_tables_plane[1], sizeof(tb)), "hipMalloc(tables)") &&
+             hip_ok(hipMemcpy(h->d_tables_plane[0], ta, sizeof(ta), hipMemcpyHostToDevice), "copy tables") &&
+             hip_ok(hipMemcpy(h->d_tables_plane[1], tb, sizeof(tb), hipMemcpyHostToDevice), "copy tables");
+        if (!ok) { delete h; return nullptr; }
+        tq::LayerView& a = h->plane_view[0];
+        a = v;
+        a.mode = tq::kSharedLut;
+        a.packed_combined = h->d_primary;
+        a.packed_primary = nullptr;
+        a.packed_residual = nullptr;
+        a.tables = h->d_tables_plane[0];
+        a.seed_residual = 0;
+        tq::LayerView& b = h->plane_view[1];
+        b = v;
+        b.mode = tq::kPrimaryOnly;
+        b.packed_primary = h->d_residual;
+        b.packed_residual = nullptr;
+        b.packed_combined = nullptr;
+        b.tables = h->d_tables_plane[1];
+        b.seed_primary = mode == tq::kDual5 ? seeds[1] : seeds[0];
+        b.seed_residual = 0;
+        h->has_plane_views = true;
     }
     return h;
 }
@@ -318,16 +359,14 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 // [batch, out]; the batch-1..15 kernel then stores silu(gate) * y.  static_ws: the workspaces of the
 // matrix-core paths come from there (TQ_STATIC_SCRATCH_BYTES) instead of the handle's own buffers,
 // and nothing is allocated.  Returns 0 on success.
-int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void* y_dev, int y_dtype,
-                 hipStream_t stream, const float* gate, void* static_ws = nullptr) {
-    // 5-bit primaries with their own residual rotation or a 4-bit residual keep their two planes and run
-    // on the generic kernels, as does every shape the tuned kernels do not take.
-    const bool two_plane5 = h->view.mode >= tq::kShared5 && !h->has_fwd_view;
-    const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
-    const bool lanes = !two_plane5 && tq::lanes_supported(V.in_features, V.block_size);
+// One layer view through the tuned kernels (or the generic ones where they do not take its shape).
+// static_ws / static_cap: the caller's share of the static array, or NULL: the handle's own workspaces.
+int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, const void* x_dev, int x_dtype, int batch,
+                 void* y_dev, int y_dtype, hipStream_t stream, const float* gate, void* static_ws, size_t static_cap) {
+    const bool lanes = !generic_only && tq::lanes_supported(V.in_features, V.block_size);
     const bool prefill = lanes && tq::prefill_supported(V, x_dtype, batch);
     const bool skinny = lanes && !prefill && !gate && tq::skinny_supported(V, x_dtype, batch);
-    if (!prefill && !skinny && (two_plane5 || !tq::shape_supported(V.in_features, V.block_size))) {
+    if (!prefill && !skinny && (generic_only || !tq::shape_supported(V.in_features, V.block_size))) {
         if (!tq::generic_supported(V)) { set_error("tq_linear_forward: unsupported layer shape"); return 1; }
         return hip_ok(tq::launch_gemv_generic(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream, gate),
                       "tq_gemv_generic launch") ? 0 : 1;
@@ -338,10 +377,10 @@ int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void
         const size_t work_need = prefill ? tq::prefill_workspace_bytes(V, batch) : tq::skinny_workspace_bytes(V, batch);
         const size_t partial_need = skinny ? tq::skinny_partial_bytes(V, batch) : 0;
         if (static_ws) {
-            if (align256(work_need) + partial_need > (size_t)TQ_STATIC_SCRATCH_BYTES) {
+            if (align256(work_need) + partial_need > static_cap) {
                 set_error("tq_linear_forward_static: this layer and batch need a workspace of " +
-                          std::to_string(align256(work_need) + partial_need) + " bytes, more than the static " +
-                          std::to_string((size_t)TQ_STATIC_SCRATCH_BYTES)); return 1;
+                          std::to_string(align256(work_need) + partial_need + ((size_t)TQ_STATIC_SCRATCH_BYTES - static_cap)) +
+                          " bytes, more than the static " + std::to_string((size_t)TQ_STATIC_SCRATCH_BYTES)); return 1;
             }
             work = static_ws;
             partial = reinterpret_cast<float*>(static_cast<unsigned char*>(static_ws) + align256(work_need));
@@ -367,6 +406,47 @@ int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void
     }
     return hip_ok(tq::launch_gemv(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream, gate),
                   "tq_gemv launch") ? 0 : 1;
+}
+
+// Bytes of fp32 partial results a two-plane 5-bit layer needs for `batch` rows written as y_dtype.
+size_t plane_sum_bytes(const tq_linear_s* h, int batch, int y_dtype) {
+    return align256((size_t)batch * h->view.out_features * sizeof(float)) * (y_dtype == tq::kF32 ? 1 : 2);
+}
+
+int forward_impl(tq_linear_s* h, const void* x_dev, int x_dtype, int batch, void* y_dev, int y_dtype,
+                 hipStream_t stream, const float* gate, void* static_ws = nullptr) {
+    // 5-bit primaries with their own residual rotation or a 4-bit residual keep their two planes.  One
+    // row runs on the generic kernels (both planes in one pass); two or more rows run each plane through
+    // the tuned kernels as a layer of its own and add the two results: y = P x~p + R x~r, the same sum the
+    // reference's kernel forms per element (metal/turboquant_dequant_mm.metal:240-248, 277-292).
+    const bool two_plane5 = h->view.mode >= tq::kShared5 && !h->has_fwd_view;
+    const size_t cap = (size_t)TQ_STATIC_SCRATCH_BYTES;
+    if (two_plane5 && batch >= 2 && !gate && h->has_plane_views) {
+        const size_t one = align256((size_t)batch * h->view.out_features * sizeof(float));
+        const size_t need = plane_sum_bytes(h, batch, y_dtype);
+        unsigned char* sums = nullptr;
+        void* sub_ws = nullptr;
+        size_t sub_cap = 0;
+        if (static_ws) {
+            if (need >= cap) {
+                set_error("tq_linear_forward_static: this layer and batch need a workspace of more than the static " +
+                          std::to_string(cap) + " bytes"); return 1;
+            }
+            sums = static_cast<unsigned char*>(static_ws);
+            sub_ws = sums + need;
+            sub_cap = cap - need;
+        } else {
+            if (!ensure_stage(&h->d_sum, &h->sum_bytes, need, stream, &h->retired)) return 1;
+            sums = static_cast<unsigned char*>(h->d_sum);
+        }
+        float* const t1 = reinterpret_cast<float*>(sums);
+        float* const t0 = y_dtype == tq::kF32 ? static_cast<float*>(y_dev) : reinterpret_cast<float*>(sums + one);
+        if (forward_view(h, h->plane_view[0], false, x_dev, x_dtype, batch, t0, tq::kF32, stream, nullptr, sub_ws, sub_cap) != 0) return 1;
+        if (forward_view(h, h->plane_view[1], false, x_dev, x_dtype, batch, t1, tq::kF32, stream, nullptr, sub_ws, sub_cap) != 0) return 1;
+        return hip_ok(tq::launch_add(t0, t1, y_dev, y_dtype, (size_t)batch * h->view.out_features, stream), "tq_add launch") ? 0 : 1;
+    }
+    const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
+    return forward_view(h, V, two_plane5, x_dev, x_dtype, batch, y_dev, y_dtype, stream, gate, static_ws, static_ws ? cap : 0);
 }
 
 extern "C" {
@@ -419,8 +499,22 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
 int tq_linear_reserve(tq_linear_t h, int max_batch) {
     try {
         if (!h || max_batch <= 0) { set_error("tq_linear_reserve: bad argument"); return 1; }
-        const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
         if (max_batch < 2) return 0;                       // one row uses no workspace
+        if (h->has_plane_views) {                          // two planes, each a layer of its own, plus their fp32 results
+            size_t work = 0, part = 0;
+            for (int k = 0; k < 2; ++k) {
+                const tq::LayerView& P = h->plane_view[k];
+                const size_t small = tq::skinny_workspace_bytes(P, max_batch < 15 ? max_batch : 15);
+                const size_t big = max_batch >= 16 ? tq::prefill_workspace_bytes(P, max_batch) : 0;
+                work = std::max(work, std::max(small, big));
+                part = std::max(part, tq::skinny_partial_bytes(P, max_batch < 15 ? max_batch : 15));
+            }
+            if (!ensure_stage(&h->d_work, &h->work_bytes, work, nullptr, &h->retired)) return 1;
+            if (!ensure_stage(&h->d_partial, &h->partial_bytes, part, nullptr, &h->retired)) return 1;
+            if (!ensure_stage(&h->d_sum, &h->sum_bytes, plane_sum_bytes(h, max_batch, tq::kBF16), nullptr, &h->retired)) return 1;
+            return 0;
+        }
+        const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
         const size_t small = tq::skinny_workspace_bytes(V, max_batch < 15 ? max_batch : 15);
         const size_t big = max_batch >= 16 ? tq::prefill_workspace_bytes(V, max_batch) : 0;
         if (!ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big, nullptr, &h->retired)) return 1;
