@@ -493,16 +493,23 @@ def main():
     L = tq.lib()
     shapes = [("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120, 5120),
               ("gate", 27648, 5120), ("up", 27648, 5120), ("down", 5120, 27648)]
-    layers = [(n_, o_, i_, make_layer(tq, torch, o_, i_, bs, seed=900 + k, sigma=0.01, shared=True,
-                                      per_layer_codebooks=True)[0]) for k, (n_, o_, i_) in enumerate(shapes)]
+    # two decoder layers of 488 MB alternate, as the two lm_head copies do: no call finds its weights in the
+    # last-level cache
+    layer_sets = [[(n_, o_, i_, make_layer(tq, torch, o_, i_, bs, seed=900 + 20 * c + k, sigma=0.01, shared=True,
+                                           per_layer_codebooks=True)[0]) for k, (n_, o_, i_) in enumerate(shapes)]
+                  for c in range(2)]
+    layers = layer_sets[0]
     for batch in (1, 4, 8):
         xs = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
         ys = {o_: torch.empty(batch, o_, device="cuda", dtype=torch.float32) for o_ in (5120, 1024, 27648)}
 
+        turn = [0]
+
         def layer_step(s):
-            for n_, o_, i_, h in layers:
+            for n_, o_, i_, h in layer_sets[turn[0] % 2]:
                 if L.tq_linear_forward(h, xs[i_].data_ptr(), tq.BF16, batch, ys[o_].data_ptr(), tq.F32, s) != 0:
                     raise RuntimeError(tq.last_error())
+            turn[0] += 1
         us_l = time_graph_fn(torch, layer_step, max(args.steps // 10, 10), 2, 7)[0] * 1e6
         Bl = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
         extra[f"decoder_layer_projections_32b_bs{batch}"] = {
@@ -511,17 +518,18 @@ def main():
     # The same seven projections at batch 1 with the layers that read the same activation row sharing a
     # launch (tq_linear_forward_group): q, k, v; o; gate, up; down (+ the rotation of its 27648-wide row).
     import ctypes as C
-    by = {n_: h for n_, _, _, h in layers}
+    by = [{n_: h for n_, _, _, h in ls} for ls in layer_sets]
     out_of = {n_: o_ for n_, o_, _, _ in layers}
     L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
                                           C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
-    def grouped(by, tag):
+    def grouped(sets, tag):
         for batch in (1, 4, 8):
             xg = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
-            yg = {n_: torch.empty(batch, out_of[n_], device="cuda", dtype=torch.float32) for n_ in by}
+            yg = {n_: torch.empty(batch, out_of[n_], device="cuda", dtype=torch.float32) for n_ in sets[0]}
+            turn = [0]
 
             def group(names, x, s):
-                hs = (C.c_void_p * len(names))(*[by[n_] for n_ in names])
+                hs = (C.c_void_p * len(names))(*[sets[turn[0] % 2][n_] for n_ in names])
                 yp = (C.c_void_p * len(names))(*[yg[n_].data_ptr() for n_ in names])
                 if L.tq_linear_forward_group(hs, len(names), x.data_ptr(), tq.BF16, batch, yp, tq.F32, s) != 0:
                     raise RuntimeError(tq.last_error())
@@ -531,6 +539,7 @@ def main():
                 group(("o",), xg[5120], s)
                 group(("gate", "up"), xg[5120], s)
                 group(("down",), xg[27648], s)
+                turn[0] += 1
             us_g = time_graph_fn(torch, grouped_step, max(args.steps // 10, 10), 2, 4)[0] * 1e6
             Bg = sum(algorithmic_bytes(o_, i_, batch, 2, 4) for _, o_, i_, _ in layers)
             extra[f"decoder_layer_projections_32b_bs{batch}{tag}_grouped_launches"] = {
@@ -538,14 +547,17 @@ def main():
                 "hbm_frac": Bg / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBS,
                 "calls": "q+k+v, o, gate+up, down through tq_linear_forward_group"}
     grouped(by, "")
-    for _, _, _, h in layers:
-        L.tq_linear_free(h)
-    # the same layer in the converter's default format: dual rotation (include/turboquant/quantizer.h:15)
-    dual = {n_: make_layer(tq, torch, o_, i_, bs, seed=950 + k, sigma=0.01, shared=False, per_layer_codebooks=True)[0]
-            for k, (n_, o_, i_) in enumerate(shapes)}
+    for ls in layer_sets:
+        for _, _, _, h in ls:
+            L.tq_linear_free(h)
+    torch.cuda.empty_cache()
+    # the same layers in the converter's default format: dual rotation (include/turboquant/quantizer.h:15)
+    dual = [{n_: make_layer(tq, torch, o_, i_, bs, seed=950 + 20 * c + k, sigma=0.01, shared=False,
+                            per_layer_codebooks=True)[0] for k, (n_, o_, i_) in enumerate(shapes)} for c in range(2)]
     grouped(dual, "_dual_rotation")
-    for h in dual.values():
-        L.tq_linear_free(h)
+    for d in dual:
+        for h in d.values():
+            L.tq_linear_free(h)
     finish(args, torch, extra, result)
 
 
