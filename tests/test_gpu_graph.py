@@ -164,37 +164,38 @@ def test_growth_is_refused_while_capturing_and_capture_survives(tq, oracle):
     layer, qw, cb = _layer(tq, o, out, inf, bs, "shared")     # no reserve
     L = tq.lib()
     rng = np.random.default_rng(6)
-    x1, x4, x12, x64 = (hip.upload(_bits(o, rng, b, inf)) for b in (1, 4, 12, 64))
+    x1, x9, x15, x64 = (hip.upload(_bits(o, rng, b, inf)) for b in (1, 9, 15, 64))
     y1, y1g = hip.alloc(out * 4), hip.alloc(out * 4)
-    y4, y4g = hip.alloc(4 * out * 4), hip.alloc(4 * out * 4)
-    y12, y64 = hip.alloc(12 * out * 4), hip.alloc(64 * out * 4)
+    y9, y9g = hip.alloc(9 * out * 4), hip.alloc(9 * out * 4)
+    y15, y64 = hip.alloc(15 * out * 4), hip.alloc(64 * out * 4)
     layer.forward_device(x1, tq.BF16, 1, y1, tq.F32, hip.stream)
     want1 = hip.download(y1, (1, out))
-    hip.fill(y4g, 4 * out * 4, 0)
+    hip.fill(y9g, 9 * out * 4, 0)
     hip.begin_capture()
-    rc = L.tq_linear_forward(layer._h, x4, tq.BF16, 4, y4g, tq.F32, hip.stream)
+    # nine rows go through per-chunk partial products in a workspace the layer does not have yet
+    rc = L.tq_linear_forward(layer._h, x9, tq.BF16, 9, y9g, tq.F32, hip.stream)
     message = tq.last_error()
     layer.forward_device(x1, tq.BF16, 1, y1g, tq.F32, hip.stream)      # one row needs no workspace: captured
     graph = hip.end_capture()
     assert rc != 0 and "tq_linear_reserve" in message
     hip.replay(graph[1])
     assert np.array_equal(hip.download(y1g, (1, out)), want1)
-    assert not hip.download(y4g, (4, out)).any()               # the refused call launched nothing
+    assert not hip.download(y9g, (9, out)).any()               # the refused call launched nothing
     # outside a capture the same call allocates and runs; afterwards it can be captured
-    layer.forward_device(x4, tq.BF16, 4, y4, tq.F32, None)
-    want4 = hip.download(y4, (4, out))
+    layer.forward_device(x9, tq.BF16, 9, y9, tq.F32, None)
+    want9 = hip.download(y9, (9, out))
     hip.begin_capture()
-    layer.forward_device(x4, tq.BF16, 4, y4g, tq.F32, hip.stream)
-    graph4 = hip.end_capture()
-    # larger batches outgrow the workspaces graph4 holds; the old ones must stay valid for graph4
-    layer.forward_device(x12, tq.BF16, 12, y12, tq.F32, None)
+    layer.forward_device(x9, tq.BF16, 9, y9g, tq.F32, hip.stream)
+    graph9 = hip.end_capture()
+    # larger batches outgrow the workspaces graph9 holds; the old ones must stay valid for graph9
+    layer.forward_device(x15, tq.BF16, 15, y15, tq.F32, None)
     layer.forward_device(x64, tq.BF16, 64, y64, tq.F32, None)
     for _ in range(3):
-        hip.fill(y4g, 4 * out * 4)
-        hip.replay(graph4[1])
-        assert np.array_equal(hip.download(y4g, (4, out)), want4)
+        hip.fill(y9g, 9 * out * 4)
+        hip.replay(graph9[1])
+        assert np.array_equal(hip.download(y9g, (9, out)), want9)
     hip.drop(graph)
-    hip.drop(graph4)
+    hip.drop(graph9)
     layer.close()
     hip.close()
 
