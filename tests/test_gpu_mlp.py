@@ -117,6 +117,47 @@ def test_mlp_block_matches_oracle(tq, oracle, shared, hidden, inter, bs, batch, 
         l.close()
 
 
+@pytest.mark.parametrize("batch,x_dt", [(1, "bf16"), (1, "f32"), (5, "bf16"), (3, "f32"), (24, "bf16")])
+def test_mlp_block_of_five_bit_two_plane_layers(tq, oracle, batch, x_dt):
+    """The block over layers in the default output format of `tq-convert --bits 5` (5-bit primary, 4-bit residual
+    with its own rotation): one row on the generic kernels with the gate folded into the store, more rows with
+    each plane through the tuned kernels."""
+    hip = _Hip()
+    o = oracle
+    hidden, inter, bs = 512, 1536, 256
+    cb5, cb4 = o.generate_codebook(5), o.generate_codebook(4)
+    layers, refs = [], []
+    for k, (out_f, in_f) in enumerate(((inter, hidden), (inter, hidden), (hidden, inter))):
+        w = (np.random.default_rng(30 + k).standard_normal((out_f, in_f)) * 0.05).astype(np.float32)
+        qw = o.quantize_weight(w, cb5, cb4, 5, 4, bs, False)
+        layers.append(tq.TurboQuantLinear(in_f, out_f, qw, cb5, cb4, bs))
+        assert layers[-1].mode() == "dual_5bit"
+        refs.append(o.dequantize_weight_cpu(qw, cb5, cb4, bs))
+    mlp = tq.TurboQuantMLP(layers[0], layers[1], layers[2], max_batch=batch)
+    x32 = np.random.default_rng(batch).standard_normal((batch, hidden)).astype(np.float32)
+    if x_dt == "bf16":
+        xbits = o.f32_to_bf16_bits(x32)
+        x_ref, x_dev, code = o.bf16_bits_to_f32(xbits), hip.upload(xbits), tq.BF16
+    else:
+        x_ref, x_dev, code = x32, hip.upload(x32), tq.F32
+    y_dev = hip.alloc(batch * hidden * 4)
+    for _ in range(2):
+        mlp.forward_device(x_dev, code, batch, y_dev, tq.F32)
+        y = hip.download(y_dev, (batch, hidden), np.float32)
+    act = _silu(o.matmul_xwT(x_ref, refs[0], acc_double=True)) * o.matmul_xwT(x_ref, refs[1], acc_double=True)
+    if batch >= 2 and x_dt == "bf16":
+        act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))
+    want = o.matmul_xwT(act.astype(np.float32), refs[2], acc_double=True)
+    # One linear on the matrix-core paths is within 5e-3 (test_five_bit_two_plane_forward, same layers).  The
+    # block is two of them in sequence, each with two separately rounded planes: independent roundings add in
+    # quadrature, 5e-3 * sqrt(2); measured 4.9e-3 at 5 rows and 5.0e-3 at 24.
+    assert _rel(y, want) < (1e-3 if (x_dt == "f32" or batch == 1) else 7.1e-3)
+    mlp.close()
+    hip.free(x_dev, y_dev)
+    for l in layers:
+        l.close()
+
+
 def test_mlp_create_rejects_mismatched_layers(tq, oracle):
     a, _ = _layer(tq, oracle, 256, 128, 128, True, 1)
     b, _ = _layer(tq, oracle, 128, 128, 128, True, 2)
