@@ -402,3 +402,49 @@ def test_cli_convert_then_dequant_model_directory(tmp_path, oracle, per_layer, s
             assert rel < 0.15, (k, rel)                              # the bound of the reference's own round-trip tests
         else:
             assert np.array_equal(got, v.astype(np.float32))
+
+
+@pytest.mark.gpu
+def test_cli_convert_five_bit_default_output_runs_forward(tmp_path, oracle):
+    """`tq-convert --bits 5` with its defaults writes a 5-bit primary plane (one index per byte) and a 4-bit
+    residual with its own rotation.  Such a file loads, dequantises to the oracle's bits and runs forward,
+    one row and several, through the same entry points as a 4-bit file."""
+    import __graft_entry__ as entry
+    tq = entry.load_package()
+    rng = np.random.default_rng(11)
+    src = tmp_path / "model"
+    src.mkdir()
+    (src / "config.json").write_text(json.dumps({"model_type": "toy", "num_hidden_layers": 1}))
+    w = (rng.standard_normal((96, 1024)) * 0.03).astype(np.float32)
+    save_file({"model.layers.0.mlp.up_proj.weight": w, "model.norm.weight": np.ones(64, np.float32)},
+              str(src / "model.safetensors"))
+    out = tmp_path / "model-tq5"
+    p = subprocess.run([os.path.join(CLI, "tq-convert"), "--model", str(src), "--output", str(out), "--bits", "5"],
+                       capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stdout + p.stderr
+    meta = _metadata(str(out / "model.safetensors"))
+    assert meta["tq_primary_bits"] == "5" and meta["tq_residual_bits"] == "4"
+    t = load_file(str(out / "model.safetensors"))
+    name = "model.layers.0.mlp.up_proj"
+    pp, pr = t[name + ".packed_primary"], t[name + ".packed_residual"]
+    assert pp.shape == (96, 1024) and pr.shape == (96, 512) and int(pp.max()) < 32
+    seeds = t[name + ".seeds"]
+    assert seeds[1] != 0 and seeds[2] == 512                           # own residual rotation, block 512
+    cbp, cbr = oracle.Codebook(t["tq_codebook_primary"], 5), oracle.Codebook(t["tq_codebook_residual"], 4)
+    assert len(cbp.centroids) == 32 and len(cbr.centroids) == 16
+    qw = oracle.QuantizedWeight(pp, pr, t[name + ".norms"], seeds)
+    w_ref = oracle.dequantize_weight_cpu(qw, cbp, cbr, 512)
+    assert np.linalg.norm(w_ref - w) / np.linalg.norm(w) < 0.15       # the bound of the reference's own round-trip tests
+    layer = tq.TurboQuantLinear(1024, 96, qw, cbp, cbr, 512)
+    assert layer.mode() == "dual_5bit"
+    assert np.array_equal(layer.dequantize(), w_ref)
+    for batch in (1, 6, 20):
+        x = rng.standard_normal((batch, 1024)).astype(np.float32)
+        y = layer.forward(x)
+        ref = oracle.matmul_xwT(x, w_ref, acc_double=True)
+        assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 1e-3
+        xb = oracle.f32_to_bf16_bits(x)
+        yb = layer.forward(xb, tq.BF16, tq.F32)
+        refb = oracle.matmul_xwT(oracle.bf16_bits_to_f32(xb), w_ref, acc_double=True)
+        assert np.linalg.norm(yb - refb) / np.linalg.norm(refb) < (1e-3 if batch == 1 else 5e-3)
+    layer.close()
