@@ -23,12 +23,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch on the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152507.9 KiB + 605.5 KiB.
-MEASURED_TRAFFIC_BYTES = 312956211
+# (profiles/gemv_lm_head_151936x2048_bs1.txt): 2.0 * 152506.3 KiB + 605.5 KiB.
+MEASURED_TRAFFIC_BYTES = 312952934
 # Average duration of the headline kernel in the rocprofv3 kernel trace of
 # `python bench.py --steps 20 --warmup 5 --no-cpu-baseline --skip-extra` (same file), in microseconds, and the
 # kernel's name there.
-PROFILED_KERNEL_US = 50.28
+PROFILED_KERNEL_US = 50.03
 HEADLINE_KERNEL = "tq_gemv_wide_kernel<shared, R=2, TILES=1, rows from an LDS counter>"
 REFERENCE_PUBLISHED_TOK_S = 47.3      # reference README.md:79-82, 151936x2048 batch 1, Apple Silicon
 
@@ -343,7 +343,7 @@ def main():
     del tensors
     torch.cuda.empty_cache()
 
-    # ---- what this machine sustains: streaming read and bf16 MFMA loop (roofline denominators) ----
+    # ---- what this machine sustains: streaming read and MFMA loops (roofline denominators) ----
     extra = {}
     import ctypes as C
     Lp = tq.lib()
@@ -355,6 +355,11 @@ def main():
         probes["hbm_stream_read_gbs"] = val.value
     for name, rnd in (("mfma_bf16_tflops_ones", 0), ("mfma_bf16_tflops_random_operands", 1)):
         if Lp.tq_probe_mfma_bf16(rnd, 20000, C.byref(val)) == 0:
+            probes[name] = val.value
+    # (the prefill kernel multiplies in fp16: same nominal rate, more toggling mantissa bits)
+    Lp.tq_probe_mfma_f16.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+    for name, rnd in (("mfma_f16_tflops_ones", 0), ("mfma_f16_tflops_random_operands", 1)):
+        if Lp.tq_probe_mfma_f16(rnd, 20000, C.byref(val)) == 0:
             probes[name] = val.value
     Lp.tq_probe_device_atomics.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
     for name, addresses in (("device_scope_fetch_adds_per_us_one_word", 1), ("device_scope_fetch_adds_per_us_eight_words", 8)):
@@ -448,7 +453,7 @@ def main():
                                                       "speed_relative_to_vendor_plain_gemm": usv / usp,
                                                       "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
                                                       "frac_of_measured_mfma_loop_random_operands":
-                                                          flops / usp / 1e6 / probes.get("mfma_bf16_tflops_random_operands",
+                                                          flops / usp / 1e6 / probes.get("mfma_f16_tflops_random_operands",
                                                                                          float("nan")),
                                                       "includes": "activation rotation kernel + dequant/MFMA GEMM kernel"}
         tq.lib().tq_linear_free(hp)

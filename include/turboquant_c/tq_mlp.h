@@ -14,7 +14,7 @@
  * codebooks, so each rotates the activation for itself.  Batch 1 and fp32 activations:
  * the gate is folded into the store of the up projection (three kernels in all).  Two
  * or more rows of 16-bit activations: the three layers run on the matrix cores with
- * one elementwise kernel in between, the activation handed on as bf16.
+ * one elementwise kernel in between, the activation handed on as fp32 (16 rows or more) or bf16.
  */
 
 #include "tq_linear.h"

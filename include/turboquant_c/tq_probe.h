@@ -3,7 +3,7 @@
 
 /*
  * Machine probes behind the roofline figures of the benchmark: what this GPU sustains on a
- * pure streaming read and on a pure bf16 MFMA loop.  No counterpart in the reference (its
+ * pure streaming read and on a pure bf16 or fp16 MFMA loop.  No counterpart in the reference (its
  * benchmarks report wall-clock only, benchmarks/bench_linear.cpp:50-76); nothing in the
  * layer path calls these.
  */
@@ -24,6 +24,10 @@ int tq_probe_hbm_read(size_t bytes, int repeats, double* gb_per_s);
  * uses all-ones operands, 1 uses pseudo-random values in (-1, 1): the sustained clock, and with
  * it the rate, depends on how many bits toggle.  Returns 0 on success. */
 int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops);
+
+/* The same loop with v_mfma_f32_32x32x16_f16, the instruction of the prefill kernel: same nominal rate,
+ * more mantissa bits that toggle. */
+int tq_probe_mfma_f16(int random_operands, int iterations, double* tflops);
 
 /* One workgroup of 16 waves per CU; every wave does `per_wave` device-scope relaxed fetch-adds on one of
  * `addresses` (1..64) words, chosen by workgroup; writes the achieved rate in fetch-adds per microsecond

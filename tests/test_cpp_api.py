@@ -181,10 +181,10 @@ def test_cpp_api_against_oracle(tmp_path, oracle, out_f, in_f, bs, batch):
         xb = o.bf16_bits_to_f32(o.f32_to_bf16_bits(x))
         yb_ref = o.matmul_xwT(xb, w_ref, acc_double=True)
         rel = np.linalg.norm(res[tag + "y_bf16_in"] - yb_ref) / np.linalg.norm(yb_ref)
-        assert rel < (1e-3 if batch == 1 else 5e-3), rel                    # bf16 activations: batch 1 exact fp32 kernel,
-                                                                            # more rows the bf16-weight MFMA kernel
+        assert rel < 1e-3, rel                                              # bf16 activations: batch 1 exact fp32 kernel,
+                                                                            # more rows the fp16-weight MFMA kernels
         rel = np.linalg.norm(res[tag + "y_f16"].astype(np.float32) - y_ref) / np.linalg.norm(y_ref)
-        assert rel < 5e-3, rel                                              # half-precision in and out
+        assert rel < 2e-3, rel                                              # half-precision in (rounds x itself) and out
 
     rot = o.wht_forward(w, 0x1234, bs)
     assert np.array_equal(res["rotated"], rot)
@@ -446,5 +446,5 @@ def test_cli_convert_five_bit_default_output_runs_forward(tmp_path, oracle):
         xb = oracle.f32_to_bf16_bits(x)
         yb = layer.forward(xb, tq.BF16, tq.F32)
         refb = oracle.matmul_xwT(oracle.bf16_bits_to_f32(xb), w_ref, acc_double=True)
-        assert np.linalg.norm(yb - refb) / np.linalg.norm(refb) < (1e-3 if batch == 1 else 5e-3)
+        assert np.linalg.norm(yb - refb) / np.linalg.norm(refb) < 1e-3
     layer.close()

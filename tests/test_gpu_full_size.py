@@ -122,7 +122,7 @@ def test_up_projection_27648x5120_prefill_512_tokens(tq, oracle):
     rows = np.sort(np.random.default_rng(13).choice(out_f, 256, replace=False))
     w_rows = o.dequantize_weight_cpu(_rows_subset(o, qw, rows), cb, cb, bs)
     want = o.matmul_xwT(x, w_rows, acc_double=True)                      # [512, 256]
-    assert _rel(y[:, rows], want) < 5e-3                                 # bf16 tiles + bf16 rounding of the outputs
+    assert _rel(y[:, rows], want) < 5e-3                                 # fp16 tiles (3e-4) + bf16 rounding of the outputs (2^-9)
     # the batch-1 kernel (fp32 weights, fp32 accumulate) on three of the tokens
     for tkn in (0, 255, 511):
         y1 = layer.forward(xbits[tkn:tkn + 1], tq.BF16, tq.F32)
@@ -285,7 +285,8 @@ def test_up_projection_27648x5120_prefill_2048_tokens(tq, oracle):
 @pytest.mark.parametrize("batch", [4, 8])
 def test_down_projection_5120x27648_small_batch(tq, oracle, batch, shared):
     """32B-shaped down projection, 54 chunks of 512 columns, 4 and 8 rows of bf16 activations: the
-    small-batch matrix-core path (bf16 weights, fp32 accumulation)."""
+    small-batch matrix-core path (fp16 weights and rotated activations, fp32 accumulation): 1e-3 with fp32
+    outputs, 5e-3 where the outputs are rounded to bf16."""
     o = oracle
     out_f, in_f, bs = 5120, 27648, 512
     layer, w_ref, qw, cp, cr = _full_layer(tq, o, out_f, in_f, bs, 0.01, 51, shared)
@@ -294,15 +295,15 @@ def test_down_projection_5120x27648_small_batch(tq, oracle, batch, shared):
     y = layer.forward(xbits, tq.BF16, tq.F32)
     assert y.shape == (batch, out_f)
     want = (x.astype(np.float64) @ w_ref.astype(np.float64).T).astype(np.float32)
-    assert _rel(y, want) < 5e-3
+    assert _rel(y, want) < 1e-3
     for b in range(batch):
-        assert _rel(y[b], want[b]) < 5e-3
+        assert _rel(y[b], want[b]) < 1e-3
     rows = np.sort(np.random.default_rng(53).choice(out_f, 256, replace=False))
     want_rows = o.matmul_xwT(x, o.dequantize_weight_cpu(_rows_subset(o, qw, rows), cp, cr, bs), acc_double=True)
-    assert _rel(y[:, rows], want_rows) < 5e-3
+    assert _rel(y[:, rows], want_rows) < 1e-3
     yb = o.bf16_bits_to_f32(layer.forward(xbits, tq.BF16, tq.BF16))
     assert _rel(yb, want) < 5e-3
     y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)          # exact fp32 batch-1 kernel
     assert _rel(y1[0], want[batch - 1]) < 1e-3
-    assert _rel(y[batch - 1:batch], y1) < 5e-3
+    assert _rel(y[batch - 1:batch], y1) < 1e-3
     layer.close()

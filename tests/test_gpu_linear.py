@@ -249,7 +249,9 @@ def test_forward_half_activations(tq, oracle, mode, xd, yd):
         y = oracle.bf16_bits_to_f32(y)
     y = y.astype(np.float32)
     want = oracle.linear_forward(qw, cbp, cbr, bs, xin)
-    assert _rel(y, want) < 5e-3
+    # three rows run on the matrix cores with fp16 weights and rotated activations (about 3e-4); a bf16
+    # output adds its own rounding (2^-9 relative)
+    assert _rel(y, want) < (5e-3 if yd == "bf16" else 1e-3)
 
 
 def test_forward_fitted_codebooks_match_dequant_matmul(tq, oracle):
@@ -285,8 +287,9 @@ def test_error_conventions(tq, oracle):
                                               (70, 64, 64, 16), (40, 192, 64, 20), (33, 256, 256, 300),
                                               (257, 384, 128, 513)])
 def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, batch):
-    """batch >= 16 with 16-bit activations takes the MFMA path (bf16 weight tiles, bf16 rotated
-    activations, fp32 accumulation): 5e-3 relative L2 against dequantise + fp32 matmul."""
+    """batch >= 16 takes the MFMA path whatever the activation type (fp16 weight tiles, fp16 rotated
+    activations, fp32 accumulation): 1e-3 relative L2 against dequantise + fp32 matmul, 5e-3 where the
+    output itself is rounded to bf16."""
     qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
     x32 = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
     xbits = oracle.f32_to_bf16_bits(x32)
@@ -295,16 +298,18 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
     y = layer.forward(xbits, tq.BF16, tq.F32)
     yb = oracle.bf16_bits_to_f32(layer.forward(xbits, tq.BF16, tq.BF16))
     y16 = layer.forward(x32.astype(np.float16), tq.F16, tq.F32)
+    y32 = layer.forward(x32)
     layer.close()
     assert y.shape == (batch, out)
-    assert _rel(y, want) < 5e-3
+    assert _rel(y, want) < 1e-3
     assert _rel(yb, want) < 5e-3                      # includes the bf16 rounding of the outputs
-    assert _rel(y16, oracle.linear_forward(qw, cbp, cbr, bs, x32.astype(np.float16).astype(np.float32))) < 5e-3
+    assert _rel(y16, oracle.linear_forward(qw, cbp, cbr, bs, x32.astype(np.float16).astype(np.float32))) < 1e-3
+    assert _rel(y32, oracle.linear_forward(qw, cbp, cbr, bs, x32)) < 1e-3      # fp32 activations take the same path
     # every row of the batch must agree with the batch-1 kernel on the same row
     layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
     y1 = layer.forward(xbits[3:4], tq.BF16, tq.F32)
     layer.close()
-    assert _rel(y[3:4], y1) < 5e-3
+    assert _rel(y[3:4], y1) < 1e-3
 
 
 # ------------------------------------------------------------------ small batches on the matrix cores
@@ -313,9 +318,9 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
                                               (1000, 5120, 512, 8), (16, 512, 64, 3), (47, 1536, 128, 9)])
 def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, inf, bs, batch):
     """2..15 rows of 16-bit activations on a layer whose width is a multiple of 512 take the
-    small-batch MFMA kernels (bf16 weights and rotated activations, fp32 accumulation over
+    small-batch MFMA kernels (fp16 weights and rotated activations, fp32 accumulation over
     512-column chunks; for dual rotation one pass per plane, each with its own rotation):
-    5e-3 relative L2, ragged row counts, every row equal to its batch-1 result."""
+    1e-3 relative L2 (5e-3 with a bf16 output), ragged row counts, every row equal to its batch-1 result."""
     qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
     x32 = np.random.default_rng(100 + batch).standard_normal((batch, inf)).astype(np.float32)
     xbits = oracle.f32_to_bf16_bits(x32)
@@ -323,16 +328,16 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
     y = layer.forward(xbits, tq.BF16, tq.F32)
     assert y.shape == (batch, out)
-    assert _rel(y, want) < 5e-3
+    assert _rel(y, want) < 1e-3
     for b in range(batch):                                   # no row leaks into another
-        assert _rel(y[b:b + 1], want[b:b + 1]) < 5e-3
+        assert _rel(y[b:b + 1], want[b:b + 1]) < 1e-3
     yb = oracle.bf16_bits_to_f32(layer.forward(xbits, tq.BF16, tq.BF16))
     assert _rel(yb, want) < 5e-3
     x16 = x32.astype(np.float16)
     y16 = layer.forward(x16, tq.F16, tq.F32)
-    assert _rel(y16, oracle.linear_forward(qw, cbp, cbr, bs, x16.astype(np.float32))) < 5e-3
+    assert _rel(y16, oracle.linear_forward(qw, cbp, cbr, bs, x16.astype(np.float32))) < 1e-3
     y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)      # exact fp32 batch-1 kernel
-    assert _rel(y[batch - 1:batch], y1) < 5e-3
+    assert _rel(y[batch - 1:batch], y1) < 1e-3
     # fp32 activations keep the exact path at any batch
     yf = layer.forward(x32)
     assert _rel(yf, oracle.linear_forward(qw, cbp, cbr, bs, x32)) < 1e-3
@@ -358,9 +363,8 @@ def _random_cases(n, seed):
 @pytest.mark.parametrize("out,inf,bs,mode,batch,xd", _random_cases(160, 20240611))
 def test_forward_random_configurations(tq, oracle, out, inf, bs, mode, batch, xd):
     """Whatever kernel a call is routed to (one-workgroup-per-CU, pre-rotated, narrow, small-batch or
-    prefill): the output agrees with the oracle's dense product on the same quantised weights, within
-    1e-3 for fp32 activations and single rows, 5e-3 where bf16 weights are used (2+ rows of 16-bit
-    activations)."""
+    prefill): the output agrees with the oracle's dense product on the same quantised weights within
+    1e-3, also where fp16 weights are used (2+ rows of 16-bit activations, 16+ rows of any type)."""
     qw, cbp, cbr = _make(oracle, out, inf, bs, mode, seed=out + inf)
     x32 = np.random.default_rng(out * 7 + batch).standard_normal((batch, inf)).astype(np.float32)
     if xd == "bf16":
@@ -373,9 +377,8 @@ def test_forward_random_configurations(tq, oracle, out, inf, bs, mode, batch, xd
     y = layer.forward(xarg, code, tq.F32)
     layer.close()
     want = oracle.linear_forward(qw, cbp, cbr, bs, xin)
-    tol = 1e-3 if (xd == "f32" or batch == 1) else 5e-3
     assert y.shape == (batch, out) and np.isfinite(y).all()
-    assert _rel(y, want) < tol
+    assert _rel(y, want) < 1e-3
 
 
 # ------------------------------------------------------------------ every shape the reference accepts

@@ -104,10 +104,12 @@ def test_mlp_block_matches_oracle(tq, oracle, shared, hidden, inter, bs, batch, 
         y = hip.download(y_dev, (batch, hidden), np.float32)
 
     act = _silu(o.matmul_xwT(x_ref, wg, acc_double=True)) * o.matmul_xwT(x_ref, wu, acc_double=True)
-    if batch >= 2 and x_dt == "bf16":
-        act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))   # handed to the matrix-core paths as bf16
+    if 2 <= batch < 16 and x_dt == "bf16":
+        act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))   # handed to the small-batch kernel as bf16
     want = o.matmul_xwT(act.astype(np.float32), wd, acc_double=True)
-    tol = 1e-3 if (x_dt == "f32" or batch == 1) else 5e-3   # three bf16-weight layers in a row
+    # two or more rows of 16-bit activations: the activation between the linears is handed on as bf16 below 16
+    # rows (2^-9 relative), as fp32 from 16 rows on; the linears themselves keep fp16 weights (3e-4)
+    tol = 1e-3 if (x_dt == "f32" or batch == 1 or batch >= 16) else 5e-3
     assert _rel(y, want) < tol
     with pytest.raises(RuntimeError):
         mlp.forward_device(x_dev, code, batch + 1, y_dev, tq.F32)
@@ -145,13 +147,10 @@ def test_mlp_block_of_five_bit_two_plane_layers(tq, oracle, batch, x_dt):
         mlp.forward_device(x_dev, code, batch, y_dev, tq.F32)
         y = hip.download(y_dev, (batch, hidden), np.float32)
     act = _silu(o.matmul_xwT(x_ref, refs[0], acc_double=True)) * o.matmul_xwT(x_ref, refs[1], acc_double=True)
-    if batch >= 2 and x_dt == "bf16":
+    if 2 <= batch < 16 and x_dt == "bf16":
         act = o.bf16_bits_to_f32(o.f32_to_bf16_bits(act.astype(np.float32)))
     want = o.matmul_xwT(act.astype(np.float32), refs[2], acc_double=True)
-    # One linear on the matrix-core paths is within 5e-3 (test_five_bit_two_plane_forward, same layers).  The
-    # block is two of them in sequence, each with two separately rounded planes: independent roundings add in
-    # quadrature, 5e-3 * sqrt(2); measured 4.9e-3 at 5 rows and 5.0e-3 at 24.
-    assert _rel(y, want) < (1e-3 if (x_dt == "f32" or batch == 1) else 7.1e-3)
+    assert _rel(y, want) < (1e-3 if (x_dt == "f32" or batch == 1 or batch >= 16) else 5e-3)
     mlp.close()
     hip.free(x_dev, y_dev)
     for l in layers:
@@ -185,7 +184,7 @@ def test_five_bit_primary_fused_forward(tq, oracle, rbits, shared, out_f, in_f, 
     assert _rel(y, o.matmul_xwT(x, w_ref, acc_double=True)) < 1e-3
     xb = o.f32_to_bf16_bits(x)
     yb = layer.forward(xb, tq.BF16, tq.F32)
-    assert _rel(yb, o.matmul_xwT(o.bf16_bits_to_f32(xb), w_ref, acc_double=True)) < 5e-3
+    assert _rel(yb, o.matmul_xwT(o.bf16_bits_to_f32(xb), w_ref, acc_double=True)) < 1e-3
     layer.close()
 
 
@@ -215,7 +214,7 @@ def test_five_bit_two_plane_forward(tq, oracle, rbits, shared, out_f, in_f, bs, 
     assert _rel(y, o.matmul_xwT(x, w_ref, acc_double=True)) < 1e-3
     xb = o.f32_to_bf16_bits(x)
     yb = layer.forward(xb, tq.BF16, tq.F32)
-    assert _rel(yb, o.matmul_xwT(o.bf16_bits_to_f32(xb), w_ref, acc_double=True)) < 5e-3
+    assert _rel(yb, o.matmul_xwT(o.bf16_bits_to_f32(xb), w_ref, acc_double=True)) < 1e-3
     y16 = o.bf16_bits_to_f32(layer.forward(x.astype(np.float16), tq.F16, tq.BF16))
     assert _rel(y16, o.matmul_xwT(x.astype(np.float16).astype(np.float32), w_ref, acc_double=True)) < 5e-3
     layer.close()
@@ -304,7 +303,7 @@ def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):
         yg = hip.download(ys_group[j], (batch, o), np.float32)
         y1 = hip.download(ys_single[j], (batch, o), np.float32)
         assert np.array_equal(yg, y1)
-        assert _rel(yg, xin @ dense[j].T) < 5e-3
+        assert _rel(yg, xin @ dense[j].T) < 1e-3
     hip.free(dx, *ys_group, *ys_single)
     for layer in layers:
         layer.close()

@@ -93,7 +93,7 @@ def test_static_forward_equals_forward_two_calls_in_a_row(tq, oracle, mode, out,
         got = hip.download(y_dev, (batch, out), np.float32)
         assert np.array_equal(got, want), f"call {k}, batch {batch}"      # same kernels: bit-exact
         ref = o.matmul_xwT(o.bf16_bits_to_f32(xbits), w_ref, acc_double=True)
-        assert _rel(got, ref) < (1e-3 if batch == 1 else 5e-3)            # and right, against the CPU oracle
+        assert _rel(got, ref) < 1e-3                                      # and right, against the CPU oracle
         bufs += [x_dev, y_ref_dev, y_dev]
     hip.free(*bufs)
     layer.close()
@@ -124,7 +124,7 @@ def test_static_forward_two_plane_five_bit_layer(tq, oracle):
         assert np.array_equal(got, want), f"call {k}, batch {batch}"
         gf = got if ydt == tq.F32 else o.bf16_bits_to_f32(got)
         ref = o.matmul_xwT(o.bf16_bits_to_f32(xbits), w_ref, acc_double=True)
-        assert _rel(gf, ref) < (1e-3 if batch == 1 else 5e-3)
+        assert _rel(gf, ref) < (5e-3 if ydt == tq.BF16 else 1e-3)      # (a bf16 output adds its own rounding)
         bufs += [x_dev, y_ref_dev, y_dev]
     hip.free(*bufs)
     layer.close()

@@ -58,7 +58,7 @@ hipError_t launch_add(const float* a, const float* b, void* out, int out_dtype, 
 hipError_t launch_combine_planes5(const uint8_t* primary, const uint8_t* residual, uint8_t* combined,
                                   size_t residual_bytes, int n_primary, int n_residual, hipStream_t stream);
 hipError_t launch_dequant(const LayerView& L, void* w, int w_dtype, hipStream_t stream);
-// Prefill (tq_prefill.hip): rotate the activations to bf16 in `workspace`, then dequant + MFMA GEMM.
+// Prefill (tq_prefill.hip): rotate the activations to fp16 in `workspace`, then dequant + MFMA GEMM.
 bool prefill_supported(const LayerView& L, int x_dtype, int batch);
 size_t prefill_workspace_bytes(const LayerView& L, int batch);
 hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
@@ -236,6 +236,14 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
     if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
+}
+
+// fp32 -> fp16 bit pattern, round to nearest even; values beyond the largest finite fp16 saturate (a
+// rotated activation that large has left the range the reference's own f16 cast of the input covers,
+// src/dequantizer.cpp:691).  The matrix-core paths keep decoded weights and rotated activations in fp16.
+__device__ __forceinline__ uint16_t float_to_f16_bits(float f) {
+    const float c = (f != f) ? f : __builtin_fminf(__builtin_fmaxf(f, -65504.0f), 65504.0f);
+    return __builtin_bit_cast(uint16_t, (_Float16)c);
 }
 
 // Load the 32 consecutive activations a lane owns and widen them to fp32.

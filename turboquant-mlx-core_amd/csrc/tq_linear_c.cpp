@@ -364,7 +364,7 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, const void* x_dev, int x_dtype, int batch,
                  void* y_dev, int y_dtype, hipStream_t stream, const float* gate, void* static_ws, size_t static_cap) {
     const bool lanes = !generic_only && tq::lanes_supported(V.in_features, V.block_size);
-    const bool prefill = lanes && tq::prefill_supported(V, x_dtype, batch);
+    const bool prefill = lanes && !gate && tq::prefill_supported(V, x_dtype, batch);   // (the gated store is a feature of the one-row kernels)
     const bool skinny = lanes && !prefill && !gate && tq::skinny_supported(V, x_dtype, batch);
     if (!prefill && !skinny && (generic_only || !tq::shape_supported(V.in_features, V.block_size))) {
         if (!tq::generic_supported(V)) { set_error("tq_linear_forward: unsupported layer shape"); return 1; }
@@ -394,13 +394,12 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
         }
     }
     if (prefill) {
-        if (gate) { set_error("tq_linear_forward: gated store is a batch < 16 feature"); return 1; }
-        // Dense contraction: rotate once, dequantise tiles to bf16 in LDS, MFMA.
+        // Dense contraction: rotate once, dequantise tiles to fp16 in LDS, MFMA.
         return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, stream),
                       "tq_prefill launch") ? 0 : 1;
     }
     if (skinny) {
-        // 2..15 rows of 16-bit activations: batch rows on the matrix cores, bf16 weights.
+        // 2..15 rows of 16-bit activations: batch rows on the matrix cores, fp16 weights.
         return hip_ok(tq::launch_skinny(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, partial, device_cu_count(), stream),
                       "tq_skinny launch") ? 0 : 1;
     }
@@ -739,14 +738,15 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
                                               nullptr, m->d_gate), "tq_gemv launch") ? 0 : 1;
             }
         }
-        if (batch == 1 || x_dtype == tq::kF32) {
+        if (batch == 1 || (x_dtype == tq::kF32 && batch < 16)) {
             // decode: three launches, the SiLU gate folded into the store of the up projection
             if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
             if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_act, tq::kF32, st, m->d_gate) != 0) return 1;
             return forward_impl(m->down, m->d_act, tq::kF32, batch, y_dev, y_dtype, st, nullptr);
         }
-        // two or more rows of 16-bit activations: matrix-core paths for all three layers (small-batch or
-        // prefill kernel), one elementwise kernel, activation handed to the down projection as bf16
+        // two or more rows of 16-bit activations, or 16 or more of any type: matrix-core paths for all three
+        // layers (small-batch or prefill kernel), one elementwise kernel; the activation is handed to the down
+        // projection as fp32 where its kernel takes that (16 rows or more), else as bf16
         const tq::LayerView both[2] = {m->gate->has_fwd_view ? m->gate->fwd_view : m->gate->view,
                                        m->up->has_fwd_view ? m->up->fwd_view : m->up->view};
         const bool plain = !(m->gate->view.mode >= tq::kShared5 && !m->gate->has_fwd_view) &&
@@ -761,8 +761,9 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
             if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
             if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_up, tq::kF32, st, nullptr) != 0) return 1;
         }
-        if (!hip_ok(tq::launch_silu_mul(m->d_gate, m->d_up, m->d_act, tq::kBF16, n, st), "silu_mul launch")) return 1;
-        return forward_impl(m->down, m->d_act, tq::kBF16, batch, y_dev, y_dtype, st, nullptr);
+        const int act_dtype = batch >= 16 ? tq::kF32 : tq::kBF16;
+        if (!hip_ok(tq::launch_silu_mul(m->d_gate, m->d_up, m->d_act, act_dtype, n, st), "silu_mul launch")) return 1;
+        return forward_impl(m->down, m->d_act, act_dtype, batch, y_dev, y_dtype, st, nullptr);
     } catch (...) { set_error("tq_mlp_forward: exception"); return 1; }
 }
 

@@ -1,17 +1,17 @@
-// TQ8 prefill: dequantise-into-LDS + bf16 MFMA GEMM for gfx950 (batch >= 16, 16-bit activations).
+// TQ8 prefill: dequantise-into-LDS + fp16 MFMA GEMM for gfx950 (batch >= 16, activations of any type).
 //
 // The reference has no batched-GEMM path: batch is a grid dimension of its per-row-FWHT kernel
 // (src/dequantizer.cpp:545-549), so every weight block is inverse-transformed once per batch row.
 // Here the activations are rotated once (X~ = H (s (.) X) per block, fp32 butterfly, rounded to
-// bf16) and the layer becomes one dense contraction
+// fp16 after the 1 / sqrt(bs) normalisation) and the layer becomes one dense contraction
 //
-//   Y[m, n] = norm[n] / sqrt(in * bs) * sum_k X~[m, k] * L[n, k],   L = centroid (sum) of the indices
+//   Y[m, n] = norm[n] / sqrt(in) * sum_k X~[m, k] * L[n, k],   L = centroid (sum) of the indices
 //
 // Workgroup tile 256 (M) x 256 (N), 8 waves as 2 (M) x 4 (N), each wave 128 x 64 built from
-// v_mfma_f32_32x32x16_bf16.  K advances in 32-column steps.  Activation tiles are copied from
+// v_mfma_f32_32x32x16_f16.  K advances in 32-column steps.  Activation tiles are copied from
 // global memory straight into LDS (three tiles in rotation, requested two steps ahead; the
 // rotate kernel stores X~ as ready-made tile images).  Index bytes travel through registers
-// (64-column stages, requested four steps ahead), are turned into bf16 through the lane-private
+// (64-column stages, requested four steps ahead), are turned into fp16 through the lane-private
 // LDS table and written to one of two weight tiles.  One barrier per step; the two waves of a
 // SIMD run the decode and the multiply half of a step in opposite order, which keeps the matrix
 // pipe fed during the decodes.
@@ -19,7 +19,7 @@
 
 namespace tq {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 
@@ -28,7 +28,7 @@ typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
 constexpr int kBM = 256, kBN = 256;
 constexpr int kBK = 32;                               // K extent of one LDS tile (one step)
 constexpr int kKLoad = 64;                            // K extent of one register stage of index bytes (two steps)
-constexpr int kBPitch = (kBK + 8) * 2;                // weight tile: bytes per row (bf16), padded -> 80
+constexpr int kBPitch = (kBK + 8) * 2;                // weight tile: bytes per row (fp16), padded -> 80
 constexpr int kBTile = 256 * kBPitch;                 // 20480
 constexpr int kATile = 256 * kBK * 2;                 // activation tile image: 256 rows x 64 B, swizzled -> 16384
 constexpr int kGemmThreads = 512;
@@ -38,7 +38,7 @@ constexpr int kAOff = kBOff + 2 * kBTile;             // three activation tiles
 constexpr int kGemmSmem = kAOff + 3 * kATile;         // 155648 of the CU's 163840 bytes
 
 struct PrefillArgs {
-    const uint16_t* xt;        // rotated activations, bf16 tile images [planes][m_tiles][K/32][16 KB]
+    const uint16_t* xt;        // rotated activations, fp16 tile images [planes][m_tiles][K/32][16 KB]
     const uint8_t* plane0;     // combined bytes [N, K] (shared) or primary nibbles [N, K/2]
     const uint8_t* plane1;     // residual nibbles [N, K/2] (dual) or NULL
     const float* tables;       // 256 floats (see build_tables in tq_linear_c.cpp)
@@ -60,9 +60,9 @@ __device__ __forceinline__ uint32_t gemm_entry_addr(uint32_t idx_bytes, uint32_t
     }
 }
 
-// Table entries are fp32 bit patterns already rounded to bf16 (low 16 bits zero): two of them
-// pack into one bf16x2 register with a single byte permute.
-__device__ __forceinline__ uint32_t pack_bf16x2(uint32_t lo_val, uint32_t hi_val) {
+// Table entries hold the fp16 value in the upper half of the dword (low 16 bits zero): two of them
+// pack into one register of two halves with a single byte permute.
+__device__ __forceinline__ uint32_t pack_half2(uint32_t lo_val, uint32_t hi_val) {
     return __builtin_amdgcn_perm(hi_val, lo_val, 0x07060302u);   // {lo.b2, lo.b3, hi.b2, hi.b3}
 }
 
@@ -170,8 +170,8 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
                     const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w, laneoff, 1));
                     const uint32_t v2 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w, laneoff, 2));
                     const uint32_t v3 = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(w, laneoff, 3));
-                    rb[2 * d] = pack_bf16x2(v0, v1);
-                    rb[2 * d + 1] = pack_bf16x2(v2, v3);
+                    rb[2 * d] = pack_half2(v0, v1);
+                    rb[2 * d + 1] = pack_half2(v2, v3);
                 }
             } else {
                 const uint32_t w2[2] = {st.b[u].x, st.b[u].y};
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
                     for (int j = 0; j < 4; ++j) {
                         const uint32_t ve = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(ce, laneoff, j));
                         const uint32_t vo = *reinterpret_cast<const uint32_t*>(smem + gemm_entry_addr(co, laneoff, j));
-                        rb[4 * d + j] = pack_bf16x2(ve, vo);
+                        rb[4 * d + j] = pack_half2(ve, vo);
                     }
                 }
             }
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
         // into the other weight tile, request activation tile t+2 and (odd steps) the index stage
         // three ahead of the one whose second half was just decoded.
         // The 8 table reads of decode half h (0/1) of stage half u, and their packing into 4
-        // registers of bf16 pairs.
+        // registers of fp16 pairs.
         auto lookup_half = [&](const Stage& st, int u, int h, uint32_t (&lv)[8]) {
             if constexpr (combined) {
                 const uint32_t w2[2] = {h == 0 ? st.b[u].x : st.b[u].z, h == 0 ? st.b[u].y : st.b[u].w};
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
         };
         auto pack_half = [&](const uint32_t (&lv)[8], uint32_t* rb) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) rb[q] = pack_bf16x2(lv[2 * q], lv[2 * q + 1]);
+            for (int q = 0; q < 4; ++q) rb[q] = pack_half2(lv[2 * q], lv[2 * q + 1]);
         };
 
         // Step t = 6q + R: multiply activation tile R % 3 with weight tile R % 2, decode step t+1
@@ -239,16 +239,16 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
             const char* As = smem + kAOff + abuf * kATile;
             const char* Bs = smem + kBOff + bbuf * kBTile + b_frag;
             const bool do_fill = t + 1 < T;
-            bf16x8 fa0[4], fb0[2], fa1[4], fb1[2];
+            f16x8 fa0[4], fb0[2], fa1[4], fb1[2];
             uint32_t lv[8], rb[8];
-            auto mm = [&](int i, const bf16x8 (&fa)[4], const bf16x8 (&fb)[2]) {
-                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[0], acc[i][0], 0, 0, 0);
-                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[1], acc[i][1], 0, 0, 0);
+            auto mm = [&](int i, const f16x8 (&fa)[4], const f16x8 (&fb)[2]) {
+                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[0], acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[1], acc[i][1], 0, 0, 0);
             };
 #pragma unroll
-            for (int j = 0; j < 2; ++j) fb0[j] = *reinterpret_cast<const bf16x8*>(Bs + j * 32 * kBPitch);
+            for (int j = 0; j < 2; ++j) fb0[j] = *reinterpret_cast<const f16x8*>(Bs + j * 32 * kBPitch);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa0[i] = *reinterpret_cast<const bf16x8*>(As + a_frag0 + i * 32 * 64);
+            for (int i = 0; i < 4; ++i) fa0[i] = *reinterpret_cast<const f16x8*>(As + a_frag0 + i * 32 * 64);
             if (do_fill) lookup_half(st, u, 0, lv);
             __builtin_amdgcn_sched_barrier(0);
             mm(0, fa0, fb0);
@@ -256,9 +256,9 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
             mm(1, fa0, fb0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) fb1[j] = *reinterpret_cast<const bf16x8*>(Bs + j * 32 * kBPitch + 32);
+            for (int j = 0; j < 2; ++j) fb1[j] = *reinterpret_cast<const f16x8*>(Bs + j * 32 * kBPitch + 32);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa1[i] = *reinterpret_cast<const bf16x8*>(As + a_frag1 + i * 32 * 64);
+            for (int i = 0; i < 4; ++i) fa1[i] = *reinterpret_cast<const f16x8*>(As + a_frag1 + i * 32 * 64);
             if (do_fill) {
                 pack_half(lv, rb);
                 lookup_half(st, u, 1, lv);
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 #pragma unroll
             for (int e = 0; e < per_wave; ++e) {
                 const int entry = wave * per_wave + e;
-                if (entry < entries) dst[entry * 64] = (uint32_t)float_to_bf16_bits(src[entry]) << 16;
+                if (entry < entries) dst[entry * 64] = (uint32_t)float_to_f16_bits(src[entry]) << 16;
             }
         }
         asm volatile("s_waitcnt vmcnt(0)"
@@ -403,14 +403,15 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 }
 
 // ---------------------------------------------------------------------------
-// Rotate activations [M, K] (f32 / f16 / bf16) -> bf16 tile images: X~ = H (s (.) X) per block,
+// Rotate activations [M, K] (f32 / f16 / bf16) -> fp16 tile images: X~ = H (s (.) X) / sqrt(bs) per block,
 // stored as [M/256][K/32] images of 256 rows x 64 bytes in the exact byte order the GEMM keeps
 // them in LDS (16-byte slots permuted by a_slot), so a tile is one contiguous 16 KB copy.
 // One wave per (row, 2048-column slab), 32 consecutive columns per lane, fp32 butterfly.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void tq_rotate_bf16_kernel(const void* __restrict__ x, int x_dtype,
+__global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restrict__ x, int x_dtype,
                                                              uint16_t* __restrict__ out, int rows, int cols,
-                                                             int chunks, int slabs, uint32_t seed, uint32_t bs) {
+                                                             int chunks, int slabs, uint32_t seed, uint32_t bs,
+                                                             float scale) {
     const int lane = threadIdx.x & 63;
     const int row = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);     // grid = row quads x slabs
     const int slab = blockIdx.y;
@@ -436,7 +437,7 @@ __global__ __launch_bounds__(256) void tq_rotate_bf16_kernel(const void* __restr
             uint32_t w[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                w[j] = (uint32_t)float_to_bf16_bits(v[8 * i + 2 * j]) | ((uint32_t)float_to_bf16_bits(v[8 * i + 2 * j + 1]) << 16);
+                w[j] = (uint32_t)float_to_f16_bits(v[8 * i + 2 * j] * scale) | ((uint32_t)float_to_f16_bits(v[8 * i + 2 * j + 1] * scale) << 16);
             dst[a_slot(r, i)] = make_uint4(w[0], w[1], w[2], w[3]);
         }
     }
@@ -449,15 +450,16 @@ size_t prefill_workspace_bytes(const LayerView& L, int batch) {
 }
 
 bool prefill_supported(const LayerView& L, int x_dtype, int batch) {
-    if (x_dtype == kF32 || batch < 16) return false;          // fp32 activations keep the exact fp32 GEMV path
+    if (batch < 16) return false;                             // (fp32 activations too: the fp16 operands keep 1e-3)
     if (L.mode != kSharedLut && L.mode != kDual && L.mode != kPrimaryOnly) return false;
+    if (!L.fp16_centroids_ok) return false;                   // decoded weights are kept in fp16
     if (!lanes_supported(L.in_features, L.block_size)) return false;
     // (the kernel addresses the index plane with 32-bit byte offsets)
     if ((unsigned long long)L.out_features * (unsigned long long)L.in_features >= (1ull << 32)) return false;
     return L.in_features % kKLoad == 0;
 }
 
-// Rotated activations of `batch` rows as bf16 tile images in `workspace` (both rotations for dual mode).
+// Rotated activations of `batch` rows as fp16 tile images in `workspace` (both rotations for dual mode).
 hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
                                hipStream_t stream) {
     const int K = L.in_features, M = batch;
@@ -465,12 +467,12 @@ hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, i
     const int chunks = K / kChunk;
     const int slabs = (chunks + kWave - 1) / kWave;
     const dim3 rgrid((unsigned)((M + 3) / 4), (unsigned)slabs);
-    hipLaunchKernelGGL(tq_rotate_bf16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
-                       L.seed_primary, L.block_size);
+    hipLaunchKernelGGL(tq_rotate_f16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
+                       L.seed_primary, L.block_size, L.inv_sqrt_bs);
     if (L.mode == kDual)
-        hipLaunchKernelGGL(tq_rotate_bf16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype,
+        hipLaunchKernelGGL(tq_rotate_f16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype,
                            xt + (size_t)((M + kBM - 1) / kBM) * kBM * K, M, K, chunks, slabs, L.seed_residual,
-                           L.block_size);
+                           L.block_size, L.inv_sqrt_bs);
     return hipGetLastError();
 }
 
@@ -491,7 +493,7 @@ hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int ba
     a.M = M; a.N = N; a.K = K; a.mode = L.mode;
     a.m_tiles = (M + kBM - 1) / kBM;
     a.n_tiles = (N + kBN - 1) / kBN;
-    a.out_scale = L.inv_scale * L.inv_sqrt_bs;
+    a.out_scale = L.inv_scale;                          // (1 / sqrt(bs) is in the rotated activations)
     const int n_groups = (a.n_tiles + 7) / 8;
     const unsigned grid = (unsigned)(n_groups * 8 * a.m_tiles);
     switch (L.mode) {

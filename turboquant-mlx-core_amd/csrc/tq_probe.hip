@@ -1,5 +1,5 @@
 // Machine probes for the roofline denominators and for design decisions: what this GPU sustains on a pure
-// streaming read, on a pure bf16 MFMA loop, and on device-scope fetch-adds from every wave of the chip.
+// streaming read, on a pure bf16 or fp16 MFMA loop, and on device-scope fetch-adds from every wave of the chip.
 // Measurement support only: nothing in the layer path calls them.
 #include "turboquant_c/tq_probe.h"
 
@@ -8,6 +8,7 @@
 namespace tq {
 
 typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 probe_f16x8 __attribute__((ext_vector_type(8)));
 typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
 
@@ -24,25 +25,32 @@ __global__ __launch_bounds__(512) void tq_probe_read_kernel(const probe_u32x4* _
     if (acc == 0x9e3779b9u) sink[0] = acc;                    // keeps the loads alive
 }
 
-// 8 waves per CU, each a loop of 16 independent v_mfma_f32_32x32x16_bf16 per iteration (the
-// instruction mix of the prefill kernel's inner step), operands fixed in registers.
+// 8 waves per CU, each a loop of 16 independent v_mfma_f32_32x32x16_bf16 (HALF: _f16, the instruction
+// of the prefill kernel's inner step) per iteration, operands fixed in registers.
+template <bool HALF>
 __global__ __launch_bounds__(512) void tq_probe_mfma_kernel(float* __restrict__ sink, int iters, int random_operands) {
     probe_f32x16 acc[8];
     for (int i = 0; i < 8; ++i)
         for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
     probe_bf16x8 a, b;
+    probe_f16x8 ah, bh;
     uint32_t h = (threadIdx.x + 1) * 2654435761u + blockIdx.x * 40503u;
     for (int j = 0; j < 8; ++j) {
         h = h * 1664525u + 1013904223u;
-        a[j] = random_operands ? (__bf16)(((int)(h >> 8) % 2001 - 1000) * 1e-3f) : (__bf16)1.0f;
+        const float va = random_operands ? ((int)(h >> 8) % 2001 - 1000) * 1e-3f : 1.0f;
         h = h * 1664525u + 1013904223u;
-        b[j] = random_operands ? (__bf16)(((int)(h >> 8) % 2001 - 1000) * 1e-3f) : (__bf16)1.0f;
+        const float vb = random_operands ? ((int)(h >> 8) % 2001 - 1000) * 1e-3f : 1.0f;
+        a[j] = (__bf16)va; b[j] = (__bf16)vb;
+        ah[j] = (_Float16)va; bh[j] = (_Float16)vb;
     }
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+            for (int i = 0; i < 8; ++i) {
+                if constexpr (HALF) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, acc[i], 0, 0, 0);
+                else acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+            }
         __syncthreads();
     }
     float s = 0.0f;
@@ -98,9 +106,9 @@ int tq_probe_hbm_read(size_t bytes, int repeats, double* gb_per_s) {
     } catch (...) { tq::set_error("tq_probe_hbm_read: exception"); return 1; }
 }
 
-int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops) {
+static int probe_mfma(bool half, int random_operands, int iterations, double* tflops) {
     try {
-        if (!tflops || iterations <= 0) { tq::set_error("tq_probe_mfma_bf16: bad argument"); return 1; }
+        if (!tflops || iterations <= 0) { tq::set_error("tq_probe_mfma: bad argument"); return 1; }
         int dev = 0, cus = 0;
         float* sink = nullptr;
         hipEvent_t t0 = nullptr, t1 = nullptr;
@@ -110,9 +118,11 @@ int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops) {
                   tq::hip_ok(hipEventCreate(&t0), "event") && tq::hip_ok(hipEventCreate(&t1), "event");
         float ms = 0.0f;
         if (ok) {
-            hipLaunchKernelGGL(tq::tq_probe_mfma_kernel, dim3(cus), dim3(512), 0, nullptr, sink, 64, random_operands);
+            if (half) hipLaunchKernelGGL(tq::tq_probe_mfma_kernel<true>, dim3(cus), dim3(512), 0, nullptr, sink, 64, random_operands);
+            else hipLaunchKernelGGL(tq::tq_probe_mfma_kernel<false>, dim3(cus), dim3(512), 0, nullptr, sink, 64, random_operands);
             (void)hipEventRecord(t0, nullptr);
-            hipLaunchKernelGGL(tq::tq_probe_mfma_kernel, dim3(cus), dim3(512), 0, nullptr, sink, iterations, random_operands);
+            if (half) hipLaunchKernelGGL(tq::tq_probe_mfma_kernel<true>, dim3(cus), dim3(512), 0, nullptr, sink, iterations, random_operands);
+            else hipLaunchKernelGGL(tq::tq_probe_mfma_kernel<false>, dim3(cus), dim3(512), 0, nullptr, sink, iterations, random_operands);
             (void)hipEventRecord(t1, nullptr);
             ok = tq::hip_ok(hipEventSynchronize(t1), "probe sync") && tq::hip_ok(hipEventElapsedTime(&ms, t0, t1), "elapsed");
         }
@@ -122,7 +132,15 @@ int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops) {
         if (t1) (void)hipEventDestroy(t1);
         if (sink) (void)hipFree(sink);
         return ok ? 0 : 1;
-    } catch (...) { tq::set_error("tq_probe_mfma_bf16: exception"); return 1; }
+    } catch (...) { tq::set_error("tq_probe_mfma: exception"); return 1; }
+}
+
+int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops) {
+    return probe_mfma(false, random_operands, iterations, tflops);
+}
+
+int tq_probe_mfma_f16(int random_operands, int iterations, double* tflops) {
+    return probe_mfma(true, random_operands, iterations, tflops);
 }
 
 int tq_probe_device_atomics(int addresses, int per_wave, double* per_microsecond) {

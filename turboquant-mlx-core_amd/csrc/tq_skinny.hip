@@ -3,36 +3,37 @@
 //
 // The batch-1 kernel multiplies every decoded weight with the activation of each batch row on the
 // vector ALU, so its time grows with the batch.  Here the batch rows are the M side of
-// v_mfma_f32_16x16x32_bf16: a decoded weight costs one table read and half a byte permute however
+// v_mfma_f32_16x16x32_f16: a decoded weight costs one table read and half a byte permute however
 // many rows there are, and the kernel stays bound by the same table-read rate as batch 1.
 //
-//   Y[m, n] = norm[n] / sqrt(in * bs) * sum_k X~[m, k] * L[n, k]
+//   Y[m, n] = norm[n] / sqrt(in) * sum_k X~[m, k] * L[n, k],   X~ = H (s (.) X) / sqrt(bs)
 //
 // K is cut into 512-column chunks.  A wave keeps the rotated activations of its chunk for all 16
 // (padded) batch rows in registers as MFMA A operands (64 VGPRs), walks 16-row groups of the weight
 // plane, decodes 16 x 512 weights per group through the lane-private LDS table (entries rounded to
-// bf16, as in the prefill kernel) and writes the 16 x 16 fp32 partial product of the chunk.  A
+// fp16, as in the prefill kernel) and writes the 16 x 16 fp32 partial product of the chunk.  A
 // second small kernel adds the chunks, applies the row norm and converts.
-// The rotated activations come from tq_rotate_bf16_kernel (tile images, see tq_prefill.hip).
+// The rotated activations come from tq_rotate_f16_kernel (tile images, see tq_prefill.hip).
 #include "tq_device.h"
 #include "tq_gemv_common.h"
 
 namespace tq {
 
-typedef __bf16 sk_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 sk_f16x8 __attribute__((ext_vector_type(8)));
 typedef float sk_f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t sk_u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kSkChunk = 512;            // columns per K chunk
 constexpr int kSkThreads = 512;          // 8 waves per workgroup, one workgroup per CU
 constexpr int kSkLutBytes = 256 * 256;
-constexpr int kSkStageBytes = 16 * kSkChunk * 2;   // 16 rows x 512 bf16 rotated activations
+constexpr int kSkStageBytes = 16 * kSkChunk * 2;   // 16 rows x 512 fp16 rotated activations
 
 struct SkinnyArgs {
     const void* x;             // FUSED: activations [batch, K], f16 or bf16
     int x_dtype;
     uint32_t seed, block_size; // FUSED: rotation of the layer (blocks of at most 512 columns)
-    const uint16_t* xt;        // otherwise: rotated activations, bf16 tile images [K/32][256 rows x 64 B] (rows >= batch unset)
+    float x_scale;             // FUSED: 1 / sqrt(block_size), applied to the rotated activations before they are rounded
+    const uint16_t* xt;        // otherwise: rotated activations, fp16 tile images [K/32][256 rows x 64 B] (rows >= batch unset)
     const uint8_t* plane;      // combined bytes [N, K]
     const float* tables;       // 256-entry sum table
     float* partial;            // [chunks][batch][N] fp32
@@ -58,7 +59,7 @@ __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t l
 // share the chunk for this layer (a launch may serve several layers).
 template <bool FUSED>
 __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk, const int wg_in_chunk) {
-    // table | 16 x 512 bf16 rotated activations (FUSED).  One workgroup of 8 waves per CU: 16 waves
+    // table | 16 x 512 fp16 rotated activations (FUSED).  One workgroup of 8 waves per CU: 16 waves
     // gained nothing, and 8 have the registers for two row groups in flight.
     __shared__ __align__(16) char smem[kSkLutBytes + kSkStageBytes];
     const int tid = threadIdx.x;
@@ -110,21 +111,21 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
     };
     if (g_begin < g_end) request(rawA, g_begin);
 
-    // Decode table -> LDS, one private column per lane, values rounded to bf16 (upper half of the dword).
+    // Decode table -> LDS, one private column per lane, values rounded to fp16 (upper half of the dword).
     {
         uint4* dst = reinterpret_cast<uint4*>(smem);
 #pragma unroll
         for (int k = 0; k < kSlots; ++k) {
-            const uint32_t v = (uint32_t)float_to_bf16_bits(tv[k]) << 16;
+            const uint32_t v = (uint32_t)float_to_f16_bits(tv[k]) << 16;
             dst[tid + k * kSkThreads] = make_uint4(v, v, v, v);
         }
     }
 
-    sk_bf16x8 afrag[16];
+    sk_f16x8 afrag[16];
     char* const stage = smem + kSkLutBytes;
     if constexpr (FUSED) {
         // Wave w rotates batch rows w and w + 8 of the chunk (one 512-column tile each, 8 values per
-        // lane; blocks of at most 512 columns: a block never leaves the chunk) and writes them as bf16,
+        // lane; blocks of at most 512 columns: a block never leaves the chunk) and writes them, scaled by 1 / sqrt(bs), as fp16,
         // [16 rows][512]; rows past the batch are zero.
         constexpr int kPitch = kSkChunk * 2;
 #pragma unroll
@@ -135,10 +136,10 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
             if (b < a.batch) {                              // wave-uniform
                 float v[8];
                 rotate_tile(xin[t], a.x_dtype, col, true, a.seed, a.block_size, lane, v);
-                packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-                packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-                packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
-                packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
+                packed.x = (uint32_t)float_to_f16_bits(v[0] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[1] * a.x_scale) << 16);
+                packed.y = (uint32_t)float_to_f16_bits(v[2] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[3] * a.x_scale) << 16);
+                packed.z = (uint32_t)float_to_f16_bits(v[4] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[5] * a.x_scale) << 16);
+                packed.w = (uint32_t)float_to_f16_bits(v[6] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[7] * a.x_scale) << 16);
             }
             *reinterpret_cast<uint4*>(stage + b * kPitch + lane * 16) = packed;
         }
@@ -147,22 +148,22 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
         // the B operand of that step decodes (any column order is fine as long as both agree).
 #pragma unroll
         for (int s = 0; s < 16; ++s)
-            afrag[s] = *reinterpret_cast<const sk_bf16x8*>(stage + m * kPitch + (64 * (s >> 1) + 16 * g + 8 * (s & 1)) * 2);
+            afrag[s] = *reinterpret_cast<const sk_f16x8*>(stage + m * kPitch + (64 * (s >> 1) + 16 * g + 8 * (s & 1)) * 2);
     } else {
-        // Tile images written by tq_rotate_bf16_kernel: [K/32][256][32] bf16 with 16-byte slots
+        // Tile images written by tq_rotate_f16_kernel: [K/32][256][32] fp16 with 16-byte slots
         // XOR-permuted per row; same column order as above.
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
             const int off = 16 * g + 8 * (s & 1);              // column inside the 64-column piece
             const int kt = chunk * 16 + 2 * (s >> 1) + (off >> 5);
             const int slot = ((off & 31) >> 3) ^ ((m >> 2) & 3);
-            afrag[s] = *reinterpret_cast<const sk_bf16x8*>(reinterpret_cast<const char*>(a.xt) +
+            afrag[s] = *reinterpret_cast<const sk_f16x8*>(reinterpret_cast<const char*>(a.xt) +
                                                            ((size_t)kt * 256 + m) * 64 + slot * 16);
         }
         __syncthreads();                                    // table visible
     }
 
-    auto lookup2 = [&](uint32_t w) {                       // 4 weights -> 2 registers of bf16 pairs
+    auto lookup2 = [&](uint32_t w) {                       // 4 weights -> 2 registers of fp16 pairs
         const uint32_t v0 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 0));
         const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 1));
         const uint32_t v2 = *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 2));
@@ -178,8 +179,8 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
             const sk_u32x4 w = raw[q];
             const uint2 p0 = lookup2(w.x), p1 = lookup2(w.y), p2 = lookup2(w.z), p3 = lookup2(w.w);
             const sk_u32x4 b0 = {p0.x, p0.y, p1.x, p1.y}, b1 = {p2.x, p2.y, p3.x, p3.y};
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * q], __builtin_bit_cast(sk_bf16x8, b0), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * q + 1], __builtin_bit_cast(sk_bf16x8, b1), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[2 * q], __builtin_bit_cast(sk_f16x8, b0), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[2 * q + 1], __builtin_bit_cast(sk_f16x8, b1), acc, 0, 0, 0);
         }
         // D layout: lane holds weight row n = lane % 16 and batch rows 4 (lane / 16) + r.
         const int n = grp * 16 + m;
@@ -230,6 +231,7 @@ struct SkinnyNibbleArgs {
     const void* x;             // activations [batch, K], f16 or bf16
     int x_dtype;
     uint32_t seed[2], block_size;
+    float x_scale;             // 1 / sqrt(block_size), applied to the rotated activations before they are rounded
     const uint8_t* plane[2];   // [N, K/2] each; plane[1] unused for primary-only layers
     const float* tables;       // 16 primary centroids, then 16 residual ones
     float* partial;            // [units][batch][N] fp32
@@ -244,10 +246,10 @@ struct SkinnyNibbleArgs {
 // unit, wg_in_unit: the (chunk, plane) unit of this workgroup and its index among the workgroups that
 // share the unit for this layer (a launch may serve several layers).
 __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, const int unit, const int wg_in_unit) {
-    // The table is indexed by a whole byte of the plane: an entry holds the bf16 centroids of both
+    // The table is indexed by a whole byte of the plane: an entry holds the fp16 centroids of both
     // its nibbles, i.e. one register of the B operand, so two weights cost one table read.
     constexpr int kTabBytes = kSkLutBytes;                 // 256 entries, one private column per lane
-    __shared__ __align__(16) char smem[kTabBytes + kSkStageBytes];   // table | 16 x 512 bf16 rotated activations
+    __shared__ __align__(16) char smem[kTabBytes + kSkStageBytes];   // table | 16 x 512 fp16 rotated activations
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -294,15 +296,15 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
     };
     if (g_begin < g_end) request(rawA, g_begin);
 
-    {                                                       // 256 entries x 16 slots of 16 bytes, values rounded to bf16
-        const uint32_t lo = (uint32_t)float_to_bf16_bits(tlo);
+    {                                                       // 256 entries x 16 slots of 16 bytes, values rounded to fp16
+        const uint32_t lo = (uint32_t)float_to_f16_bits(tlo);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const uint32_t v = lo | ((uint32_t)float_to_bf16_bits(thi[k]) << 16);
+            const uint32_t v = lo | ((uint32_t)float_to_f16_bits(thi[k]) << 16);
             reinterpret_cast<uint4*>(smem)[tid + k * kSkThreads] = make_uint4(v, v, v, v);
         }
     }
-    // Rotate batch rows w and w + 8 of the chunk with this plane's seed -> bf16 [16][512] in LDS.
+    // Rotate batch rows w and w + 8 of the chunk with this plane's seed -> fp16 [16][512] in LDS.
     constexpr int kPitch = kSkChunk * 2;
     char* const stage = smem + kTabBytes;
 #pragma unroll
@@ -313,10 +315,10 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
         if (b < a.batch) {                                  // wave-uniform
             float v[8];
             rotate_tile(xin[t], a.x_dtype, col, true, a.seed[pl], a.block_size, lane, v);
-            packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-            packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-            packed.z = (uint32_t)float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
-            packed.w = (uint32_t)float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
+            packed.x = (uint32_t)float_to_f16_bits(v[0] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[1] * a.x_scale) << 16);
+            packed.y = (uint32_t)float_to_f16_bits(v[2] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[3] * a.x_scale) << 16);
+            packed.z = (uint32_t)float_to_f16_bits(v[4] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[5] * a.x_scale) << 16);
+            packed.w = (uint32_t)float_to_f16_bits(v[6] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[7] * a.x_scale) << 16);
         }
         *reinterpret_cast<uint4*>(stage + b * kPitch + lane * 16) = packed;
     }
@@ -324,10 +326,10 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
     // A operands.  Matrix step s = 4 q + d multiplies columns 128 q + 32 g + 8 d + [0, 8) of the chunk:
     // the 8 nibbles of dword d of the lane's 16-byte piece q (piece q of lane group g starts at byte
     // 64 q + 16 g of the row's 256 bytes).
-    sk_bf16x8 afrag[16];
+    sk_f16x8 afrag[16];
 #pragma unroll
     for (int s = 0; s < 16; ++s)
-        afrag[s] = *reinterpret_cast<const sk_bf16x8*>(stage + m * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
+        afrag[s] = *reinterpret_cast<const sk_f16x8*>(stage + m * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
 
     // One dword = 8 weights of 8 consecutive columns (low nibble first) -> one B operand: byte j of
     // the dword selects the register that holds columns 2 j and 2 j + 1.
@@ -336,17 +338,17 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
                             *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 1)),
                             *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 2)),
                             *reinterpret_cast<const uint32_t*>(smem + sk_entry_addr(w, laneoff, 3))};
-        return __builtin_bit_cast(sk_bf16x8, r);
+        return __builtin_bit_cast(sk_f16x8, r);
     };
     auto multiply = [&](const sk_u32x4 (&raw)[4], int grp) {
         sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const sk_u32x4 w = raw[q];
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 0], operand(w.x), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 1], operand(w.y), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 2], operand(w.z), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[4 * q + 3], operand(w.w), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 0], operand(w.x), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 1], operand(w.y), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 2], operand(w.z), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 3], operand(w.w), acc, 0, 0, 0);
         }
         const int n = grp * 16 + m;
         if (n < a.N) {
@@ -444,6 +446,7 @@ static bool skinny_nibble(const LayerView& L) {
 bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
     if (x_dtype == kF32 || batch < 2 || batch >= 16 || L.in_features % kSkChunk != 0) return false;
     if (!lanes_supported(L.in_features, L.block_size)) return false;
+    if (!L.fp16_centroids_ok) return false;                   // decoded weights are kept in fp16
     return (L.mode == kSharedLut && L.packed_combined) || skinny_nibble(L);
 }
 
@@ -465,6 +468,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     if (skinny_nibble(L)) {
         SkinnyNibbleArgs n{};
         n.x = x; n.x_dtype = x_dtype; n.seed[0] = L.seed_primary; n.seed[1] = L.seed_residual; n.block_size = L.block_size;
+        n.x_scale = L.inv_sqrt_bs;
         n.plane[0] = L.packed_primary; n.plane[1] = L.packed_residual;
         n.tables = L.tables;
         n.partial = partial;
@@ -481,7 +485,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         if (en != hipSuccess) return en;
         const unsigned blocks_n = (unsigned)((L.out_features + 63) / 64);
         hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks_n, batch), dim3(256), 0, stream,
-                           partial, L.norms, y, y_dtype, batch, L.out_features, n.units, L.inv_scale * L.inv_sqrt_bs);
+                           partial, L.norms, y, y_dtype, batch, L.out_features, n.units, L.inv_scale);
         return hipGetLastError();
     }
     const bool fused = L.block_size <= (uint32_t)kSkChunk;
@@ -491,7 +495,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         if (e != hipSuccess) return e;
     }
     SkinnyArgs a{};
-    a.x = x; a.x_dtype = x_dtype; a.seed = L.seed_primary; a.block_size = L.block_size;
+    a.x = x; a.x_dtype = x_dtype; a.seed = L.seed_primary; a.block_size = L.block_size; a.x_scale = L.inv_sqrt_bs;
     a.xt = static_cast<const uint16_t*>(xt_workspace);
     a.plane = L.packed_combined;
     a.tables = L.tables;
@@ -509,7 +513,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     if (e != hipSuccess) return e;
     const unsigned blocks = (unsigned)((L.out_features + 63) / 64);
     hipLaunchKernelGGL(tq_skinny_reduce_kernel, dim3(blocks, batch), dim3(256), 0, stream,
-                       partial, L.norms, y, y_dtype, batch, L.out_features, a.chunks, L.inv_scale * L.inv_sqrt_bs);
+                       partial, L.norms, y, y_dtype, batch, L.out_features, a.chunks, L.inv_scale);
     return hipGetLastError();
 }
 
@@ -553,6 +557,7 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
             const LayerView& L = Ls[j];
             SkinnyNibbleArgs& q = gn.a[j];
             q.x = x; q.x_dtype = x_dtype; q.seed[0] = L.seed_primary; q.seed[1] = L.seed_residual; q.block_size = L.block_size;
+            q.x_scale = L.inv_sqrt_bs;
             q.plane[0] = L.packed_primary; q.plane[1] = L.packed_residual;
             q.tables = L.tables;
             q.partial = partials[j];
@@ -565,7 +570,7 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
             q.groups_rem = q.groups % (wgs[j] * (kSkThreads / 64));
             gn.first[j + 1] = gn.first[j] + wgs[j];
             SkinnyArgs& a = g.a[j];
-            a.x = x; a.x_dtype = x_dtype; a.seed = L.seed_primary; a.block_size = L.block_size;
+            a.x = x; a.x_dtype = x_dtype; a.seed = L.seed_primary; a.block_size = L.block_size; a.x_scale = L.inv_sqrt_bs;
             a.xt = nullptr;
             a.plane = L.packed_combined;
             a.tables = L.tables;
@@ -578,7 +583,7 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
             a.groups_q = a.groups / workers;
             a.groups_rem = a.groups % workers;
             r.partial[j] = partials[j]; r.norms[j] = L.norms; r.y[j] = ys[j]; r.N[j] = L.out_features;
-            r.out_scale[j] = L.inv_scale * L.inv_sqrt_bs;
+            r.out_scale[j] = L.inv_scale;
             g.first[j + 1] = g.first[j] + wgs[j];
             r.first[j + 1] = r.first[j] + (L.out_features + 63) / 64;
         } else {
