@@ -74,6 +74,13 @@ __device__ __forceinline__ uint32_t entry_addr(uint32_t idx_bytes, uint32_t lane
     return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0000u | ((4u + J) << 8));
 }
 
+// The same with bits 16..23 of laneoff kept: (table << 16) | (entry << 8) | (lane << 2), for 64 KB
+// tables that follow each other in LDS.
+template <int J>
+__device__ __forceinline__ uint32_t entry_addr_hi(uint32_t idx_bytes, uint32_t laneoff) {
+    return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c020000u | ((4u + J) << 8));
+}
+
 __device__ __forceinline__ float lds_f32(const char* lds, uint32_t byte_addr) {
     return *reinterpret_cast<const float*>(lds + byte_addr);
 }
@@ -83,9 +90,12 @@ __device__ __forceinline__ float lds_f32(const char* lds, uint32_t byte_addr) {
 //           column); each byte indexes the 256-entry sum table of shared rotation
 //           (reference src/dequantizer.cpp:144-169).
 //   else  : P holds 32 nibbles of one plane (lo nibble = even column); 16-entry table at TABLE_OFF.
+//           table_bits: 0, or 0x10101010 for the 16-entry table that follows the first one (entry
+//           numbers 16..31; selecting the table in the index costs one OR per eight lookups, a table
+//           base that is not a constant one addition per lookup).
 template <bool LUT256, int TABLE_OFF>
 __device__ __forceinline__ void lookup32(const uint4& P, const uint4& Q, const char* lds, uint32_t laneoff,
-                                         float (&val)[kChunk]) {
+                                         float (&val)[kChunk], uint32_t table_bits = 0) {
     const char* tab = lds + TABLE_OFF;
     if constexpr (LUT256) {
         const uint32_t w[8] = {P.x, P.y, P.z, P.w, Q.x, Q.y, Q.z, Q.w};
@@ -100,8 +110,8 @@ __device__ __forceinline__ void lookup32(const uint4& P, const uint4& Q, const c
         const uint32_t pw[4] = {P.x, P.y, P.z, P.w};
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-            const uint32_t ce = pw[d] & 0x0F0F0F0Fu;
-            const uint32_t co = (pw[d] >> 4) & 0x0F0F0F0Fu;
+            const uint32_t ce = (pw[d] & 0x0F0F0F0Fu) | table_bits;
+            const uint32_t co = ((pw[d] >> 4) & 0x0F0F0F0Fu) | table_bits;
             val[8 * d + 0] = lds_f32(tab, entry_addr<0>(ce, laneoff));
             val[8 * d + 1] = lds_f32(tab, entry_addr<0>(co, laneoff));
             val[8 * d + 2] = lds_f32(tab, entry_addr<1>(ce, laneoff));

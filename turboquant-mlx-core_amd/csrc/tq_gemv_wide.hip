@@ -151,7 +151,11 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     constexpr int NS = 2;                           // register ring: one group decoded, one in flight
     constexpr int V = PAIR ? 2 * R : R;             // rows, and sums, per row group
     constexpr int NX = PAIR ? 16 : kChunk;          // rotated activations per lane
-    extern __shared__ __align__(16) char smem[];    // tables | cross-wave partial sums | activation image
+    // tables | cross-wave partial sums | activation image.  A static array: its address is a constant
+    // the compiler folds into the LDS instructions (with a dynamic one every table read carried an
+    // address addition of its own, a third of the vector instructions of the decode).
+    constexpr int kImageBytes = PRE ? 0 : ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float);
+    __shared__ __align__(16) char smem[kRegion + kPartialBytes + kImageBytes];
     float* partial = reinterpret_cast<float*>(smem + kRegion);   // [2][waves][V]
 
     const int tid = threadIdx.x;
@@ -170,6 +174,10 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     const int col_b = PAIR ? col_a : (combined ? col_a + 1024 : col_a + 16);
     const bool act_a = col_a < a.L.in_features, act_b = col_b < a.L.in_features;
     const uint32_t laneoff = (uint32_t)lane << 2;
+    [[maybe_unused]] const uint32_t laneoff_plane = laneoff | ((uint32_t)plane << 16);   // kLut256Bytes = 1 << 16
+    [[maybe_unused]] const uint32_t table_bits = plane ? 0x10101010u : 0u;               // 16-entry tables: kTab16Bytes = 16 entries
+    [[maybe_unused]] const uint32_t laneoff_res = laneoff | (1u << 16);                   // BOTH: the residual plane's table
+    static_assert(kLut256Bytes == (1 << 16), "the table number sits in bits 16.. of a table address");
     const int out = a.L.out_features;
     const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
     constexpr bool use_res = (MODE == kSharedLut) || BOTH;  // second 16-byte load per row
@@ -344,10 +352,10 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
                 pv[1] = *reinterpret_cast<const uint32_t*>(smem + entry_addr<1>(pw[d], laneoff));
                 pv[2] = *reinterpret_cast<const uint32_t*>(smem + entry_addr<2>(pw[d], laneoff));
                 pv[3] = *reinterpret_cast<const uint32_t*>(smem + entry_addr<3>(pw[d], laneoff));
-                qv[0] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<0>(qw[d], laneoff));
-                qv[1] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<1>(qw[d], laneoff));
-                qv[2] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<2>(qw[d], laneoff));
-                qv[3] = *reinterpret_cast<const uint32_t*>(smem + kLut256Bytes + entry_addr<3>(qw[d], laneoff));
+                qv[0] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<0>(qw[d], laneoff_res));
+                qv[1] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<1>(qw[d], laneoff_res));
+                qv[2] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<2>(qw[d], laneoff_res));
+                qv[3] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<3>(qw[d], laneoff_res));
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {        // byte 4 d + j: columns 8 d + 2 j and 8 d + 2 j + 1
                     const int c = 8 * d + 2 * j;
@@ -361,15 +369,15 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
             return;
         }
         if constexpr (PT) {
-            const char* tabp = smem + plane * kLut256Bytes;
+            // (the table of the wave's plane: 64 KB per plane, the plane number travels in the address permute)
             const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
             uint32_t pv[16];
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                pv[4 * d + 0] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<0>(pw[d], laneoff));
-                pv[4 * d + 1] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<1>(pw[d], laneoff));
-                pv[4 * d + 2] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<2>(pw[d], laneoff));
-                pv[4 * d + 3] = *reinterpret_cast<const uint32_t*>(tabp + entry_addr<3>(pw[d], laneoff));
+                pv[4 * d + 0] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<0>(pw[d], laneoff_plane));
+                pv[4 * d + 1] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<1>(pw[d], laneoff_plane));
+                pv[4 * d + 2] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<2>(pw[d], laneoff_plane));
+                pv[4 * d + 3] = *reinterpret_cast<const uint32_t*>(smem + entry_addr_hi<3>(pw[d], laneoff_plane));
             }
             float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
@@ -384,7 +392,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
         }
         float val[kChunk];
         // (dual rotation: the residual table follows the primary one, 16 entries of 256 bytes each)
-        lookup32<MODE == kSharedLut, 0>(p, q, smem + plane * kTab16Bytes, laneoff, val);
+        lookup32<MODE == kSharedLut, 0>(p, q, smem, laneoff, val, table_bits);
         if constexpr (PAIR) {
             float s0 = 0.0f, s1 = 0.0f, t0 = 0.0f, t1 = 0.0f;
 #pragma unroll
@@ -528,23 +536,7 @@ __global__ __launch_bounds__(1024) void tq_gemv_wide_group_kernel(GemvGroup g) {
 
 template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false, bool PT = false, bool BOTH = false>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
-    constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
-    const size_t lds = (size_t)kRegion + kPartialBytes + (PRE ? 0 : (size_t)a.img_cols * sizeof(float));
-    auto* kernel = tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE, PT, BOTH>;
-    // More LDS than the default limit has to be asked for, once per kernel and device (any host
-    // thread may get here first; asking twice is harmless).
-    static std::atomic<bool> asked[64];
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64 || !asked[dev].load(std::memory_order_acquire)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kRegion + kPartialBytes +
-                                    ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float));
-        if (e != hipSuccess) return e;
-        if (dev >= 0 && dev < 64) asked[dev].store(true, std::memory_order_release);
-    }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a);
+    hipLaunchKernelGGL((tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE, PT, BOTH>), dim3(grid), dim3(threads), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -628,21 +620,8 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
 }
 
 template <int MODE, int R, bool PAIR, bool PT>
-hipError_t launch_group_one(const GemvGroup& g, int grid, int threads, size_t lds, hipStream_t stream) {
-    auto* kernel = tq_gemv_wide_group_kernel<MODE, R, PAIR, PT>;
-    static std::atomic<bool> asked[64];
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64 || !asked[dev].load(std::memory_order_acquire)) {
-        constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kRegion + kPartialBytes +
-                                    ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float));
-        if (e != hipSuccess) return e;
-        if (dev >= 0 && dev < 64) asked[dev].store(true, std::memory_order_release);
-    }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, g);
+hipError_t launch_group_one(const GemvGroup& g, int grid, int threads, hipStream_t stream) {
+    hipLaunchKernelGGL((tq_gemv_wide_group_kernel<MODE, R, PAIR, PT>), dim3(grid), dim3(threads), 0, stream, g);
     return hipGetLastError();
 }
 
@@ -688,13 +667,11 @@ hipError_t launch_group_mode(GemvGroup& g, int n, int num_cus, hipStream_t strea
         const int max_rows = g.a[j].rows_q + (g.a[j].rows_rem ? 1 : 0);
         g.a[j].iters = (max_rows + R * per_r - 1) / (R * per_r);
     }
-    constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;
-    const size_t lds = (size_t)kRegion + kPartialBytes + (size_t)slabs * kSlab * sizeof(float);
     if constexpr (MODE != kSharedLut) {
-        if (R == 4) return launch_group_one<MODE, 4, PAIR, PT>(g, used, threads, lds, stream);
+        if (R == 4) return launch_group_one<MODE, 4, PAIR, PT>(g, used, threads, stream);
     }
-    if (R == 2) return launch_group_one<MODE, 2, PAIR, PT>(g, used, threads, lds, stream);
-    return launch_group_one<MODE, 1, PAIR, PT>(g, used, threads, lds, stream);
+    if (R == 2) return launch_group_one<MODE, 2, PAIR, PT>(g, used, threads, stream);
+    return launch_group_one<MODE, 1, PAIR, PT>(g, used, threads, stream);
 }
 
 }  // namespace
