@@ -415,49 +415,50 @@ def main():
         del handles
         torch.cuda.empty_cache()
 
-        # ---- prefill: Qwen2.5-32B up-projection 27648 x 5120, M = 512 and 2048, bf16 in / bf16 out ----
-        outp, inp = 27648, 5120
-        hp, _ = make_layer(tq, torch, outp, inp, bs, seed=500, sigma=0.01, shared=True, per_layer_codebooks=True)
-        for M in (512, 2048):
-            xp = torch.randn(M, inp, device="cuda", generator=g).to(torch.bfloat16)
-            yp = torch.empty(M, outp, device="cuda", dtype=torch.bfloat16)
-            L = tq.lib()
-            for _ in range(2):
-                if L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None) != 0:
-                    raise RuntimeError(tq.last_error())
-            torch.cuda.synchronize()
-            st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            reps = 10
-            st.record()
-            for _ in range(reps):
-                L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None)
-            en.record()
-            torch.cuda.synchronize()
-            usp = st.elapsed_time(en) * 1e3 / reps
-            flops = 2.0 * M * outp * inp
-            # The vendor library's plain bf16 GEMM of the same shape on already dequantised weights
-            # (torch.matmul -> hipBLASLt): what a matrix kernel with no decode work reaches on this machine.
-            wv = (torch.randn(outp, inp, device="cuda", generator=g) * 0.01).to(torch.bfloat16)
-            for _ in range(3):
-                torch.matmul(xp, wv.t(), out=yp)
-            st.record()
-            for _ in range(reps):
-                torch.matmul(xp, wv.t(), out=yp)
-            en.record()
-            torch.cuda.synchronize()
-            usv = st.elapsed_time(en) * 1e3 / reps
-            del wv
-            extra[f"prefill_27648x5120_M{M}_bf16"] = {"us_per_layer": usp, "tflops": flops / usp / 1e6,
-                                                      "vendor_plain_bf16_gemm_same_shape_us": usv,
-                                                      "vendor_plain_bf16_gemm_tflops": flops / usv / 1e6,
-                                                      "speed_relative_to_vendor_plain_gemm": usv / usp,
-                                                      "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
-                                                      "frac_of_measured_mfma_loop_random_operands":
-                                                          flops / usp / 1e6 / probes.get("mfma_f16_tflops_random_operands",
-                                                                                         float("nan")),
-                                                      "includes": "activation rotation kernel + dequant/MFMA GEMM kernel"}
-        tq.lib().tq_linear_free(hp)
-        torch.cuda.empty_cache()
+        # ---- prefill: Qwen2.5-32B up-projection 27648 x 5120 at M = 512 and 2048, and the down projection
+        # 5120 x 27648 at M = 512 (40 output tiles for 256 CUs: K is cut into ranges), bf16 in / bf16 out ----
+        for outp, inp, token_counts in ((27648, 5120, (512, 2048)), (5120, 27648, (512,))):
+            hp, _ = make_layer(tq, torch, outp, inp, bs, seed=500, sigma=0.01, shared=True, per_layer_codebooks=True)
+            for M in token_counts:
+                xp = torch.randn(M, inp, device="cuda", generator=g).to(torch.bfloat16)
+                yp = torch.empty(M, outp, device="cuda", dtype=torch.bfloat16)
+                L = tq.lib()
+                for _ in range(2):
+                    if L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None) != 0:
+                        raise RuntimeError(tq.last_error())
+                torch.cuda.synchronize()
+                st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                reps = 10
+                st.record()
+                for _ in range(reps):
+                    L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None)
+                en.record()
+                torch.cuda.synchronize()
+                usp = st.elapsed_time(en) * 1e3 / reps
+                flops = 2.0 * M * outp * inp
+                # The vendor library's plain bf16 GEMM of the same shape on already dequantised weights
+                # (torch.matmul -> hipBLASLt): what a matrix kernel with no decode work reaches on this machine.
+                wv = (torch.randn(outp, inp, device="cuda", generator=g) * 0.01).to(torch.bfloat16)
+                for _ in range(3):
+                    torch.matmul(xp, wv.t(), out=yp)
+                st.record()
+                for _ in range(reps):
+                    torch.matmul(xp, wv.t(), out=yp)
+                en.record()
+                torch.cuda.synchronize()
+                usv = st.elapsed_time(en) * 1e3 / reps
+                del wv
+                extra[f"prefill_{outp}x{inp}_M{M}_bf16"] = {"us_per_layer": usp, "tflops": flops / usp / 1e6,
+                                                          "vendor_plain_bf16_gemm_same_shape_us": usv,
+                                                          "vendor_plain_bf16_gemm_tflops": flops / usv / 1e6,
+                                                          "speed_relative_to_vendor_plain_gemm": usv / usp,
+                                                          "mfma_frac_of_2500_tflops": flops / usp / 1e6 / 2500.0,
+                                                          "frac_of_measured_mfma_loop_random_operands":
+                                                              flops / usp / 1e6 / probes.get("mfma_f16_tflops_random_operands",
+                                                                                             float("nan")),
+                                                          "includes": "activation rotation kernel + dequant/MFMA GEMM kernel (+ the sum of the K ranges where K is cut)"}
+            tq.lib().tq_linear_free(hp)
+            torch.cuda.empty_cache()
 
         # ---- decode MLP block, Qwen2.5-7B shape: gate/up 18944 x 3584, down 3584 x 18944, batch 1 ----
         L = tq.lib()

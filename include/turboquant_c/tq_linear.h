@@ -100,7 +100,7 @@ int tq_linear_forward(tq_linear_t layer, const void* x_dev, int x_dtype, int bat
 /**
  * Size the layer's workspaces for calls of up to max_batch rows now, so that no later
  * tq_linear_forward / tq_linear_forward_group call with at most that many rows allocates (the
- * matrix-core paths for 2 or more rows of 16-bit activations otherwise allocate on first use, which
+ * matrix-core paths for 2 or more rows of 16-bit activations and for 16 or more rows of any type otherwise allocate on first use, which
  * synchronises the device and cannot be captured in a HIP graph; a call that would have to grow a
  * workspace while its stream is being captured fails instead).  The reference allocates its output
  * per call (src/dequantizer.cpp:516) and has no such entry.
@@ -111,12 +111,15 @@ int tq_linear_reserve(tq_linear_t layer, int max_batch);
  * tq_linear_forward for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
  * kernels and the same results as tq_linear_forward, but the workspaces of the matrix-core paths
- * (2 or more rows of 16-bit activations: rotated activations and per-chunk partial products) live in
- * a fixed array of TQ_STATIC_SCRATCH_BYTES inside the library instead of buffers the handle allocates
- * on first use; the call allocates and frees nothing.  It fails (non-zero, tq_last_error says how many
- * bytes were needed) when layer and batch need more than that.  Each GPU has one such array, shared
+ * (2 or more rows of 16-bit activations, 16 or more rows of any type: rotated activations and partial
+ * products) live in a fixed array of TQ_STATIC_SCRATCH_BYTES inside the library instead of buffers the
+ * handle allocates on first use; the call allocates and frees nothing.  It fails (non-zero,
+ * tq_last_error says how many bytes were needed) when layer and batch need more than that.  (From 16
+ * rows on, a layer with few output tiles cuts K into ranges whose fp32 products are added afterwards:
+ * here into as many ranges as the array holds, so the last bits of a result can differ from
+ * tq_linear_forward's by the order of those sums.)  Each GPU has one such array, shared
  * by every call on it and keeping the previous call's contents: calls that overlap on one GPU
- * (different streams or threads) race.  One row, and fp32 activations, use no workspace.
+ * (different streams or threads) race.  One row, and 2 to 15 rows of fp32 activations, use no workspace.
  */
 #define TQ_STATIC_SCRATCH_BYTES (32u << 20)
 int tq_linear_forward_static(tq_linear_t layer, const void* x_dev, int x_dtype, int batch,

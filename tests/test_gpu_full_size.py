@@ -1,6 +1,6 @@
 """Parity at the full sizes of the benchmark configurations (4096 x 4096, the 151936 x 2048
 lm_head, the 18944 x 3584 / 3584 x 18944 MLP block, the 27648 x 5120 up-projection at 512 and 2048
-tokens, the 5120 x 27648 down projection at 4 and 8 rows).
+tokens, the 5120 x 27648 down projection at 4 and 8 rows and at 40, 512 and 2048 tokens).
 
 A whole-matrix fp32 reference product is too slow for the CPU oracle at these sizes, so each case
 is checked three ways:
@@ -306,4 +306,35 @@ def test_down_projection_5120x27648_small_batch(tq, oracle, batch, shared):
     y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)          # exact fp32 batch-1 kernel
     assert _rel(y1[0], want[batch - 1]) < 1e-3
     assert _rel(y[batch - 1:batch], y1) < 1e-3
+    layer.close()
+
+
+@pytest.mark.parametrize("shared", [True, False], ids=["shared_rotation", "dual_rotation"])
+def test_down_projection_5120x27648_prefill_few_output_tiles(tq, oracle, shared):
+    """32B-shaped down projection at 512 and 40 tokens: 2 x 20 (1 x 20) output tiles for 256 CUs, so K is cut
+    into 6 (12) ranges of 144 (72) steps whose fp32 products a second kernel adds.  All tokens against
+    sampled rows of the oracle's weight, every output tile hit; 2048 tokens (160 tiles, one range) on a
+    token slice for comparison."""
+    o = oracle
+    out_f, in_f, bs = 5120, 27648, 512
+    layer, w_ref, qw, cp, cr = _full_layer(tq, o, out_f, in_f, bs, 0.01, 61, shared)
+    rs = np.random.default_rng(62)
+    rows = np.sort(np.concatenate([t * 256 + rs.choice(256, 6, replace=False) for t in range(out_f // 256)]))
+    w_rows = np.ascontiguousarray(w_ref[rows])
+    del w_ref
+    xbits = o.f32_to_bf16_bits(rs.standard_normal((2048, in_f)).astype(np.float32))
+    x = o.bf16_bits_to_f32(xbits)
+    o.set_threads(8)
+    want = o.matmul_xwT(x, w_rows, acc_double=True)                      # [2048, 120]
+    o.set_threads(1)
+    for m in (512, 40, 2048):
+        y = layer.forward(xbits[:m], tq.BF16, tq.F32)
+        assert y.shape == (m, out_f) and np.isfinite(y).all()
+        assert _rel(y[:, rows], want[:m]) < 1e-3
+        for n0 in range(0, len(rows), 6):                                # no output tile is off
+            assert _rel(y[:, rows[n0:n0 + 6]], want[:m, n0:n0 + 6]) < 1e-3
+        for t0 in range(0, m, 256):                                      # nor a token tile
+            assert _rel(y[t0:t0 + 256][:, rows], want[t0:min(t0 + 256, m)]) < 1e-3
+    yb = o.bf16_bits_to_f32(layer.forward(xbits[:512], tq.BF16, tq.BF16))
+    assert _rel(yb[:, rows], want[:512]) < 5e-3
     layer.close()

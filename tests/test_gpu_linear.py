@@ -285,7 +285,9 @@ def test_error_conventions(tq, oracle):
                                               (256, 5120, 512, 300), (1000, 896 * 2, 128, 17),
                                               # K = 64, 192, 256, 384: 2, 6, 8, 12 steps of the 6-step pipeline
                                               (70, 64, 64, 16), (40, 192, 64, 20), (33, 256, 256, 300),
-                                              (257, 384, 128, 513)])
+                                              (257, 384, 128, 513),
+                                              # few output tiles: K is cut into ranges (5 of 32 steps; 34 + 34 + 32; 7 x 34 + 20)
+                                              (256, 5120, 512, 40), (130, 3200, 128, 40), (90, 8256, 64, 130)])
 def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, batch):
     """batch >= 16 takes the MFMA path whatever the activation type (fp16 weight tiles, fp16 rotated
     activations, fp32 accumulation): 1e-3 relative L2 against dequantise + fp32 matmul, 5e-3 where the

@@ -130,6 +130,35 @@ def test_static_forward_two_plane_five_bit_layer(tq, oracle):
     layer.close()
 
 
+def test_static_forward_cuts_k_into_fewer_ranges_when_the_array_is_short(tq, oracle):
+    """1536 x 16384 at 500 tokens: 2 x 6 output tiles, so the allocating entry point cuts K into 16 ranges
+    (16 MiB of tile images + 16 x 2.9 MiB of fp32 products); the static array holds the images and five ranges.
+    Same result up to the order of the fp32 sums, and right against the CPU oracle."""
+    hip = _Hip()
+    o = oracle
+    out, inf, bs, batch = 1536, 16384, 512, 500
+    qw, cb = _make(o, out, inf, bs, "shared")
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    o.set_threads(8)
+    w_ref = o.dequantize_weight_cpu(qw, cb, cb, bs)
+    xbits = o.f32_to_bf16_bits(np.random.default_rng(70).standard_normal((batch, inf)).astype(np.float32))
+    ref = o.matmul_xwT(o.bf16_bits_to_f32(xbits), w_ref, acc_double=True)
+    o.set_threads(1)
+    x_dev = hip.upload(xbits)
+    y_ref_dev, y_dev = hip.alloc(batch * out * 4), hip.alloc(batch * out * 4)
+    layer.forward_device(x_dev, tq.BF16, batch, y_ref_dev, tq.F32)
+    want = hip.download(y_ref_dev, (batch, out), np.float32)
+    for _ in range(2):
+        layer.forward_static_device(x_dev, tq.BF16, batch, y_dev, tq.F32)
+        got = hip.download(y_dev, (batch, out), np.float32)
+        assert _rel(got, want) < 1e-5
+        assert _rel(got, ref) < 1e-3
+        assert hip.rt.hipMemset(y_dev, 0xFF, batch * out * 4) == 0             # the second call starts from NaNs again
+    assert _rel(want, ref) < 1e-3
+    hip.free(x_dev, y_ref_dev, y_dev)
+    layer.close()
+
+
 def test_static_forward_refuses_a_workspace_beyond_the_array(tq, oracle):
     hip = _Hip()
     o = oracle

@@ -60,9 +60,14 @@ hipError_t launch_combine_planes5(const uint8_t* primary, const uint8_t* residua
 hipError_t launch_dequant(const LayerView& L, void* w, int w_dtype, hipStream_t stream);
 // Prefill (tq_prefill.hip): rotate the activations to fp16 in `workspace`, then dequant + MFMA GEMM.
 bool prefill_supported(const LayerView& L, int x_dtype, int batch);
-size_t prefill_workspace_bytes(const LayerView& L, int batch);
+size_t prefill_workspace_bytes(const LayerView& L, int batch);        // the rotated activations (tile images) alone
+// K ranges of a call (splits > 1: few output tiles), their length in 32-column steps, and the workspace: tile
+// images (xt_bytes, rounded up to 256) followed by splits x [batch, out] fp32 products.
+struct PrefillPlan { int splits; int steps_per_split; size_t xt_bytes; size_t total_bytes; };
+PrefillPlan prefill_plan(const LayerView& L, int batch, int num_cus, size_t capacity);
+size_t prefill_reserve_bytes(const LayerView& L, int max_batch, int num_cus);
 hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
-                          void* workspace, hipStream_t stream);
+                          void* workspace, const PrefillPlan& plan, hipStream_t stream);
 hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
                                hipStream_t stream);
 // Small batches (tq_skinny.hip): 2..15 rows of 16-bit activations on shared-rotation layers, batch rows as

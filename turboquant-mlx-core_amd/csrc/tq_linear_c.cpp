@@ -373,8 +373,10 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
     }
     void* work = nullptr;
     float* partial = nullptr;
+    tq::PrefillPlan plan{};
+    if (prefill) plan = tq::prefill_plan(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0);
     if (prefill || skinny) {
-        const size_t work_need = prefill ? tq::prefill_workspace_bytes(V, batch) : tq::skinny_workspace_bytes(V, batch);
+        const size_t work_need = prefill ? plan.total_bytes : tq::skinny_workspace_bytes(V, batch);
         const size_t partial_need = skinny ? tq::skinny_partial_bytes(V, batch) : 0;
         if (static_ws) {
             if (align256(work_need) + partial_need > static_cap) {
@@ -395,7 +397,7 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
     }
     if (prefill) {
         // Dense contraction: rotate once, dequantise tiles to fp16 in LDS, MFMA.
-        return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, stream),
+        return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, plan, stream),
                       "tq_prefill launch") ? 0 : 1;
     }
     if (skinny) {
@@ -504,7 +506,7 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
             for (int k = 0; k < 2; ++k) {
                 const tq::LayerView& P = h->plane_view[k];
                 const size_t small = tq::skinny_workspace_bytes(P, max_batch < 15 ? max_batch : 15);
-                const size_t big = max_batch >= 16 ? tq::prefill_workspace_bytes(P, max_batch) : 0;
+                const size_t big = max_batch >= 16 ? tq::prefill_reserve_bytes(P, max_batch, device_cu_count()) : 0;
                 work = std::max(work, std::max(small, big));
                 part = std::max(part, tq::skinny_partial_bytes(P, max_batch < 15 ? max_batch : 15));
             }
@@ -515,7 +517,7 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
         }
         const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
         const size_t small = tq::skinny_workspace_bytes(V, max_batch < 15 ? max_batch : 15);
-        const size_t big = max_batch >= 16 ? tq::prefill_workspace_bytes(V, max_batch) : 0;
+        const size_t big = max_batch >= 16 ? tq::prefill_reserve_bytes(V, max_batch, device_cu_count()) : 0;
         if (!ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big, nullptr, &h->retired)) return 1;
         if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < 15 ? max_batch : 15), nullptr, &h->retired)) return 1;
         return 0;

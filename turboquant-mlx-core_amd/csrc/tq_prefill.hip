@@ -49,6 +49,11 @@ struct PrefillArgs {
     int mode;
     int m_tiles, n_tiles;
     float out_scale;
+    // K cut into ranges (blockIdx.y) when the output tiles alone would leave most CUs idle: a range is
+    // steps_per_split 32-column steps (even; the last range may be shorter), and every workgroup writes
+    // its fp32 products to partial[range][M][N] instead of y (NULL: one range, y written directly).
+    int steps_per_split;
+    float* partial;
 };
 
 __device__ __forceinline__ uint32_t gemm_entry_addr(uint32_t idx_bytes, uint32_t laneoff, int j) {
@@ -91,23 +96,27 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs (id % 8), so the
     // M tiles that share one N tile of weights are given to the same XCD back to back.
+    // With K ranges (few tiles) the tiles are numbered densely instead: an XCD would otherwise be handed
+    // whole N tiles times all ranges, more workgroups than it has CUs, while others idle.
     const int id = blockIdx.x;
     const int xcd = id & 7, slot = id >> 3;
-    const int n_tile = (slot / a.m_tiles) * 8 + xcd;
-    const int m_tile = slot % a.m_tiles;
+    const int n_tile = a.partial ? id / a.m_tiles : (slot / a.m_tiles) * 8 + xcd;
+    const int m_tile = a.partial ? id % a.m_tiles : slot % a.m_tiles;
     if (n_tile >= a.n_tiles) return;                       // whole workgroup leaves together
     const int m0 = m_tile * kBM, n0 = n_tile * kBN;
 
     constexpr bool combined = (MODE == kSharedLut);
     constexpr int kPlanes = (MODE == kDual) ? 2 : 1;
-    const int T = a.K / kBK;                               // 32-column steps (even)
-    const int G = a.K / kKLoad;                            // 64-column index stages
+    const int T_all = a.K / kBK;                           // 32-column steps of the whole row (even)
+    const int t_begin = (int)blockIdx.y * a.steps_per_split;          // this workgroup's K range
+    const int T = T_all - t_begin < a.steps_per_split ? T_all - t_begin : a.steps_per_split;   // its steps (even)
+    const int G = T / 2;                                   // 64-column index stages
 
     // Weight loader mapping: thread -> (tile row, 16-column half of a 32-column tile).
     const int lrow = tid >> 1, lh = tid & 1;
     const int b_row = (n0 + lrow < a.N) ? n0 + lrow : a.N - 1;
-    const uint32_t b_voff = combined ? (uint32_t)b_row * (uint32_t)a.K + lh * 16
-                                     : (uint32_t)b_row * (uint32_t)(a.K >> 1) + lh * 8;
+    const uint32_t b_voff = combined ? (uint32_t)b_row * (uint32_t)a.K + (uint32_t)t_begin * kBK + lh * 16
+                                     : (uint32_t)b_row * (uint32_t)(a.K >> 1) + (uint32_t)t_begin * (kBK / 2) + lh * 8;
     // Activation copy: wave w moves bytes [2048 w, 2048 w + 2048) of every 16 KB tile image.
     const uint32_t dma_voff = (uint32_t)wave * 2048 + (uint32_t)lane * 16;
     const uint32_t lds_base = (uint32_t)(uintptr_t)smem;
@@ -133,7 +142,7 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         const char* a_tiles = reinterpret_cast<const char*>(a.xt) +
-                              ((size_t)plane * a.m_tiles + m_tile) * (size_t)T * kATile;
+                              (((size_t)plane * a.m_tiles + m_tile) * (size_t)T_all + t_begin) * kATile;
         const uint8_t* w_plane = combined ? a.plane0 : (plane == 0 ? a.plane0 : a.plane1);
 
         // Activation tile t -> LDS tile `buf`, straight from global memory.
@@ -337,16 +346,19 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
     // Epilogue: * norm[n] / sqrt(in * bs), convert, store.  Each wave transposes its 128 x 64 tile
     // through a private LDS region so that every store instruction writes whole 128-byte rows;
     // row counts that break the 16-byte alignment of those stores take the element-wise path.
+    // (K ranges: the raw fp32 products go to this range's slice of the partial buffer; the sum kernel scales)
+    void* const y_out = a.partial ? static_cast<void*>(a.partial + (size_t)blockIdx.y * a.M * a.N) : a.y;
+    const int y_type = a.partial ? (int)kF32 : a.y_dtype;
     float scale[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int col = n0 + wn * 64 + j * 32 + (lane & 31);
-        scale[j] = col < a.N ? a.out_scale * a.norms[col] : 0.0f;
+        scale[j] = col < a.N ? (a.partial ? 1.0f : a.out_scale * a.norms[col]) : 0.0f;
     }
     constexpr int kEpiPitch = 144;                                   // 128 data bytes + 16: conflict-light, 16-byte aligned
     char* const stage = smem + wave * (128 * kEpiPitch);
     const int row_base = m0 + wm * 128, col_base = n0 + wn * 64;
-    if (a.y_dtype != kF32 && (a.N & 7) == 0) {
+    if (y_type != kF32 && (a.N & 7) == 0) {
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -355,11 +367,11 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
                 for (int r = 0; r < 16; ++r) {
                     const int row = i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
                     const float v = acc[i][j][r] * scale[j];
-                    const uint16_t h = a.y_dtype == kBF16 ? float_to_bf16_bits(v)
+                    const uint16_t h = y_type == kBF16 ? float_to_bf16_bits(v)
                                                           : __builtin_bit_cast(uint16_t, (_Float16)v);
                     *reinterpret_cast<uint16_t*>(stage + row * kEpiPitch + (j * 32 + (lane & 31)) * 2) = h;
                 }
-        uint16_t* y = static_cast<uint16_t*>(a.y);
+        uint16_t* y = static_cast<uint16_t*>(y_out);
 #pragma unroll
         for (int it = 0; it < 16; ++it) {
             const int row = it * 8 + (lane >> 3), piece = lane & 7;
@@ -367,8 +379,8 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
             const int grow = row_base + row, gcol = col_base + piece * 8;
             if (grow < a.M && gcol < a.N) *reinterpret_cast<u32x4v*>(y + (size_t)grow * a.N + gcol) = v;
         }
-    } else if (a.y_dtype == kF32 && (a.N & 3) == 0) {
-        float* y = static_cast<float*>(a.y);
+    } else if (y_type == kF32 && (a.N & 3) == 0) {
+        float* y = static_cast<float*>(y_out);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -396,7 +408,7 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
                 for (int r = 0; r < 16; ++r) {
                     const int row = row_base + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
                     if (col < a.N && row < a.M)
-                        store_scalar(a.y, a.y_dtype, (size_t)row * a.N + col, acc[i][j][r] * scale[j]);
+                        store_scalar(y_out, y_type, (size_t)row * a.N + col, acc[i][j][r] * scale[j]);
                 }
         }
     }
@@ -443,10 +455,76 @@ __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restri
     }
 }
 
+// Sum of the K ranges: y[m, n] = out_scale * norm[n] * (partial[0][m, n] + partial[1][m, n] + ...), ranges added
+// in their order.  One thread per four neighbouring outputs (QUAD: N is a multiple of 4) or per output.
+template <bool QUAD>
+__global__ __launch_bounds__(256) void tq_prefill_sum_kernel(const float* __restrict__ partial, int splits,
+                                                              const float* __restrict__ norms, float out_scale,
+                                                              void* __restrict__ y, int y_dtype, int M, int N) {
+    const size_t total = (size_t)M * N;
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * (QUAD ? 4 : 1);
+    if (i >= total) return;
+    const int n = (int)(i % (size_t)N);
+    if constexpr (QUAD) {
+        float4 s = *reinterpret_cast<const float4*>(partial + i);
+        for (int k = 1; k < splits; ++k) {
+            const float4 v = *reinterpret_cast<const float4*>(partial + (size_t)k * total + i);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        store_scalar(y, y_dtype, i, s.x * (out_scale * norms[n]));          // (the caller's norms need not be 16-byte aligned)
+        store_scalar(y, y_dtype, i + 1, s.y * (out_scale * norms[n + 1]));
+        store_scalar(y, y_dtype, i + 2, s.z * (out_scale * norms[n + 2]));
+        store_scalar(y, y_dtype, i + 3, s.w * (out_scale * norms[n + 3]));
+    } else {
+        float s = partial[i];
+        for (int k = 1; k < splits; ++k) s += partial[(size_t)k * total + i];
+        store_scalar(y, y_dtype, i, s * (out_scale * norms[n]));
+    }
+}
+
 size_t prefill_workspace_bytes(const LayerView& L, int batch) {
     const size_t planes = (L.mode == kDual) ? 2 : 1;
     const size_t m_tiles = ((size_t)batch + kBM - 1) / kBM;            // whole tile images
     return planes * m_tiles * kBM * L.in_features * sizeof(uint16_t);
+}
+
+// How a call is cut.  With fewer output tiles than half the CUs (few output rows: the q, o and down projections;
+// few tokens) K is cut into ranges so that about one workgroup per CU runs, no range shorter than 32 steps; the
+// ranges' fp32 products follow the tile images in the workspace.  capacity: bytes the caller can give
+// (fewer ranges are used where the products would not fit).
+PrefillPlan prefill_plan(const LayerView& L, int batch, int num_cus, size_t capacity) {
+    PrefillPlan p{};
+    const int steps = L.in_features / kBK;
+    const long long tiles = (long long)((batch + kBM - 1) / kBM) * ((L.out_features + kBN - 1) / kBN);
+    p.xt_bytes = (prefill_workspace_bytes(L, batch) + 255) & ~(size_t)255;
+    int splits = 1;
+    if (tiles * 2 <= num_cus) {
+        splits = (int)(num_cus / tiles);
+        if (splits > steps / 32) splits = steps / 32;
+        if (splits < 1) splits = 1;
+    }
+    const size_t one = (size_t)batch * L.out_features * sizeof(float);
+    for (;; --splits) {
+        int per = (steps + splits - 1) / splits;
+        per += per & 1;                                               // even: the kernel steps in pairs
+        p.steps_per_split = per;
+        p.splits = (steps + per - 1) / per;
+        p.total_bytes = p.xt_bytes + (p.splits > 1 ? (size_t)p.splits * one : 0);
+        if (p.splits == 1 || p.total_bytes <= capacity) break;
+    }
+    return p;
+}
+
+// Largest workspace any call of 16 .. max_batch rows needs (fewer rows can mean more ranges).
+size_t prefill_reserve_bytes(const LayerView& L, int max_batch, int num_cus) {
+    size_t need = 0;
+    for (int m_tiles = 1; (m_tiles - 1) * kBM < max_batch; ++m_tiles) {
+        const int rows = m_tiles * kBM < max_batch ? m_tiles * kBM : max_batch;
+        if (rows < 16) continue;
+        const size_t n = prefill_plan(L, rows, num_cus, ~(size_t)0).total_bytes;
+        if (n > need) need = n;
+    }
+    return need;
 }
 
 bool prefill_supported(const LayerView& L, int x_dtype, int batch) {
@@ -477,7 +555,7 @@ hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, i
 }
 
 hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
-                          void* workspace, hipStream_t stream) {
+                          void* workspace, const PrefillPlan& plan, hipStream_t stream) {
     const int K = L.in_features, N = L.out_features, M = batch;
     uint16_t* xt = static_cast<uint16_t*>(workspace);
     hipError_t e = launch_rotate_tiles(L, x, x_dtype, batch, workspace, stream);
@@ -494,16 +572,28 @@ hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int ba
     a.m_tiles = (M + kBM - 1) / kBM;
     a.n_tiles = (N + kBN - 1) / kBN;
     a.out_scale = L.inv_scale;                          // (1 / sqrt(bs) is in the rotated activations)
+    a.steps_per_split = plan.steps_per_split;
+    a.partial = plan.splits > 1 ? reinterpret_cast<float*>(static_cast<char*>(workspace) + plan.xt_bytes) : nullptr;
     const int n_groups = (a.n_tiles + 7) / 8;
-    const unsigned grid = (unsigned)(n_groups * 8 * a.m_tiles);
+    // (x: tiles, in XCD-aware order or, with K ranges, densely numbered; y: K ranges)
+    const dim3 grid((unsigned)(plan.splits > 1 ? a.n_tiles * a.m_tiles : n_groups * 8 * a.m_tiles), (unsigned)plan.splits);
     switch (L.mode) {
         case kSharedLut:
-            hipLaunchKernelGGL(tq_prefill_gemm_kernel<kSharedLut>, dim3(grid), dim3(kGemmThreads), 0, stream, a); break;
+            hipLaunchKernelGGL(tq_prefill_gemm_kernel<kSharedLut>, grid, dim3(kGemmThreads), 0, stream, a); break;
         case kDual:
-            hipLaunchKernelGGL(tq_prefill_gemm_kernel<kDual>, dim3(grid), dim3(kGemmThreads), 0, stream, a); break;
+            hipLaunchKernelGGL(tq_prefill_gemm_kernel<kDual>, grid, dim3(kGemmThreads), 0, stream, a); break;
         default:
-            hipLaunchKernelGGL(tq_prefill_gemm_kernel<kPrimaryOnly>, dim3(grid), dim3(kGemmThreads), 0, stream, a); break;
+            hipLaunchKernelGGL(tq_prefill_gemm_kernel<kPrimaryOnly>, grid, dim3(kGemmThreads), 0, stream, a); break;
     }
+    e = hipGetLastError();
+    if (e != hipSuccess || plan.splits == 1) return e;
+    const size_t total = (size_t)M * N;
+    if ((N & 3) == 0)
+        hipLaunchKernelGGL(tq_prefill_sum_kernel<true>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
+                           a.partial, plan.splits, L.norms, L.inv_scale, y, y_dtype, M, N);
+    else
+        hipLaunchKernelGGL(tq_prefill_sum_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                           a.partial, plan.splits, L.norms, L.inv_scale, y, y_dtype, M, N);
     return hipGetLastError();
 }
 
