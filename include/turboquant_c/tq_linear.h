@@ -100,7 +100,7 @@ int tq_linear_forward(tq_linear_t layer, const void* x_dev, int x_dtype, int bat
 /**
  * Size the layer's workspaces for calls of up to max_batch rows now, so that no later
  * tq_linear_forward / tq_linear_forward_group call with at most that many rows allocates (the
- * matrix-core paths for 2 or more rows of 16-bit activations and for 16 or more rows of any type otherwise allocate on first use, which
+ * matrix-core paths for 2 or more rows otherwise allocate on first use, which
  * synchronises the device and cannot be captured in a HIP graph; a call that would have to grow a
  * workspace while its stream is being captured fails instead).  The reference allocates its output
  * per call (src/dequantizer.cpp:516) and has no such entry.
@@ -111,7 +111,7 @@ int tq_linear_reserve(tq_linear_t layer, int max_batch);
  * tq_linear_forward for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
  * kernels and the same results as tq_linear_forward, but the workspaces of the matrix-core paths
- * (2 or more rows of 16-bit activations, 16 or more rows of any type: rotated activations and partial
+ * (2 or more rows: rotated activations and partial
  * products) live in a fixed array of TQ_STATIC_SCRATCH_BYTES inside the library instead of buffers the
  * handle allocates on first use; the call allocates and frees nothing.  It fails (non-zero,
  * tq_last_error says how many bytes were needed) when layer and batch need more than that.  (From 16
@@ -119,7 +119,7 @@ int tq_linear_reserve(tq_linear_t layer, int max_batch);
  * here into as many ranges as the array holds, so the last bits of a result can differ from
  * tq_linear_forward's by the order of those sums.)  Each GPU has one such array, shared
  * by every call on it and keeping the previous call's contents: calls that overlap on one GPU
- * (different streams or threads) race.  One row, and 2 to 15 rows of fp32 activations, use no workspace.
+ * (different streams or threads) race.  One row uses no workspace.
  */
 #define TQ_STATIC_SCRATCH_BYTES (32u << 20)
 int tq_linear_forward_static(tq_linear_t layer, const void* x_dev, int x_dtype, int batch,
@@ -129,7 +129,7 @@ int tq_linear_forward_static(tq_linear_t layer, const void* x_dev, int x_dtype, 
  * One to three layers applied to the SAME activations: y_devs[j][batch, out_j] = x[batch, in] . W_j^T,
  * e.g. the q, k, v or the gate, up projections of a decoder layer.  Layers of equal width and mode share
  * their kernel launches where the kernels allow it (batch 1: shared or dual rotation, blocks <= 512, more
- * than 2048 columns for shared rotation; 2..15 rows of 16-bit activations: blocks <= 512);
+ * than 2048 columns for shared rotation; 2..15 rows: blocks <= 512);
  * anything else is run one layer after the other.  Results are identical to n calls of tq_linear_forward.
  * No counterpart in the reference, whose forward is per layer (include/turboquant/linear.h:21-22).
  */

@@ -11,10 +11,10 @@
  * (src/dequantizer.cpp:606-721).  This entry point keeps the intermediates in buffers
  * owned by the block and enqueues the whole block on one stream without allocating,
  * so it can be captured in a HIP graph.  gate and up have their own seeds and
- * codebooks, so each rotates the activation for itself.  Batch 1 and fp32 activations:
- * the gate is folded into the store of the up projection (three kernels in all).  Two
- * or more rows of 16-bit activations: the three layers run on the matrix cores with
- * one elementwise kernel in between, the activation handed on as fp32 (16 rows or more) or bf16.
+ * codebooks, so each rotates the activation for itself.  Batch 1: the gate is folded
+ * into the store of the up projection (three kernels in all).  Two or more rows: the
+ * three layers run on the matrix cores with one elementwise kernel in between, the
+ * activation handed on as fp32.
  */
 
 #include "tq_linear.h"

@@ -155,12 +155,14 @@ def test_forward_batch1_wide_rows(tq, oracle, mode, out, inf, bs):
     xb = oracle.bf16_bits_to_f32(xbits)
     yb = layer.forward(xbits, tq.BF16, tq.F32)
     assert _rel(yb, oracle.linear_forward(qw, cbp, cbr, bs, xb)) < 1e-3
-    # three rows of fp32 activations: the first two go through the two-row kernel, the third alone.
-    # (Nibble planes: the one-row kernel reads centroid pairs rounded to fp16, the two-row kernel fp32
-    # centroids, so the two agree to the fp32 tolerance only.)
+    # three rows of fp32 activations: the small-batch kernels (fp16 operands on the matrix cores where the
+    # width is a multiple of 512, else the fp32 kernels two rows at a time): each row agrees with the one-row
+    # kernel to the forward tolerance, and the rows with each other as their inputs do (factors -1 and 0.5
+    # are exact in fp16 and in fp32).
     x3 = np.concatenate([x, -x, 0.5 * x], axis=0)
     y3 = layer.forward(x3)
-    assert _rel(y3[2:3], 0.5 * y) < 1e-6 and _rel(y3[0:1], y) < (1e-6 if mode == "shared" else 1e-3)
+    assert _rel(y3[0:1], y) < 1e-3 and _rel(y3, oracle.linear_forward(qw, cbp, cbr, bs, x3)) < 1e-3
+    assert _rel(y3[1:2], -y3[0:1]) < 1e-6 and _rel(y3[2:3], 0.5 * y3[0:1]) < 1e-6
     layer.close()
 
 
@@ -224,9 +226,10 @@ def test_forward_batch1_rows_beyond_16384_columns(tq, oracle, mode, out, inf, bs
     yh = layer.forward(xh, tq.F16, tq.F32)
     assert _rel(yh, oracle.linear_forward(qw, cbp, cbr, bs, xh.astype(np.float32))) < 1e-3
     assert np.array_equal(layer.forward(x), y)                             # the scratch holds nothing stale
-    x3 = np.concatenate([x, -x, 0.5 * x], axis=0)                          # three rows, one launch pair each
+    x3 = np.concatenate([x, -x, 0.5 * x], axis=0)                          # three rows: the small-batch kernels
     y3 = layer.forward(x3)
-    assert _rel(y3[2:3], 0.5 * y) < 1e-6 and _rel(y3[0:1], y) < 1e-6 and _rel(y3[1:2], -y) < 1e-6
+    assert _rel(y3[0:1], y) < 1e-3 and _rel(y3, oracle.linear_forward(qw, cbp, cbr, bs, x3)) < 1e-3
+    assert _rel(y3[1:2], -y3[0:1]) < 1e-6 and _rel(y3[2:3], 0.5 * y3[0:1]) < 1e-6
     layer.close()
 
 
@@ -340,7 +343,7 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     assert _rel(y16, oracle.linear_forward(qw, cbp, cbr, bs, x16.astype(np.float32))) < 1e-3
     y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)      # exact fp32 batch-1 kernel
     assert _rel(y[batch - 1:batch], y1) < 1e-3
-    # fp32 activations keep the exact path at any batch
+    # fp32 activations take the same kernels
     yf = layer.forward(x32)
     assert _rel(yf, oracle.linear_forward(qw, cbp, cbr, bs, x32)) < 1e-3
     layer.close()

@@ -401,7 +401,7 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
                       "tq_prefill launch") ? 0 : 1;
     }
     if (skinny) {
-        // 2..15 rows of 16-bit activations: batch rows on the matrix cores, fp16 weights.
+        // 2..15 rows: batch rows on the matrix cores, fp16 weights and rotated activations.
         return hip_ok(tq::launch_skinny(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, partial, device_cu_count(), stream),
                       "tq_skinny launch") ? 0 : 1;
     }
@@ -681,7 +681,7 @@ struct tq_mlp_s {
     int max_batch;
     float* d_gate = nullptr;    // [max_batch, intermediate] fp32
     float* d_up = nullptr;      // [max_batch, intermediate] fp32 (batched path only)
-    void* d_act = nullptr;      // [max_batch, intermediate] fp32 (decode) or bf16 (batched path)
+    void* d_act = nullptr;      // [max_batch, intermediate] fp32
     ~tq_mlp_s() {
         if (d_gate) (void)hipFree(d_gate);
         if (d_up) (void)hipFree(d_up);
@@ -740,15 +740,14 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
                                               nullptr, m->d_gate), "tq_gemv launch") ? 0 : 1;
             }
         }
-        if (batch == 1 || (x_dtype == tq::kF32 && batch < 16)) {
+        if (batch == 1) {
             // decode: three launches, the SiLU gate folded into the store of the up projection
             if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
             if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_act, tq::kF32, st, m->d_gate) != 0) return 1;
             return forward_impl(m->down, m->d_act, tq::kF32, batch, y_dev, y_dtype, st, nullptr);
         }
-        // two or more rows of 16-bit activations, or 16 or more of any type: matrix-core paths for all three
-        // layers (small-batch or prefill kernel), one elementwise kernel; the activation is handed to the down
-        // projection as fp32 where its kernel takes that (16 rows or more), else as bf16
+        // two or more rows: matrix-core paths for all three layers (small-batch or prefill kernel), one
+        // elementwise kernel; the activation is handed to the down projection as fp32
         const tq::LayerView both[2] = {m->gate->has_fwd_view ? m->gate->fwd_view : m->gate->view,
                                        m->up->has_fwd_view ? m->up->fwd_view : m->up->view};
         const bool plain = !(m->gate->view.mode >= tq::kShared5 && !m->gate->has_fwd_view) &&
@@ -763,7 +762,7 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
             if (forward_impl(m->gate, x_dev, x_dtype, batch, m->d_gate, tq::kF32, st, nullptr) != 0) return 1;
             if (forward_impl(m->up, x_dev, x_dtype, batch, m->d_up, tq::kF32, st, nullptr) != 0) return 1;
         }
-        const int act_dtype = batch >= 16 ? tq::kF32 : tq::kBF16;
+        const int act_dtype = tq::kF32;
         if (!hip_ok(tq::launch_silu_mul(m->d_gate, m->d_up, m->d_act, act_dtype, n, st), "silu_mul launch")) return 1;
         return forward_impl(m->down, m->d_act, act_dtype, batch, y_dev, y_dtype, st, nullptr);
     } catch (...) { set_error("tq_mlp_forward: exception"); return 1; }

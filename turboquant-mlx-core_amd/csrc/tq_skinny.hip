@@ -1,4 +1,4 @@
-// TQ8 small-batch forward for gfx950: 2..15 activation rows with 16-bit activations, shared-rotation
+// TQ8 small-batch forward for gfx950: 2..15 activation rows (any activation type), shared-rotation
 // layers (one byte per weight).
 //
 // The batch-1 kernel multiplies every decoded weight with the activation of each batch row on the
@@ -29,7 +29,7 @@ constexpr int kSkLutBytes = 256 * 256;
 constexpr int kSkStageBytes = 16 * kSkChunk * 2;   // 16 rows x 512 fp16 rotated activations
 
 struct SkinnyArgs {
-    const void* x;             // FUSED: activations [batch, K], f16 or bf16
+    const void* x;             // FUSED: activations [batch, K], f32, f16 or bf16
     int x_dtype;
     uint32_t seed, block_size; // FUSED: rotation of the layer (blocks of at most 512 columns)
     float x_scale;             // FUSED: 1 / sqrt(block_size), applied to the rotated activations before they are rounded
@@ -94,9 +94,7 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
 #pragma unroll
         for (int t = 0; t < 2; ++t) {                      // batch rows w and w + 8 (row 0 again past the batch: not used)
             const int b = wave + 8 * t;
-            xin[t].a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) +
-                                                       (size_t)(b < a.batch ? b : 0) * a.K + chunk * kSkChunk + lane * 8);
-            xin[t].b = make_uint4(0, 0, 0, 0);
+            xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, chunk * kSkChunk + lane * 8);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -228,7 +226,7 @@ __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 // reduction kernel adds all units, which is the sum of the two passes.  Blocks of at most 512
 // columns only (the workgroup rotates its chunk itself).
 struct SkinnyNibbleArgs {
-    const void* x;             // activations [batch, K], f16 or bf16
+    const void* x;             // activations [batch, K], f32, f16 or bf16
     int x_dtype;
     uint32_t seed[2], block_size;
     float x_scale;             // 1 / sqrt(block_size), applied to the rotated activations before they are rounded
@@ -283,9 +281,7 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
 #pragma unroll
     for (int t = 0; t < 2; ++t) {                          // batch rows w and w + 8 (row 0 again past the batch: not used)
         const int b = wave + 8 * t;
-        xin[t].a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) +
-                                                   (size_t)(b < a.batch ? b : 0) * a.K + chunk * kSkChunk + lane * 8);
-        xin[t].b = make_uint4(0, 0, 0, 0);
+        xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, chunk * kSkChunk + lane * 8);
     }
     __builtin_amdgcn_sched_barrier(0);
     sk_u32x4 rawA[4], rawB[4];                             // two row groups: one decoded, one in flight
@@ -444,7 +440,7 @@ static bool skinny_nibble(const LayerView& L) {
 }
 
 bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
-    if (x_dtype == kF32 || batch < 2 || batch >= 16 || L.in_features % kSkChunk != 0) return false;
+    if (batch < 2 || batch >= 16 || L.in_features % kSkChunk != 0) return false;   // (any activation type)
     if (!lanes_supported(L.in_features, L.block_size)) return false;
     if (!L.fp16_centroids_ok) return false;                   // decoded weights are kept in fp16
     return (L.mode == kSharedLut && L.packed_combined) || skinny_nibble(L);
@@ -518,7 +514,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
 }
 
 // Layers that can share the two launches: two or three layers of equal width and mode with blocks
-// of at most 512 columns (the workgroup rotates its chunk itself), 2..15 rows of 16-bit activations,
+// of at most 512 columns (the workgroup rotates its chunk itself), 2..15 rows,
 // and at least one workgroup per work unit and layer.
 bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, int num_cus) {
     if (n < 2 || n > 3) return false;
