@@ -129,7 +129,7 @@ int tq_linear_forward_static(tq_linear_t layer, const void* x_dev, int x_dtype, 
  * One to three layers applied to the SAME activations: y_devs[j][batch, out_j] = x[batch, in] . W_j^T,
  * e.g. the q, k, v or the gate, up projections of a decoder layer.  Layers of equal width and mode share
  * their kernel launches where the kernels allow it (batch 1: shared or dual rotation, blocks <= 512, more
- * than 2048 columns for shared rotation; 2..15 rows: blocks <= 512);
+ * than 2048 columns for shared rotation; 2..32 rows: blocks <= 512);
  * anything else is run one layer after the other.  Results are identical to n calls of tq_linear_forward.
  * No counterpart in the reference, whose forward is per layer (include/turboquant/linear.h:21-22).
  */

@@ -272,7 +272,7 @@ def test_forward_group_rejects_bad_arguments(tq, oracle):
 
 
 @pytest.mark.parametrize("shared", [True, False])
-@pytest.mark.parametrize("batch", [2, 5, 8, 15])
+@pytest.mark.parametrize("batch", [2, 5, 8, 15, 16, 27, 32])
 @pytest.mark.parametrize("outs,in_f,bs", [((640, 128, 131), 5120, 512), ((1100, 1000), 4096, 256), ((50, 33), 1024, 512),
                                           ((40, 24), 2048, 1024)])
 def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):

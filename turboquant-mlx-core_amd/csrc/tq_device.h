@@ -70,8 +70,9 @@ hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int ba
                           void* workspace, const PrefillPlan& plan, hipStream_t stream);
 hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
                                hipStream_t stream);
-// Small batches (tq_skinny.hip): 2..15 rows (any activation type) on shared-rotation layers, batch rows as
+// Small batches (tq_skinny.hip): 2..32 rows (any activation type) on shared-rotation layers, batch rows as
 // the M side of 16x16x32 MFMAs.  xt_workspace as for launch_prefill; partial: skinny_partial_bytes() for this batch.
+constexpr int kSkinnyMaxRows = 32;
 bool skinny_supported(const LayerView& L, int x_dtype, int batch);
 size_t skinny_partial_bytes(const LayerView& L, int batch);
 size_t skinny_workspace_bytes(const LayerView& L, int batch);

@@ -364,8 +364,9 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, const void* x_dev, int x_dtype, int batch,
                  void* y_dev, int y_dtype, hipStream_t stream, const float* gate, void* static_ws, size_t static_cap) {
     const bool lanes = !generic_only && tq::lanes_supported(V.in_features, V.block_size);
-    const bool prefill = lanes && !gate && tq::prefill_supported(V, x_dtype, batch);   // (the gated store is a feature of the one-row kernels)
-    const bool skinny = lanes && !prefill && !gate && tq::skinny_supported(V, x_dtype, batch);
+    // (the gated store is a feature of the one-row kernels; 16..32 rows: the small-batch kernel where it takes the layer)
+    const bool skinny = lanes && !gate && tq::skinny_supported(V, x_dtype, batch);
+    const bool prefill = lanes && !skinny && !gate && tq::prefill_supported(V, x_dtype, batch);
     if (!prefill && !skinny && (generic_only || !tq::shape_supported(V.in_features, V.block_size))) {
         if (!tq::generic_supported(V)) { set_error("tq_linear_forward: unsupported layer shape"); return 1; }
         return hip_ok(tq::launch_gemv_generic(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream, gate),
@@ -401,7 +402,7 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
                       "tq_prefill launch") ? 0 : 1;
     }
     if (skinny) {
-        // 2..15 rows: batch rows on the matrix cores, fp16 weights and rotated activations.
+        // 2..32 rows: batch rows on the matrix cores, fp16 weights and rotated activations.
         return hip_ok(tq::launch_skinny(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, partial, device_cu_count(), stream),
                       "tq_skinny launch") ? 0 : 1;
     }
@@ -505,10 +506,10 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
             size_t work = 0, part = 0;
             for (int k = 0; k < 2; ++k) {
                 const tq::LayerView& P = h->plane_view[k];
-                const size_t small = tq::skinny_workspace_bytes(P, max_batch < 15 ? max_batch : 15);
+                const size_t small = tq::skinny_workspace_bytes(P, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows);
                 const size_t big = max_batch >= 16 ? tq::prefill_reserve_bytes(P, max_batch, device_cu_count()) : 0;
                 work = std::max(work, std::max(small, big));
-                part = std::max(part, tq::skinny_partial_bytes(P, max_batch < 15 ? max_batch : 15));
+                part = std::max(part, tq::skinny_partial_bytes(P, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows));
             }
             if (!ensure_stage(&h->d_work, &h->work_bytes, work, nullptr, &h->retired)) return 1;
             if (!ensure_stage(&h->d_partial, &h->partial_bytes, part, nullptr, &h->retired)) return 1;
@@ -516,10 +517,10 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
             return 0;
         }
         const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
-        const size_t small = tq::skinny_workspace_bytes(V, max_batch < 15 ? max_batch : 15);
+        const size_t small = tq::skinny_workspace_bytes(V, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows);
         const size_t big = max_batch >= 16 ? tq::prefill_reserve_bytes(V, max_batch, device_cu_count()) : 0;
         if (!ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big, nullptr, &h->retired)) return 1;
-        if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < 15 ? max_batch : 15), nullptr, &h->retired)) return 1;
+        if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows), nullptr, &h->retired)) return 1;
         return 0;
     } catch (...) { set_error("tq_linear_reserve: exception"); return 1; }
 }
@@ -565,7 +566,7 @@ int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int
             return hip_ok(tq::launch_gemv_wide_group(as, n, device_cu_count(), st), "tq_gemv group launch") ? 0 : 1;
         }
         if (plain && tq::skinny_group_supported(views, n, x_dtype, batch, device_cu_count())) {
-            // 2..15 rows on the matrix cores; the per-chunk partial products are per layer and allocated
+            // 2..32 rows on the matrix cores; the per-chunk partial products are per layer and allocated
             // on the first such call (not capturable in a graph), as in tq_linear_forward.
             float* partials[3] = {nullptr, nullptr, nullptr};
             for (int j = 0; j < n; ++j) {

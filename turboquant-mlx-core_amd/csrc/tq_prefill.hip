@@ -1,4 +1,4 @@
-// TQ8 prefill: dequantise-into-LDS + fp16 MFMA GEMM for gfx950 (batch >= 16, activations of any type).
+// TQ8 prefill: dequantise-into-LDS + fp16 MFMA GEMM for gfx950 (batch >= 16, or >= 33 where the small-batch kernels take the layer; activations of any type).
 //
 // The reference has no batched-GEMM path: batch is a grid dimension of its per-row-FWHT kernel
 // (src/dequantizer.cpp:545-549), so every weight block is inverse-transformed once per batch row.

@@ -1,4 +1,4 @@
-// TQ8 small-batch forward for gfx950: 2..15 activation rows (any activation type), shared-rotation
+// TQ8 small-batch forward for gfx950: 2..32 activation rows (any activation type), shared-rotation
 // layers (one byte per weight).
 //
 // The batch-1 kernel multiplies every decoded weight with the activation of each batch row on the
@@ -9,7 +9,8 @@
 //   Y[m, n] = norm[n] / sqrt(in) * sum_k X~[m, k] * L[n, k],   X~ = H (s (.) X) / sqrt(bs)
 //
 // K is cut into 512-column chunks.  A wave keeps the rotated activations of its chunk for all 16
-// (padded) batch rows in registers as MFMA A operands (64 VGPRs), walks 16-row groups of the weight
+// (padded) batch rows in registers as MFMA A operands (64 VGPRs; two such sets for 17..32 rows, which
+// multiply the same decoded weights), walks 16-row groups of the weight
 // plane, decodes 16 x 512 weights per group through the lane-private LDS table (entries rounded to
 // fp16, as in the prefill kernel) and writes the 16 x 16 fp32 partial product of the chunk.  A
 // second small kernel adds the chunks, applies the row norm and converts.
@@ -27,6 +28,7 @@ constexpr int kSkChunk = 512;            // columns per K chunk
 constexpr int kSkThreads = 512;          // 8 waves per workgroup, one workgroup per CU
 constexpr int kSkLutBytes = 256 * 256;
 constexpr int kSkStageBytes = 16 * kSkChunk * 2;   // 16 rows x 512 fp16 rotated activations
+constexpr int kSkMaxRows = kSkinnyMaxRows;   // two sets of 16 batch rows per decoded weight
 
 struct SkinnyArgs {
     const void* x;             // FUSED: activations [batch, K], f32, f16 or bf16
@@ -57,11 +59,13 @@ __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t l
 // columns: a block never leaves the chunk), instead of reading tile images a separate kernel wrote.
 // chunk, wg_in_chunk: the 512-column chunk of this workgroup and its index among the workgroups that
 // share the chunk for this layer (a launch may serve several layers).
-template <bool FUSED>
+// SETS: 1 (up to 16 batch rows) or 2 (17..32 rows: a second set of A operands multiplies the same decoded
+// weights, so the weights are still read and decoded once).
+template <bool FUSED, int SETS>
 __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk, const int wg_in_chunk) {
-    // table | 16 x 512 fp16 rotated activations (FUSED).  One workgroup of 8 waves per CU: 16 waves
+    // table | 16 SETS x 512 fp16 rotated activations (FUSED).  One workgroup of 8 waves per CU: 16 waves
     // gained nothing, and 8 have the registers for two row groups in flight.
-    __shared__ __align__(16) char smem[kSkLutBytes + kSkStageBytes];
+    __shared__ __align__(16) char smem[kSkLutBytes + SETS * kSkStageBytes];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -89,10 +93,10 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
     float tv[kSlots];
 #pragma unroll
     for (int k = 0; k < kSlots; ++k) tv[k] = a.tables[(tid + k * kSkThreads) >> 4];
-    TileRaw xin[2];
+    TileRaw xin[2 * SETS];
     if constexpr (FUSED) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {                      // batch rows w and w + 8 (row 0 again past the batch: not used)
+        for (int t = 0; t < 2 * SETS; ++t) {               // batch rows w, w + 8, .. (row 0 again past the batch: not used)
             const int b = wave + 8 * t;
             xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, chunk * kSkChunk + lane * 8);
         }
@@ -119,15 +123,15 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
         }
     }
 
-    sk_f16x8 afrag[16];
+    sk_f16x8 afrag[SETS][16];
     char* const stage = smem + kSkLutBytes;
     if constexpr (FUSED) {
-        // Wave w rotates batch rows w and w + 8 of the chunk (one 512-column tile each, 8 values per
+        // Wave w rotates batch rows w, w + 8, .. of the chunk (one 512-column tile each, 8 values per
         // lane; blocks of at most 512 columns: a block never leaves the chunk) and writes them, scaled by 1 / sqrt(bs), as fp16,
-        // [16 rows][512]; rows past the batch are zero.
+        // [16 SETS rows][512]; rows past the batch are zero.
         constexpr int kPitch = kSkChunk * 2;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 2 * SETS; ++t) {
             const int b = wave + 8 * t;
             const int col = chunk * kSkChunk + lane * 8;
             uint4 packed = make_uint4(0, 0, 0, 0);
@@ -145,19 +149,23 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
         // k-step s covers columns 64 (s/2) + 16 g + 8 (s%2) + [0, 8) of the chunk, the same columns
         // the B operand of that step decodes (any column order is fine as long as both agree).
 #pragma unroll
-        for (int s = 0; s < 16; ++s)
-            afrag[s] = *reinterpret_cast<const sk_f16x8*>(stage + m * kPitch + (64 * (s >> 1) + 16 * g + 8 * (s & 1)) * 2);
+        for (int e = 0; e < SETS; ++e)
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                afrag[e][s] = *reinterpret_cast<const sk_f16x8*>(stage + (m + 16 * e) * kPitch + (64 * (s >> 1) + 16 * g + 8 * (s & 1)) * 2);
     } else {
         // Tile images written by tq_rotate_f16_kernel: [K/32][256][32] fp16 with 16-byte slots
         // XOR-permuted per row; same column order as above.
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
-            const int off = 16 * g + 8 * (s & 1);              // column inside the 64-column piece
-            const int kt = chunk * 16 + 2 * (s >> 1) + (off >> 5);
-            const int slot = ((off & 31) >> 3) ^ ((m >> 2) & 3);
-            afrag[s] = *reinterpret_cast<const sk_f16x8*>(reinterpret_cast<const char*>(a.xt) +
-                                                           ((size_t)kt * 256 + m) * 64 + slot * 16);
-        }
+        for (int e = 0; e < SETS; ++e)
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                const int off = 16 * g + 8 * (s & 1);              // column inside the 64-column piece
+                const int kt = chunk * 16 + 2 * (s >> 1) + (off >> 5);
+                const int slot = ((off & 31) >> 3) ^ ((m >> 2) & 3);      // (rows m and m + 16: the same permutation)
+                afrag[e][s] = *reinterpret_cast<const sk_f16x8*>(reinterpret_cast<const char*>(a.xt) +
+                                                                  ((size_t)kt * 256 + m + 16 * e) * 64 + slot * 16);
+            }
         __syncthreads();                                    // table visible
     }
 
@@ -171,23 +179,30 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
     };
     // One row group: 16 x 512 weights of the chunk -> 16 x 16 partial product.
     auto multiply = [&](const sk_u32x4 (&raw)[8], int grp) {
-        sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        sk_f32x4 acc[SETS];
+#pragma unroll
+        for (int e = 0; e < SETS; ++e) acc[e] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             const sk_u32x4 w = raw[q];
             const uint2 p0 = lookup2(w.x), p1 = lookup2(w.y), p2 = lookup2(w.z), p3 = lookup2(w.w);
             const sk_u32x4 b0 = {p0.x, p0.y, p1.x, p1.y}, b1 = {p2.x, p2.y, p3.x, p3.y};
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[2 * q], __builtin_bit_cast(sk_f16x8, b0), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[2 * q + 1], __builtin_bit_cast(sk_f16x8, b1), acc, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < SETS; ++e) {
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][2 * q], __builtin_bit_cast(sk_f16x8, b0), acc[e], 0, 0, 0);
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][2 * q + 1], __builtin_bit_cast(sk_f16x8, b1), acc[e], 0, 0, 0);
+            }
         }
-        // D layout: lane holds weight row n = lane % 16 and batch rows 4 (lane / 16) + r.
+        // D layout: lane holds weight row n = lane % 16 and batch rows 16 e + 4 (lane / 16) + r.
         const int n = grp * 16 + m;
         if (n < a.N) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int b = 4 * g + r;
-                if (b < a.batch) a.partial[((size_t)chunk * a.batch + b) * a.N + n] = acc[r];
-            }
+            for (int e = 0; e < SETS; ++e)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int b = 16 * e + 4 * g + r;
+                    if (b < a.batch) a.partial[((size_t)chunk * a.batch + b) * a.N + n] = acc[e][r];
+                }
         }
     };
 
@@ -202,9 +217,9 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
 }
 
 // grid = chunks x workgroups per chunk
-template <bool FUSED>
+template <bool FUSED, int SETS>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_kernel(SkinnyArgs a) {
-    skinny_body<FUSED>(a, (int)blockIdx.x, (int)blockIdx.y);
+    skinny_body<FUSED, SETS>(a, (int)blockIdx.x, (int)blockIdx.y);
 }
 
 // Two or three layers of equal width on the same activation rows (q, k, v or gate, up), one launch:
@@ -214,10 +229,11 @@ struct SkinnyGroup {
     SkinnyArgs a[3];
     int first[4];
 };
+template <int SETS>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_group_kernel(SkinnyGroup g) {
     const int b = (int)blockIdx.y;
     const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
-    skinny_body<true>(g.a[j], (int)blockIdx.x, b - g.first[j]);
+    skinny_body<true, SETS>(g.a[j], (int)blockIdx.x, b - g.first[j]);
 }
 
 // Nibble planes (dual rotation, primary only): the same scheme on a plane of two weights per
@@ -243,11 +259,12 @@ struct SkinnyNibbleArgs {
 
 // unit, wg_in_unit: the (chunk, plane) unit of this workgroup and its index among the workgroups that
 // share the unit for this layer (a launch may serve several layers).
+template <int SETS>
 __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, const int unit, const int wg_in_unit) {
     // The table is indexed by a whole byte of the plane: an entry holds the fp16 centroids of both
     // its nibbles, i.e. one register of the B operand, so two weights cost one table read.
     constexpr int kTabBytes = kSkLutBytes;                 // 256 entries, one private column per lane
-    __shared__ __align__(16) char smem[kTabBytes + kSkStageBytes];   // table | 16 x 512 fp16 rotated activations
+    __shared__ __align__(16) char smem[kTabBytes + SETS * kSkStageBytes];   // table | 16 SETS x 512 fp16 rotated activations
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -277,9 +294,9 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
     float thi[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) thi[k] = a.tables[16 * pl + (tid >> 8) + 2 * k];
-    TileRaw xin[2];
+    TileRaw xin[2 * SETS];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {                          // batch rows w and w + 8 (row 0 again past the batch: not used)
+    for (int t = 0; t < 2 * SETS; ++t) {                   // batch rows w, w + 8, .. (row 0 again past the batch: not used)
         const int b = wave + 8 * t;
         xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, chunk * kSkChunk + lane * 8);
     }
@@ -300,11 +317,11 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
             reinterpret_cast<uint4*>(smem)[tid + k * kSkThreads] = make_uint4(v, v, v, v);
         }
     }
-    // Rotate batch rows w and w + 8 of the chunk with this plane's seed -> fp16 [16][512] in LDS.
+    // Rotate batch rows w, w + 8, .. of the chunk with this plane's seed -> fp16 [16 SETS][512] in LDS.
     constexpr int kPitch = kSkChunk * 2;
     char* const stage = smem + kTabBytes;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < 2 * SETS; ++t) {
         const int b = wave + 8 * t;
         const int col = chunk * kSkChunk + lane * 8;
         uint4 packed = make_uint4(0, 0, 0, 0);
@@ -322,10 +339,12 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
     // A operands.  Matrix step s = 4 q + d multiplies columns 128 q + 32 g + 8 d + [0, 8) of the chunk:
     // the 8 nibbles of dword d of the lane's 16-byte piece q (piece q of lane group g starts at byte
     // 64 q + 16 g of the row's 256 bytes).
-    sk_f16x8 afrag[16];
+    sk_f16x8 afrag[SETS][16];
 #pragma unroll
-    for (int s = 0; s < 16; ++s)
-        afrag[s] = *reinterpret_cast<const sk_f16x8*>(stage + m * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
+    for (int e = 0; e < SETS; ++e)
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+            afrag[e][s] = *reinterpret_cast<const sk_f16x8*>(stage + (m + 16 * e) * kPitch + (128 * (s >> 2) + 32 * g + 8 * (s & 3)) * 2);
 
     // One dword = 8 weights of 8 consecutive columns (low nibble first) -> one B operand: byte j of
     // the dword selects the register that holds columns 2 j and 2 j + 1.
@@ -337,22 +356,30 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
         return __builtin_bit_cast(sk_f16x8, r);
     };
     auto multiply = [&](const sk_u32x4 (&raw)[4], int grp) {
-        sk_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        sk_f32x4 acc[SETS];
+#pragma unroll
+        for (int e = 0; e < SETS; ++e) acc[e] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const sk_u32x4 w = raw[q];
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 0], operand(w.x), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 1], operand(w.y), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 2], operand(w.z), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[4 * q + 3], operand(w.w), acc, 0, 0, 0);
+            const sk_f16x8 b0 = operand(w.x), b1 = operand(w.y), b2 = operand(w.z), b3 = operand(w.w);
+#pragma unroll
+            for (int e = 0; e < SETS; ++e) {
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 0], b0, acc[e], 0, 0, 0);
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 1], b1, acc[e], 0, 0, 0);
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 2], b2, acc[e], 0, 0, 0);
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 3], b3, acc[e], 0, 0, 0);
+            }
         }
         const int n = grp * 16 + m;
         if (n < a.N) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int b = 4 * g + r;
-                if (b < a.batch) a.partial[((size_t)unit * a.batch + b) * a.N + n] = acc[r];
-            }
+            for (int e = 0; e < SETS; ++e)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int b = 16 * e + 4 * g + r;
+                    if (b < a.batch) a.partial[((size_t)unit * a.batch + b) * a.N + n] = acc[e][r];
+                }
         }
     };
     // The next group is requested before the current one is decoded (unrolled twice: static buffers).
@@ -366,8 +393,9 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
 }
 
 // grid = units x workgroups per unit
+template <int SETS>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
-    skinny_nibble_body(a, (int)blockIdx.x, (int)blockIdx.y);
+    skinny_nibble_body<SETS>(a, (int)blockIdx.x, (int)blockIdx.y);
 }
 
 // Layers of equal width and mode on the same activation rows, one launch (see SkinnyGroup).
@@ -375,10 +403,11 @@ struct SkinnyNibbleGroup {
     SkinnyNibbleArgs a[3];
     int first[4];
 };
+template <int SETS>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_group_kernel(SkinnyNibbleGroup g) {
     const int b = (int)blockIdx.y;
     const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
-    skinny_nibble_body(g.a[j], (int)blockIdx.x, b - g.first[j]);
+    skinny_nibble_body<SETS>(g.a[j], (int)blockIdx.x, b - g.first[j]);
 }
 
 // y[b, n] = norm[n] * out_scale * sum over chunks of partial[c][b][n]
@@ -440,7 +469,7 @@ static bool skinny_nibble(const LayerView& L) {
 }
 
 bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
-    if (batch < 2 || batch >= 16 || L.in_features % kSkChunk != 0) return false;   // (any activation type)
+    if (batch < 2 || batch > kSkMaxRows || L.in_features % kSkChunk != 0) return false;   // (any activation type)
     if (!lanes_supported(L.in_features, L.block_size)) return false;
     if (!L.fp16_centroids_ok) return false;                   // decoded weights are kept in fp16
     return (L.mode == kSharedLut && L.packed_combined) || skinny_nibble(L);
@@ -476,7 +505,8 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         const int workers_n = n.wgs_per_unit * (kSkThreads / 64);
         n.groups_q = n.groups / workers_n;
         n.groups_rem = n.groups % workers_n;
-        hipLaunchKernelGGL(tq_skinny_nibble_kernel, dim3(n.units, n.wgs_per_unit), dim3(kSkThreads), 0, stream, n);
+        if (batch > 16) hipLaunchKernelGGL(tq_skinny_nibble_kernel<2>, dim3(n.units, n.wgs_per_unit), dim3(kSkThreads), 0, stream, n);
+        else hipLaunchKernelGGL(tq_skinny_nibble_kernel<1>, dim3(n.units, n.wgs_per_unit), dim3(kSkThreads), 0, stream, n);
         hipError_t en = hipGetLastError();
         if (en != hipSuccess) return en;
         const unsigned blocks_n = (unsigned)((L.out_features + 63) / 64);
@@ -503,8 +533,11 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     const int workers = a.wgs_per_chunk * (kSkThreads / 64);
     a.groups_q = a.groups / workers;
     a.groups_rem = a.groups % workers;
-    if (fused) hipLaunchKernelGGL(tq_skinny_kernel<true>, dim3(a.chunks, a.wgs_per_chunk), dim3(kSkThreads), 0, stream, a);
-    else hipLaunchKernelGGL(tq_skinny_kernel<false>, dim3(a.chunks, a.wgs_per_chunk), dim3(kSkThreads), 0, stream, a);
+    const dim3 grid(a.chunks, a.wgs_per_chunk);
+    if (fused && batch > 16) hipLaunchKernelGGL((tq_skinny_kernel<true, 2>), grid, dim3(kSkThreads), 0, stream, a);
+    else if (fused) hipLaunchKernelGGL((tq_skinny_kernel<true, 1>), grid, dim3(kSkThreads), 0, stream, a);
+    else if (batch > 16) hipLaunchKernelGGL((tq_skinny_kernel<false, 2>), grid, dim3(kSkThreads), 0, stream, a);
+    else hipLaunchKernelGGL((tq_skinny_kernel<false, 1>), grid, dim3(kSkThreads), 0, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     const unsigned blocks = (unsigned)((L.out_features + 63) / 64);
@@ -514,7 +547,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
 }
 
 // Layers that can share the two launches: two or three layers of equal width and mode with blocks
-// of at most 512 columns (the workgroup rotates its chunk itself), 2..15 rows,
+// of at most 512 columns (the workgroup rotates its chunk itself), 2..32 rows,
 // and at least one workgroup per work unit and layer.
 bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, int num_cus) {
     if (n < 2 || n > 3) return false;
@@ -591,8 +624,11 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
     int reduce_blocks = 0;
     for (int j = 0; j < n; ++j) reduce_blocks += (Ls[j].out_features + 63) / 64;
     r.y_dtype = y_dtype; r.chunks = chunks;
-    if (nibble) hipLaunchKernelGGL(tq_skinny_nibble_group_kernel, dim3(chunks, used), dim3(kSkThreads), 0, stream, gn);
-    else hipLaunchKernelGGL(tq_skinny_group_kernel, dim3(chunks, used), dim3(kSkThreads), 0, stream, g);
+    const dim3 grid(chunks, used);
+    if (nibble && batch > 16) hipLaunchKernelGGL(tq_skinny_nibble_group_kernel<2>, grid, dim3(kSkThreads), 0, stream, gn);
+    else if (nibble) hipLaunchKernelGGL(tq_skinny_nibble_group_kernel<1>, grid, dim3(kSkThreads), 0, stream, gn);
+    else if (batch > 16) hipLaunchKernelGGL(tq_skinny_group_kernel<2>, grid, dim3(kSkThreads), 0, stream, g);
+    else hipLaunchKernelGGL(tq_skinny_group_kernel<1>, grid, dim3(kSkThreads), 0, stream, g);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(tq_skinny_reduce_group_kernel, dim3(reduce_blocks, batch), dim3(256), 0, stream, r);
