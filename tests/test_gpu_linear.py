@@ -323,9 +323,13 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
                                               (1000, 5120, 512, 8), (16, 512, 64, 3), (47, 1536, 128, 9),
                                               # 17..32 rows: a second set of 16 batch rows on the same decoded weights
                                               (513, 2048, 512, 16), (300, 1024, 256, 17), (1000, 5120, 512, 32),
-                                              (64, 512, 512, 25), (257, 2048, 1024, 31), (90, 1536, 512, 20)])
+                                              (64, 512, 512, 25), (257, 2048, 1024, 31), (90, 1536, 512, 20),
+                                              # widths that do not fill their last 512-column chunk (5.5, 2.625, 0.875,
+                                              # 21.5, 1.75 and 0.375 chunks), the last two with two sets of rows
+                                              (130, 2816, 256, 5), (77, 1344, 64, 3), (64, 448, 64, 9),
+                                              (200, 11008, 256, 4), (90, 896, 128, 20), (33, 192, 64, 31)])
 def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, inf, bs, batch):
-    """2..32 rows on a layer whose width is a multiple of 512 take the
+    """2..32 rows on a layer whose width is a multiple of 64 (nibble planes: of 128) take the
     small-batch MFMA kernels (fp16 weights and rotated activations, fp32 accumulation over
     512-column chunks; for dual rotation one pass per plane, each with its own rotation):
     1e-3 relative L2 (5e-3 with a bf16 output), ragged row counts, every row equal to its batch-1 result."""

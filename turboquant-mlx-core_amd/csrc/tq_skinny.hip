@@ -85,6 +85,13 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
         if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
         return a.plane + (size_t)row * a.K + col0;
     };
+    // A last chunk that the row does not fill (K a multiple of 64, not of 512; blocks of at most 256 columns):
+    // its 64-column pieces past the row are read from piece 0 again (valid memory, any byte decodes to a
+    // finite centroid) and multiply rotated activations that are zero.  Wave-uniform.
+    const int pieces = a.K - chunk * kSkChunk >= kSkChunk ? 8 : (a.K - chunk * kSkChunk) >> 6;
+    int piece_off[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) piece_off[q] = q < pieces ? 64 * q : 0;
 
     // Everything that has to come from memory is requested up front, the small things first (loads
     // complete in order): table values, the activations this wave rotates, then the first row group,
@@ -98,7 +105,8 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
 #pragma unroll
         for (int t = 0; t < 2 * SETS; ++t) {               // batch rows w, w + 8, .. (row 0 again past the batch: not used)
             const int b = wave + 8 * t;
-            xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, chunk * kSkChunk + lane * 8);
+            const int col = chunk * kSkChunk + lane * 8;     // (columns past the row: read column 0, rotated as zeros)
+            xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, col < a.K ? col : 0);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -109,7 +117,7 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
     auto request = [&](sk_u32x4 (&raw)[8], int grp) {
         const uint8_t* p = row_ptr(grp);
 #pragma unroll
-        for (int q = 0; q < 8; ++q) raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+        for (int q = 0; q < 8; ++q) raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + piece_off[q]));
     };
     if (g_begin < g_end) request(rawA, g_begin);
 
@@ -137,7 +145,7 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
             uint4 packed = make_uint4(0, 0, 0, 0);
             if (b < a.batch) {                              // wave-uniform
                 float v[8];
-                rotate_tile(xin[t], a.x_dtype, col, true, a.seed, a.block_size, lane, v);
+                rotate_tile(xin[t], a.x_dtype, col, col < a.K, a.seed, a.block_size, lane, v);
                 packed.x = (uint32_t)float_to_f16_bits(v[0] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[1] * a.x_scale) << 16);
                 packed.y = (uint32_t)float_to_f16_bits(v[2] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[3] * a.x_scale) << 16);
                 packed.z = (uint32_t)float_to_f16_bits(v[4] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[5] * a.x_scale) << 16);
@@ -285,6 +293,12 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
         if (row >= a.N) row = a.N - 1;                     // rows past N re-read row N-1: never stored
         return plane + (size_t)row * row_bytes + byte0;
     };
+    // A last chunk that the row does not fill (K a multiple of 128, not of 512): its 128-column pieces past
+    // the row are read from piece 0 again and multiply rotated activations that are zero.  Wave-uniform.
+    const int pieces = a.K - chunk * kSkChunk >= kSkChunk ? 4 : (a.K - chunk * kSkChunk) >> 7;
+    int piece_off[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) piece_off[q] = q < pieces ? 64 * q : 0;
 
     // Small loads first (they complete in order), then the first row group, which travels while the
     // activations are rotated.
@@ -298,14 +312,15 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
 #pragma unroll
     for (int t = 0; t < 2 * SETS; ++t) {                   // batch rows w, w + 8, .. (row 0 again past the batch: not used)
         const int b = wave + 8 * t;
-        xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, chunk * kSkChunk + lane * 8);
+        const int col = chunk * kSkChunk + lane * 8;         // (columns past the row: read column 0, rotated as zeros)
+        xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, col < a.K ? col : 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     sk_u32x4 rawA[4], rawB[4];                             // two row groups: one decoded, one in flight
     auto request = [&](sk_u32x4 (&raw)[4], int grp) {
         const uint8_t* p = row_ptr(grp);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + 64 * q));
+        for (int q = 0; q < 4; ++q) raw[q] = (*reinterpret_cast<const sk_u32x4*>(p + piece_off[q]));
     };
     if (g_begin < g_end) request(rawA, g_begin);
 
@@ -327,7 +342,7 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
         uint4 packed = make_uint4(0, 0, 0, 0);
         if (b < a.batch) {                                  // wave-uniform
             float v[8];
-            rotate_tile(xin[t], a.x_dtype, col, true, a.seed[pl], a.block_size, lane, v);
+            rotate_tile(xin[t], a.x_dtype, col, col < a.K, a.seed[pl], a.block_size, lane, v);
             packed.x = (uint32_t)float_to_f16_bits(v[0] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[1] * a.x_scale) << 16);
             packed.y = (uint32_t)float_to_f16_bits(v[2] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[3] * a.x_scale) << 16);
             packed.z = (uint32_t)float_to_f16_bits(v[4] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[5] * a.x_scale) << 16);
@@ -469,14 +484,17 @@ static bool skinny_nibble(const LayerView& L) {
 }
 
 bool skinny_supported(const LayerView& L, int x_dtype, int batch) {
-    if (batch < 2 || batch > kSkMaxRows || L.in_features % kSkChunk != 0) return false;   // (any activation type)
+    if (batch < 2 || batch > kSkMaxRows) return false;                                   // (any activation type)
+    // whole 64-column pieces (nibble planes: 128-column pieces); a row that does not fill its last 512-column
+    // chunk has blocks of at most 256 columns, which the workgroup rotates itself
+    if (L.in_features % ((L.mode == kSharedLut) ? 64 : 128) != 0) return false;
     if (!lanes_supported(L.in_features, L.block_size)) return false;
     if (!L.fp16_centroids_ok) return false;                   // decoded weights are kept in fp16
     return (L.mode == kSharedLut && L.packed_combined) || skinny_nibble(L);
 }
 
 size_t skinny_partial_bytes(const LayerView& L, int batch) {
-    const size_t units = (size_t)(L.in_features / kSkChunk) * (L.mode == kDual ? 2 : 1);
+    const size_t units = (size_t)((L.in_features + kSkChunk - 1) / kSkChunk) * (L.mode == kDual ? 2 : 1);
     return units * (size_t)batch * L.out_features * sizeof(float);
 }
 
@@ -499,7 +517,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         n.partial = partial;
         n.batch = batch; n.N = L.out_features; n.K = L.in_features;
         n.planes = L.mode == kDual ? 2 : 1;
-        n.units = L.in_features / kSkChunk * n.planes;
+        n.units = (L.in_features + kSkChunk - 1) / kSkChunk * n.planes;
         n.groups = (L.out_features + 15) / 16;
         n.wgs_per_unit = num_cus / n.units > 0 ? num_cus / n.units : 1;   // one workgroup per CU
         const int workers_n = n.wgs_per_unit * (kSkThreads / 64);
@@ -527,7 +545,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     a.tables = L.tables;
     a.partial = partial;
     a.batch = batch; a.N = L.out_features; a.K = L.in_features;
-    a.chunks = L.in_features / kSkChunk;
+    a.chunks = (L.in_features + kSkChunk - 1) / kSkChunk;
     a.groups = (L.out_features + 15) / 16;
     a.wgs_per_chunk = num_cus / a.chunks > 0 ? num_cus / a.chunks : 1;   // one workgroup per CU
     const int workers = a.wgs_per_chunk * (kSkThreads / 64);
@@ -557,7 +575,7 @@ bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, 
         if (!nibble && (Ls[j].mode != kSharedLut || !Ls[j].packed_combined)) return false;
         if (Ls[j].in_features != Ls[0].in_features || !skinny_supported(Ls[j], x_dtype, batch)) return false;
     }
-    const int units = Ls[0].in_features / kSkChunk * (Ls[0].mode == kDual ? 2 : 1);
+    const int units = (Ls[0].in_features + kSkChunk - 1) / kSkChunk * (Ls[0].mode == kDual ? 2 : 1);
     return num_cus / units >= n;
 }
 
@@ -565,7 +583,7 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
                                int y_dtype, float* const* partials, int num_cus, hipStream_t stream) {
     const bool nibble = Ls[0].mode == kDual || Ls[0].mode == kPrimaryOnly;
     const int planes = Ls[0].mode == kDual ? 2 : 1;
-    const int K = Ls[0].in_features, chunks = K / kSkChunk * planes;   // work units: (chunk, plane)
+    const int K = Ls[0].in_features, chunks = (K + kSkChunk - 1) / kSkChunk * planes;   // work units: (chunk, plane)
     const int total_wgs = num_cus / chunks;                       // workgroups per unit, all layers together
     long long rows = 0;
     for (int j = 0; j < n; ++j) rows += Ls[j].out_features;
