@@ -495,7 +495,7 @@ def main():
                     L.tq_linear_free(h)
             torch.cuda.empty_cache()
 
-    # ---- decoder-layer projections, Qwen2.5-32B shape, batch 1 / 4 / 8, bf16 activations ----
+    # ---- decoder-layer projections, Qwen2.5-32B shape, batch 1 / 4 / 8 (grouped launches: and 32), bf16 activations ----
     L = tq.lib()
     shapes = [("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120, 5120),
               ("gate", 27648, 5120), ("up", 27648, 5120), ("down", 5120, 27648)]
@@ -529,7 +529,7 @@ def main():
     L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
                                           C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
     def grouped(sets, tag):
-        for batch in (1, 4, 8):
+        for batch in (1, 4, 8, 32):
             xg = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
             yg = {n_: torch.empty(batch, out_of[n_], device="cuda", dtype=torch.float32) for n_ in sets[0]}
             turn = [0]

@@ -61,8 +61,11 @@ __device__ __forceinline__ uint32_t sk_entry_addr(uint32_t idx_bytes, uint32_t l
 // share the chunk for this layer (a launch may serve several layers).
 // SETS: 1 (up to 16 batch rows) or 2 (17..32 rows: a second set of A operands multiplies the same decoded
 // weights, so the weights are still read and decoded once).
-template <bool FUSED, int SETS>
+// RAGGED: the row does not fill its last 512-column chunk (a kernel of its own, so that the loads of whole
+// chunks keep their constant offsets and the compiler its exact wait counts).
+template <bool FUSED, int SETS, bool RAGGED>
 __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk, const int wg_in_chunk) {
+    static_assert(FUSED || !RAGGED, "blocks wider than a chunk divide the row into whole chunks");
     // table | 16 SETS x 512 fp16 rotated activations (FUSED).  One workgroup of 8 waves per CU: 16 waves
     // gained nothing, and 8 have the registers for two row groups in flight.
     __shared__ __align__(16) char smem[kSkLutBytes + SETS * kSkStageBytes];
@@ -88,10 +91,10 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
     // A last chunk that the row does not fill (K a multiple of 64, not of 512; blocks of at most 256 columns):
     // its 64-column pieces past the row are read from piece 0 again (valid memory, any byte decodes to a
     // finite centroid) and multiply rotated activations that are zero.  Wave-uniform.
-    const int pieces = a.K - chunk * kSkChunk >= kSkChunk ? 8 : (a.K - chunk * kSkChunk) >> 6;
+    const int pieces = (!RAGGED || a.K - chunk * kSkChunk >= kSkChunk) ? 8 : (a.K - chunk * kSkChunk) >> 6;
     int piece_off[8];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) piece_off[q] = q < pieces ? 64 * q : 0;
+    for (int q = 0; q < 8; ++q) piece_off[q] = (!RAGGED || q < pieces) ? 64 * q : 0;
 
     // Everything that has to come from memory is requested up front, the small things first (loads
     // complete in order): table values, the activations this wave rotates, then the first row group,
@@ -106,7 +109,7 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
         for (int t = 0; t < 2 * SETS; ++t) {               // batch rows w, w + 8, .. (row 0 again past the batch: not used)
             const int b = wave + 8 * t;
             const int col = chunk * kSkChunk + lane * 8;     // (columns past the row: read column 0, rotated as zeros)
-            xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, col < a.K ? col : 0);
+            xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, (!RAGGED || col < a.K) ? col : 0);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -145,7 +148,7 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
             uint4 packed = make_uint4(0, 0, 0, 0);
             if (b < a.batch) {                              // wave-uniform
                 float v[8];
-                rotate_tile(xin[t], a.x_dtype, col, col < a.K, a.seed, a.block_size, lane, v);
+                rotate_tile(xin[t], a.x_dtype, col, !RAGGED || col < a.K, a.seed, a.block_size, lane, v);
                 packed.x = (uint32_t)float_to_f16_bits(v[0] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[1] * a.x_scale) << 16);
                 packed.y = (uint32_t)float_to_f16_bits(v[2] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[3] * a.x_scale) << 16);
                 packed.z = (uint32_t)float_to_f16_bits(v[4] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[5] * a.x_scale) << 16);
@@ -225,9 +228,9 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, const int chunk
 }
 
 // grid = chunks x workgroups per chunk
-template <bool FUSED, int SETS>
+template <bool FUSED, int SETS, bool RAGGED>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_kernel(SkinnyArgs a) {
-    skinny_body<FUSED, SETS>(a, (int)blockIdx.x, (int)blockIdx.y);
+    skinny_body<FUSED, SETS, RAGGED>(a, (int)blockIdx.x, (int)blockIdx.y);
 }
 
 // Two or three layers of equal width on the same activation rows (q, k, v or gate, up), one launch:
@@ -237,11 +240,11 @@ struct SkinnyGroup {
     SkinnyArgs a[3];
     int first[4];
 };
-template <int SETS>
+template <int SETS, bool RAGGED>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_group_kernel(SkinnyGroup g) {
     const int b = (int)blockIdx.y;
     const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
-    skinny_body<true, SETS>(g.a[j], (int)blockIdx.x, b - g.first[j]);
+    skinny_body<true, SETS, RAGGED>(g.a[j], (int)blockIdx.x, b - g.first[j]);
 }
 
 // Nibble planes (dual rotation, primary only): the same scheme on a plane of two weights per
@@ -267,7 +270,7 @@ struct SkinnyNibbleArgs {
 
 // unit, wg_in_unit: the (chunk, plane) unit of this workgroup and its index among the workgroups that
 // share the unit for this layer (a launch may serve several layers).
-template <int SETS>
+template <int SETS, bool RAGGED>
 __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, const int unit, const int wg_in_unit) {
     // The table is indexed by a whole byte of the plane: an entry holds the fp16 centroids of both
     // its nibbles, i.e. one register of the B operand, so two weights cost one table read.
@@ -295,10 +298,10 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
     };
     // A last chunk that the row does not fill (K a multiple of 128, not of 512): its 128-column pieces past
     // the row are read from piece 0 again and multiply rotated activations that are zero.  Wave-uniform.
-    const int pieces = a.K - chunk * kSkChunk >= kSkChunk ? 4 : (a.K - chunk * kSkChunk) >> 7;
+    const int pieces = (!RAGGED || a.K - chunk * kSkChunk >= kSkChunk) ? 4 : (a.K - chunk * kSkChunk) >> 7;
     int piece_off[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) piece_off[q] = q < pieces ? 64 * q : 0;
+    for (int q = 0; q < 4; ++q) piece_off[q] = (!RAGGED || q < pieces) ? 64 * q : 0;
 
     // Small loads first (they complete in order), then the first row group, which travels while the
     // activations are rotated.
@@ -313,7 +316,7 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
     for (int t = 0; t < 2 * SETS; ++t) {                   // batch rows w, w + 8, .. (row 0 again past the batch: not used)
         const int b = wave + 8 * t;
         const int col = chunk * kSkChunk + lane * 8;         // (columns past the row: read column 0, rotated as zeros)
-        xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, col < a.K ? col : 0);
+        xin[t] = load_tile_raw(a.x, a.x_dtype, (size_t)(b < a.batch ? b : 0) * a.K, (!RAGGED || col < a.K) ? col : 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     sk_u32x4 rawA[4], rawB[4];                             // two row groups: one decoded, one in flight
@@ -342,7 +345,7 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
         uint4 packed = make_uint4(0, 0, 0, 0);
         if (b < a.batch) {                                  // wave-uniform
             float v[8];
-            rotate_tile(xin[t], a.x_dtype, col, col < a.K, a.seed[pl], a.block_size, lane, v);
+            rotate_tile(xin[t], a.x_dtype, col, !RAGGED || col < a.K, a.seed[pl], a.block_size, lane, v);
             packed.x = (uint32_t)float_to_f16_bits(v[0] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[1] * a.x_scale) << 16);
             packed.y = (uint32_t)float_to_f16_bits(v[2] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[3] * a.x_scale) << 16);
             packed.z = (uint32_t)float_to_f16_bits(v[4] * a.x_scale) | ((uint32_t)float_to_f16_bits(v[5] * a.x_scale) << 16);
@@ -377,13 +380,13 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const sk_u32x4 w = raw[q];
-            const sk_f16x8 b0 = operand(w.x), b1 = operand(w.y), b2 = operand(w.z), b3 = operand(w.w);
+            const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-            for (int e = 0; e < SETS; ++e) {
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 0], b0, acc[e], 0, 0, 0);
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 1], b1, acc[e], 0, 0, 0);
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 2], b2, acc[e], 0, 0, 0);
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + 3], b3, acc[e], 0, 0, 0);
+            for (int d = 0; d < 4; ++d) {                   // one operand, then the matrix instructions that use it
+                const sk_f16x8 b = operand(wd[d]);
+#pragma unroll
+                for (int e = 0; e < SETS; ++e)
+                    acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[e][4 * q + d], b, acc[e], 0, 0, 0);
             }
         }
         const int n = grp * 16 + m;
@@ -408,9 +411,9 @@ __device__ __forceinline__ void skinny_nibble_body(const SkinnyNibbleArgs& a, co
 }
 
 // grid = units x workgroups per unit
-template <int SETS>
+template <int SETS, bool RAGGED>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_kernel(SkinnyNibbleArgs a) {
-    skinny_nibble_body<SETS>(a, (int)blockIdx.x, (int)blockIdx.y);
+    skinny_nibble_body<SETS, RAGGED>(a, (int)blockIdx.x, (int)blockIdx.y);
 }
 
 // Layers of equal width and mode on the same activation rows, one launch (see SkinnyGroup).
@@ -418,11 +421,11 @@ struct SkinnyNibbleGroup {
     SkinnyNibbleArgs a[3];
     int first[4];
 };
-template <int SETS>
+template <int SETS, bool RAGGED>
 __global__ __launch_bounds__(kSkThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tq_skinny_nibble_group_kernel(SkinnyNibbleGroup g) {
     const int b = (int)blockIdx.y;
     const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
-    skinny_nibble_body<SETS>(g.a[j], (int)blockIdx.x, b - g.first[j]);
+    skinny_nibble_body<SETS, RAGGED>(g.a[j], (int)blockIdx.x, b - g.first[j]);
 }
 
 // y[b, n] = norm[n] * out_scale * sum over chunks of partial[c][b][n]
@@ -523,8 +526,12 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
         const int workers_n = n.wgs_per_unit * (kSkThreads / 64);
         n.groups_q = n.groups / workers_n;
         n.groups_rem = n.groups % workers_n;
-        if (batch > 16) hipLaunchKernelGGL(tq_skinny_nibble_kernel<2>, dim3(n.units, n.wgs_per_unit), dim3(kSkThreads), 0, stream, n);
-        else hipLaunchKernelGGL(tq_skinny_nibble_kernel<1>, dim3(n.units, n.wgs_per_unit), dim3(kSkThreads), 0, stream, n);
+        const dim3 grid_n(n.units, n.wgs_per_unit);
+        const bool two = batch > 16, ragged = L.in_features % kSkChunk != 0;
+        if (two && ragged) hipLaunchKernelGGL((tq_skinny_nibble_kernel<2, true>), grid_n, dim3(kSkThreads), 0, stream, n);
+        else if (two) hipLaunchKernelGGL((tq_skinny_nibble_kernel<2, false>), grid_n, dim3(kSkThreads), 0, stream, n);
+        else if (ragged) hipLaunchKernelGGL((tq_skinny_nibble_kernel<1, true>), grid_n, dim3(kSkThreads), 0, stream, n);
+        else hipLaunchKernelGGL((tq_skinny_nibble_kernel<1, false>), grid_n, dim3(kSkThreads), 0, stream, n);
         hipError_t en = hipGetLastError();
         if (en != hipSuccess) return en;
         const unsigned blocks_n = (unsigned)((L.out_features + 63) / 64);
@@ -552,10 +559,13 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
     a.groups_q = a.groups / workers;
     a.groups_rem = a.groups % workers;
     const dim3 grid(a.chunks, a.wgs_per_chunk);
-    if (fused && batch > 16) hipLaunchKernelGGL((tq_skinny_kernel<true, 2>), grid, dim3(kSkThreads), 0, stream, a);
-    else if (fused) hipLaunchKernelGGL((tq_skinny_kernel<true, 1>), grid, dim3(kSkThreads), 0, stream, a);
-    else if (batch > 16) hipLaunchKernelGGL((tq_skinny_kernel<false, 2>), grid, dim3(kSkThreads), 0, stream, a);
-    else hipLaunchKernelGGL((tq_skinny_kernel<false, 1>), grid, dim3(kSkThreads), 0, stream, a);
+    const bool two = batch > 16, ragged = L.in_features % kSkChunk != 0;     // (ragged rows have blocks <= 256: fused)
+    if (fused && ragged && two) hipLaunchKernelGGL((tq_skinny_kernel<true, 2, true>), grid, dim3(kSkThreads), 0, stream, a);
+    else if (fused && ragged) hipLaunchKernelGGL((tq_skinny_kernel<true, 1, true>), grid, dim3(kSkThreads), 0, stream, a);
+    else if (fused && two) hipLaunchKernelGGL((tq_skinny_kernel<true, 2, false>), grid, dim3(kSkThreads), 0, stream, a);
+    else if (fused) hipLaunchKernelGGL((tq_skinny_kernel<true, 1, false>), grid, dim3(kSkThreads), 0, stream, a);
+    else if (two) hipLaunchKernelGGL((tq_skinny_kernel<false, 2, false>), grid, dim3(kSkThreads), 0, stream, a);
+    else hipLaunchKernelGGL((tq_skinny_kernel<false, 1, false>), grid, dim3(kSkThreads), 0, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     const unsigned blocks = (unsigned)((L.out_features + 63) / 64);
@@ -643,10 +653,18 @@ hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_
     for (int j = 0; j < n; ++j) reduce_blocks += (Ls[j].out_features + 63) / 64;
     r.y_dtype = y_dtype; r.chunks = chunks;
     const dim3 grid(chunks, used);
-    if (nibble && batch > 16) hipLaunchKernelGGL(tq_skinny_nibble_group_kernel<2>, grid, dim3(kSkThreads), 0, stream, gn);
-    else if (nibble) hipLaunchKernelGGL(tq_skinny_nibble_group_kernel<1>, grid, dim3(kSkThreads), 0, stream, gn);
-    else if (batch > 16) hipLaunchKernelGGL(tq_skinny_group_kernel<2>, grid, dim3(kSkThreads), 0, stream, g);
-    else hipLaunchKernelGGL(tq_skinny_group_kernel<1>, grid, dim3(kSkThreads), 0, stream, g);
+    const bool two = batch > 16, ragged = K % kSkChunk != 0;
+    if (nibble) {
+        if (two && ragged) hipLaunchKernelGGL((tq_skinny_nibble_group_kernel<2, true>), grid, dim3(kSkThreads), 0, stream, gn);
+        else if (two) hipLaunchKernelGGL((tq_skinny_nibble_group_kernel<2, false>), grid, dim3(kSkThreads), 0, stream, gn);
+        else if (ragged) hipLaunchKernelGGL((tq_skinny_nibble_group_kernel<1, true>), grid, dim3(kSkThreads), 0, stream, gn);
+        else hipLaunchKernelGGL((tq_skinny_nibble_group_kernel<1, false>), grid, dim3(kSkThreads), 0, stream, gn);
+    } else {
+        if (two && ragged) hipLaunchKernelGGL((tq_skinny_group_kernel<2, true>), grid, dim3(kSkThreads), 0, stream, g);
+        else if (two) hipLaunchKernelGGL((tq_skinny_group_kernel<2, false>), grid, dim3(kSkThreads), 0, stream, g);
+        else if (ragged) hipLaunchKernelGGL((tq_skinny_group_kernel<1, true>), grid, dim3(kSkThreads), 0, stream, g);
+        else hipLaunchKernelGGL((tq_skinny_group_kernel<1, false>), grid, dim3(kSkThreads), 0, stream, g);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(tq_skinny_reduce_group_kernel, dim3(reduce_blocks, batch), dim3(256), 0, stream, r);
