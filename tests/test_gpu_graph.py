@@ -118,7 +118,7 @@ def _bits(o, rng, batch, inf):
     return o.f32_to_bf16_bits(rng.standard_normal((batch, inf)).astype(np.float32))
 
 
-BATCHES = (1, 4, 15, 40)          # batch-1 kernel, small-batch kernels (two sizes), prefill kernel
+BATCHES = (1, 4, 15, 24, 40)      # batch-1 kernel, small-batch kernels (one and two sets of rows), prefill kernel
 
 
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only", "dual_5bit"])
