@@ -249,6 +249,12 @@ def main():
     ap.add_argument("--timeline", action="store_true",
                     help="instead of the benchmark: per-wave wall-clock marks inside the batch-1 kernel (the "
                          "timeline build of the library), last of 300 back-to-back launches, as a text table")
+    ap.add_argument("--prefill-ablations", metavar="MASK", default=None,
+                    help="instead of the benchmark: eight 512-token calls of the prefill workload (27648 x 5120) on "
+                         "the build of the library with parts of the prefill panel kernel's loop compiled out "
+                         "(`make ablations`; MASK as in csrc/tq_prefill_panel.hip, 0 = the product library).  Meant to "
+                         "run under rocprofv3 --pmc: the results are wrong by construction, the cycle counters of "
+                         "the kernel are what is compared")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy three times (reference reading for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -268,6 +274,19 @@ def main():
     torch.cuda.set_device(0)
     if args.timeline:
         timeline(tq, torch)
+        return
+    if args.prefill_ablations is not None:
+        mask = int(args.prefill_ablations)
+        if mask:
+            tq.LIB_PATH = os.path.join(os.path.dirname(tq.LIB_PATH), "ablate", f"libturboquant_amd_ablate{mask}.so")
+        hp, _ = make_layer(tq, torch, 27648, 5120, 512, seed=500, sigma=0.01, shared=True)
+        xp = torch.randn(512, 5120, device="cuda").to(torch.bfloat16)
+        yp = torch.empty(512, 27648, device="cuda", dtype=torch.bfloat16)
+        for _ in range(8):
+            if tq.lib().tq_linear_forward(hp, xp.data_ptr(), tq.BF16, 512, yp.data_ptr(), tq.BF16, None) != 0:
+                raise RuntimeError(tq.last_error())
+        torch.cuda.synchronize()
+        print(f"prefill ablation mask {mask}: 8 calls of 27648 x 5120 at 512 tokens done ({tq.LIB_PATH})")
         return
 
     # ---- headline: lm_head 151936 x 2048, bf16 x, fp32 y, batch 1 -------------------
@@ -346,25 +365,29 @@ def main():
     # ---- what this machine sustains: streaming read and MFMA loops (roofline denominators) ----
     extra = {}
     import ctypes as C
-    Lp = tq.lib()
-    Lp.tq_probe_hbm_read.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
-    Lp.tq_probe_mfma_bf16.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
-    val = C.c_double()
+    probe_path = os.path.join(os.path.dirname(tq.LIB_PATH), "libtq_probe.so")      # `make probe`: a library of its own
     probes = {}
-    if Lp.tq_probe_hbm_read(1 << 30, 10, C.byref(val)) == 0:
-        probes["hbm_stream_read_gbs"] = val.value
-    for name, rnd in (("mfma_bf16_tflops_ones", 0), ("mfma_bf16_tflops_random_operands", 1)):
-        if Lp.tq_probe_mfma_bf16(rnd, 20000, C.byref(val)) == 0:
-            probes[name] = val.value
-    # (the prefill kernel multiplies in fp16: same nominal rate, more toggling mantissa bits)
-    Lp.tq_probe_mfma_f16.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
-    for name, rnd in (("mfma_f16_tflops_ones", 0), ("mfma_f16_tflops_random_operands", 1)):
-        if Lp.tq_probe_mfma_f16(rnd, 20000, C.byref(val)) == 0:
-            probes[name] = val.value
-    Lp.tq_probe_device_atomics.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
-    for name, addresses in (("device_scope_fetch_adds_per_us_one_word", 1), ("device_scope_fetch_adds_per_us_eight_words", 8)):
-        if Lp.tq_probe_device_atomics(addresses, 20, C.byref(val)) == 0:
-            probes[name] = val.value
+    if os.path.exists(probe_path):
+        Lp = C.CDLL(probe_path)
+        Lp.tq_probe_hbm_read.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
+        Lp.tq_probe_mfma_bf16.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+        Lp.tq_probe_mfma_f16.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+        Lp.tq_probe_empty_launch.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
+        val = C.c_double()
+        if Lp.tq_probe_hbm_read(1 << 30, 10, C.byref(val)) == 0:
+            probes["hbm_stream_read_gbs"] = val.value
+        for name, rnd in (("mfma_bf16_tflops_ones", 0), ("mfma_bf16_tflops_random_operands", 1)):
+            if Lp.tq_probe_mfma_bf16(rnd, 20000, C.byref(val)) == 0:
+                probes[name] = val.value
+        # (the prefill kernels multiply in fp16: same nominal rate, more toggling mantissa bits)
+        for name, rnd in (("mfma_f16_tflops_ones", 0), ("mfma_f16_tflops_random_operands", 1)):
+            if Lp.tq_probe_mfma_f16(rnd, 20000, C.byref(val)) == 0:
+                probes[name] = val.value
+        # launch to launch of a kernel that does nothing, as nodes of one HIP graph: a single wave, and the grid of
+        # the batch-1 kernel (one workgroup of 16 waves per CU)
+        for name, wgs, threads in (("empty_kernel_us_per_graph_node_1x64", 1, 64), ("empty_kernel_us_per_graph_node_256x1024", 256, 1024)):
+            if Lp.tq_probe_empty_launch(wgs, threads, 200, C.byref(val)) == 0:
+                probes[name] = val.value
     extra["machine_probes"] = probes
     if "hbm_stream_read_gbs" in probes:
         result["roofline"]["frac_of_measured_stream_read"] = achieved / probes["hbm_stream_read_gbs"]

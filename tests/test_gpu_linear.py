@@ -317,6 +317,71 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
     assert _rel(y[3:4], y1) < 1e-3
 
 
+# ------------------------------------------------------------------ prefill, 512-row activation panels
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("out,inf,bs,batch", [(16500, 256, 256, 257),      # one ragged panel, ragged last weight tile
+                                              (16640, 512, 128, 600),      # two panels, the second with 88 rows
+                                              (33000, 768, 256, 1030),     # three panels
+                                              (8300, 1024, 512, 1537)])    # four panels, 65 tiles each
+def test_prefill_panel_kernel_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, batch):
+    """More than 256 rows on a layer with enough 512 x 128 output tiles for the chip and a width that is a
+    multiple of 256 take tq_prefill_panel_kernel (activations as MFMA-operand images read straight from
+    global memory, 128 x 128 accumulators per wave): same tolerances as the other prefill kernel, every
+    output dtype, and a row of the batch equal to its batch-1 result."""
+    qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf + batch)
+    x32 = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
+    xbits = oracle.f32_to_bf16_bits(x32)
+    want = oracle.linear_forward(qw, cb, cb, bs, oracle.bf16_bits_to_f32(xbits))
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    y = layer.forward(xbits, tq.BF16, tq.F32)
+    assert y.shape == (batch, out) and np.isfinite(y).all()
+    assert _rel(y, want) < 1e-3
+    for b in (0, 255, 256, batch - 1):                       # no row leaks into another
+        assert _rel(y[b:b + 1], want[b:b + 1]) < 1e-3
+    for c in (0, 127, 128, out - 1):                         # nor a column
+        assert _rel(y[:, c:c + 1], want[:, c:c + 1]) < 1e-3
+    yb = oracle.bf16_bits_to_f32(layer.forward(xbits, tq.BF16, tq.BF16))
+    assert _rel(yb, want) < 5e-3                             # includes the bf16 rounding of the outputs
+    yh = layer.forward(xbits, tq.BF16, tq.F16).astype(np.float32)
+    assert _rel(yh, want) < 1e-3
+    y32 = layer.forward(x32)                                 # fp32 activations take the same path
+    assert _rel(y32, oracle.linear_forward(qw, cb, cb, bs, x32)) < 1e-3
+    y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)
+    assert _rel(y[batch - 1:batch], y1) < 1e-3
+    layer.close()
+
+
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("out,inf,bs,batch,ydt", [(8448, 2048, 512, 2000, "f32"),    # 4 x 66 tiles: 8 left after one round of 256
+                                                  (8400, 2304, 256, 1600, "bf16"),   # ragged last tile, 144 sub-steps in 4 parts
+                                                  (16500, 2048, 128, 1025, "f16")])  # 3 x 129 tiles: 131 left after one round -> 1 part, whole
+def test_prefill_panel_kernel_tail_tiles_in_k_ranges(tq, oracle, mode, out, inf, bs, batch, ydt):
+    """Tiles left over after the last full round of the chip (at most half a round of them, rows of 2048 columns
+    or more) are cut into 2..4 K ranges (dual rotation: one per plane) whose fp32 products a second kernel adds:
+    sampled rows of every panel against the oracle, in particular rows of the last panel, whose last tiles are
+    the ones that are cut."""
+    qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf + batch)
+    x32 = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
+    xbits = oracle.f32_to_bf16_bits(x32)
+    last = (batch - 1) // 512 * 512
+    rows = sorted(r for r in {0, 511, 512, last - 1, last, last + 1, (last + batch) // 2, batch - 2, batch - 1} if r < batch)
+    want = oracle.linear_forward(qw, cb, cb, bs, oracle.bf16_bits_to_f32(xbits[rows]))
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    code = {"f32": tq.F32, "bf16": tq.BF16, "f16": tq.F16}[ydt]
+    y = layer.forward(xbits, tq.BF16, code)
+    y = oracle.bf16_bits_to_f32(y) if ydt == "bf16" else y.astype(np.float32)
+    assert y.shape == (batch, out) and np.isfinite(y).all()
+    tol = 5e-3 if ydt == "bf16" else 1e-3
+    assert _rel(y[rows], want) < tol
+    for k, r in enumerate(rows):
+        assert _rel(y[r:r + 1], want[k:k + 1]) < tol
+    for c0 in range(0, out, 128):                            # every tile of weights, cut or whole
+        assert _rel(y[rows][:, c0:c0 + 128], want[:, c0:c0 + 128]) < tol
+    y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)
+    assert _rel(y[batch - 1:batch], y1) < tol
+    layer.close()
+
+
 # ------------------------------------------------------------------ small batches on the matrix cores
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("out,inf,bs,batch", [(64, 512, 512, 2), (300, 1024, 256, 5), (513, 2048, 512, 15),

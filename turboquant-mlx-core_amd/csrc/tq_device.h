@@ -68,8 +68,9 @@ PrefillPlan prefill_plan(const LayerView& L, int batch, int num_cus, size_t capa
 size_t prefill_reserve_bytes(const LayerView& L, int max_batch, int num_cus);
 hipError_t launch_prefill(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                           void* workspace, const PrefillPlan& plan, hipStream_t stream);
+// panel: fragment images of 512 rows for tq_prefill_panel_kernel instead of 256-row tile images.
 hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
-                               hipStream_t stream);
+                               hipStream_t stream, bool panel = false);
 // Small batches (tq_skinny.hip): 2..32 rows (any activation type) on shared-rotation layers, batch rows as
 // the M side of 16x16x32 MFMAs.  xt_workspace as for launch_prefill; partial: skinny_partial_bytes() for this batch.
 constexpr int kSkinnyMaxRows = 32;

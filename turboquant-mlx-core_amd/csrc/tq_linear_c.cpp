@@ -18,6 +18,7 @@
 
 #include "tq_device.h"
 #include "tq_gemv_common.h"
+#include "tq_prefill_common.h"
 
 namespace {
 thread_local std::string g_last_error;
@@ -375,9 +376,12 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
     void* work = nullptr;
     float* partial = nullptr;
     tq::PrefillPlan plan{};
-    if (prefill) plan = tq::prefill_plan(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0);
+    // (more than 256 rows and enough output tiles: 512-row activation panels, tq_prefill_panel.hip)
+    const bool panel = prefill && tq::prefill_panel_supported(V, batch, device_cu_count());
+    if (prefill && !panel) plan = tq::prefill_plan(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0);
     if (prefill || skinny) {
-        const size_t work_need = prefill ? plan.total_bytes : tq::skinny_workspace_bytes(V, batch);
+        const size_t work_need = panel ? tq::prefill_panel_workspace_bytes(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0)
+                                       : prefill ? plan.total_bytes : tq::skinny_workspace_bytes(V, batch);
         const size_t partial_need = skinny ? tq::skinny_partial_bytes(V, batch) : 0;
         if (static_ws) {
             if (align256(work_need) + partial_need > static_cap) {
@@ -396,6 +400,11 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
             partial = static_cast<float*>(h->d_partial);
         }
     }
+    if (panel)
+        return hip_ok(tq::launch_prefill_panel(V, x_dev, x_dtype, batch, y_dev, y_dtype, work,
+                                               tq::prefill_panel_workspace_bytes(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0),
+                                               device_cu_count(), stream),
+                      "tq_prefill_panel launch") ? 0 : 1;
     if (prefill) {
         // Dense contraction: rotate once, dequantise tiles to fp16 in LDS, MFMA.
         return hip_ok(tq::launch_prefill(V, x_dev, x_dtype, batch, y_dev, y_dtype, work, plan, stream),

@@ -15,15 +15,9 @@
 // LDS table and written to one of two weight tiles.  One barrier per step; the two waves of a
 // SIMD run the decode and the multiply half of a step in opposite order, which keeps the matrix
 // pipe fed during the decodes.
-#include "tq_device.h"
+#include "tq_prefill_common.h"
 
 namespace tq {
-
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
-
-typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
 
 constexpr int kBM = 256, kBN = 256;
 constexpr int kBK = 32;                               // K extent of one LDS tile (one step)
@@ -55,21 +49,6 @@ struct PrefillArgs {
     int steps_per_split;
     float* partial;
 };
-
-__device__ __forceinline__ uint32_t gemm_entry_addr(uint32_t idx_bytes, uint32_t laneoff, int j) {
-    switch (j) {
-        case 0: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0400u);
-        case 1: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0500u);
-        case 2: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0600u);
-        default: return __builtin_amdgcn_perm(idx_bytes, laneoff, 0x0c0c0700u);
-    }
-}
-
-// Table entries hold the fp16 value in the upper half of the dword (low 16 bits zero): two of them
-// pack into one register of two halves with a single byte permute.
-__device__ __forceinline__ uint32_t pack_half2(uint32_t lo_val, uint32_t hi_val) {
-    return __builtin_amdgcn_perm(hi_val, lo_val, 0x07060302u);   // {lo.b2, lo.b3, hi.b2, hi.b3}
-}
 
 // Position of the 16-byte slot that holds columns [8c, 8c+8) of row r inside a 64-byte tile row.
 // The XOR spreads the 16 rows a 128-bit LDS read touches at once over all 16 slot phases
@@ -419,7 +398,11 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 // stored as [M/256][K/32] images of 256 rows x 64 bytes in the exact byte order the GEMM keeps
 // them in LDS (16-byte slots permuted by a_slot), so a tile is one contiguous 16 KB copy.
 // One wave per (row, 2048-column slab), 32 consecutive columns per lane, fp32 butterfly.
+// PANEL: fragment images for tq_prefill_panel_kernel instead, [M/512][K/16][4 waves][4 row blocks][64 lanes x 16 B]:
+// the 8 columns [16 u + 8 g, +8) of row r sit where lane 32 g + r % 32 of wave (r % 512) / 128 expects the
+// A operand of row block (r % 128) / 32 in sub-step u.
 // ---------------------------------------------------------------------------
+template <bool PANEL>
 __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restrict__ x, int x_dtype,
                                                              uint16_t* __restrict__ out, int rows, int cols,
                                                              int chunks, int slabs, uint32_t seed, uint32_t bs,
@@ -444,13 +427,16 @@ __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restri
     if (active) {
         const int m_tile = row >> 8, r = row & 255;
         uint4* dst = reinterpret_cast<uint4*>(out + (((size_t)m_tile * chunks + chunk) * 256 + r) * kBK);
+        // (PANEL: 16-byte units; sub-step 2 chunk + i / 2 of panel row >> 9, block of (wave, row block), lane)
+        uint4* pdst = reinterpret_cast<uint4*>(out) + ((((size_t)(row >> 9) * chunks + chunk) * 2 * 4 + ((row >> 7) & 3)) * 4 + ((row >> 5) & 3)) * 64 + (row & 31);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t w[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 w[j] = (uint32_t)float_to_f16_bits(v[8 * i + 2 * j] * scale) | ((uint32_t)float_to_f16_bits(v[8 * i + 2 * j + 1] * scale) << 16);
-            dst[a_slot(r, i)] = make_uint4(w[0], w[1], w[2], w[3]);
+            if constexpr (PANEL) pdst[(i >> 1) * 1024 + (i & 1) * 32] = make_uint4(w[0], w[1], w[2], w[3]);
+            else dst[a_slot(r, i)] = make_uint4(w[0], w[1], w[2], w[3]);
         }
     }
 }
@@ -521,7 +507,8 @@ size_t prefill_reserve_bytes(const LayerView& L, int max_batch, int num_cus) {
     for (int m_tiles = 1; (m_tiles - 1) * kBM < max_batch; ++m_tiles) {
         const int rows = m_tiles * kBM < max_batch ? m_tiles * kBM : max_batch;
         if (rows < 16) continue;
-        const size_t n = prefill_plan(L, rows, num_cus, ~(size_t)0).total_bytes;
+        const size_t n = prefill_panel_supported(L, rows, num_cus) ? prefill_panel_workspace_bytes(L, rows, num_cus, ~(size_t)0)
+                                                                   : prefill_plan(L, rows, num_cus, ~(size_t)0).total_bytes;
         if (n > need) need = n;
     }
     return need;
@@ -539,18 +526,27 @@ bool prefill_supported(const LayerView& L, int x_dtype, int batch) {
 
 // Rotated activations of `batch` rows as fp16 tile images in `workspace` (both rotations for dual mode).
 hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, int batch, void* workspace,
-                               hipStream_t stream) {
+                               hipStream_t stream, bool panel) {
     const int K = L.in_features, M = batch;
     uint16_t* xt = static_cast<uint16_t*>(workspace);
     const int chunks = K / kChunk;
     const int slabs = (chunks + kWave - 1) / kWave;
     const dim3 rgrid((unsigned)((M + 3) / 4), (unsigned)slabs);
-    hipLaunchKernelGGL(tq_rotate_f16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
+    const int tile_m = panel ? kPanelM : kBM;                      // rows of one image
+    uint16_t* const xt2 = xt + (size_t)((M + tile_m - 1) / tile_m) * tile_m * K;
+    if (panel) {
+        hipLaunchKernelGGL(tq_rotate_f16_kernel<true>, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
+                           L.seed_primary, L.block_size, L.inv_sqrt_bs);
+        if (L.mode == kDual)
+            hipLaunchKernelGGL(tq_rotate_f16_kernel<true>, rgrid, dim3(256), 0, stream, x, x_dtype, xt2, M, K, chunks,
+                               slabs, L.seed_residual, L.block_size, L.inv_sqrt_bs);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(tq_rotate_f16_kernel<false>, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
                        L.seed_primary, L.block_size, L.inv_sqrt_bs);
     if (L.mode == kDual)
-        hipLaunchKernelGGL(tq_rotate_f16_kernel, rgrid, dim3(256), 0, stream, x, x_dtype,
-                           xt + (size_t)((M + kBM - 1) / kBM) * kBM * K, M, K, chunks, slabs, L.seed_residual,
-                           L.block_size, L.inv_sqrt_bs);
+        hipLaunchKernelGGL(tq_rotate_f16_kernel<false>, rgrid, dim3(256), 0, stream, x, x_dtype, xt2, M, K, chunks,
+                           slabs, L.seed_residual, L.block_size, L.inv_sqrt_bs);
     return hipGetLastError();
 }
 

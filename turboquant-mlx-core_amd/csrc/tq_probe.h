@@ -1,11 +1,11 @@
-#ifndef TURBOQUANT_C_TQ_PROBE_H
-#define TURBOQUANT_C_TQ_PROBE_H
+#ifndef TQ_PROBE_H
+#define TQ_PROBE_H
 
 /*
  * Machine probes behind the roofline figures of the benchmark: what this GPU sustains on a
- * pure streaming read and on a pure bf16 or fp16 MFMA loop.  No counterpart in the reference (its
- * benchmarks report wall-clock only, benchmarks/bench_linear.cpp:50-76); nothing in the
- * layer path calls these.
+ * pure streaming read and on a pure bf16 or fp16 MFMA loop, and what an empty launch costs.  No counterpart in
+ * the reference (its benchmarks report wall-clock only, benchmarks/bench_linear.cpp:50-76).  Built into
+ * libtq_probe.so (make probe), which only bench.py loads; not part of the product library or its headers.
  */
 
 #include <stddef.h>
@@ -29,16 +29,13 @@ int tq_probe_mfma_bf16(int random_operands, int iterations, double* tflops);
  * more mantissa bits that toggle. */
 int tq_probe_mfma_f16(int random_operands, int iterations, double* tflops);
 
-/* One workgroup of 16 waves per CU; every wave does `per_wave` device-scope relaxed fetch-adds on one of
- * `addresses` (1..64) words, chosen by workgroup; writes the achieved rate in fetch-adds per microsecond
- * over the whole chip.  What a device-wide work counter could hand out: on MI355X about 90 per
- * microsecond on one word (11 ns each, whoever asks), which is why the batch-1 kernel hands its row
- * groups out from counters in LDS and not from one in memory (an lm_head launch has 76 000 of them in
- * 45 us).  Returns 0 on success. */
-int tq_probe_device_atomics(int addresses, int per_wave, double* per_microsecond);
+/* `launches` launches of a kernel that does nothing (`workgroups` x `threads`), captured in one HIP graph and
+ * replayed: writes the time from one launch to the next in microseconds.  What a layer call costs on this
+ * machine before its first instruction: the floor under the microseconds of a small layer. */
+int tq_probe_empty_launch(int workgroups, int threads, int launches, double* us_per_launch);
 
 #ifdef __cplusplus
 }
 #endif
 
-#endif /* TURBOQUANT_C_TQ_PROBE_H */
+#endif /* TQ_PROBE_H */

@@ -1,11 +1,23 @@
 // Machine probes for the roofline denominators and for design decisions: what this GPU sustains on a pure
-// streaming read, on a pure bf16 or fp16 MFMA loop, and on device-scope fetch-adds from every wave of the chip.
-// Measurement support only: nothing in the layer path calls them.
-#include "turboquant_c/tq_probe.h"
+// streaming read and on a pure bf16 or fp16 MFMA loop, and what a kernel launch costs before it does anything.
+// Measurement support only, a library of its own (libtq_probe.so, `make probe`): nothing in the layer path calls
+// them and the product library does not contain them.
+#include "tq_probe.h"
 
-#include "tq_device.h"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
 
 namespace tq {
+
+namespace {
+bool hip_ok(hipError_t e, const char* what) {
+    if (e == hipSuccess) return true;
+    fprintf(stderr, "tq_probe: %s: %s\n", what, hipGetErrorString(e));
+    return false;
+}
+void set_error(const char* msg) { fprintf(stderr, "%s\n", msg); }
+}  // namespace
 
 typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 probe_f16x8 __attribute__((ext_vector_type(8)));
@@ -58,18 +70,9 @@ __global__ __launch_bounds__(512) void tq_probe_mfma_kernel(float* __restrict__ 
     if (s == 123.456f) sink[0] = s;
 }
 
-// Every wave of a one-workgroup-per-CU launch does `per_wave` device-scope relaxed fetch-adds (lane 0) on
-// one of `addresses` words, 256 bytes apart, chosen by workgroup.
-__global__ __launch_bounds__(1024) void tq_probe_atomic_kernel(unsigned* ctr, int per_wave, int addresses, unsigned* sink) {
-    const int lane = threadIdx.x & 63;
-    unsigned* const c = ctr + (blockIdx.x % addresses) * 64;
-    unsigned acc = 0;
-    for (int i = 0; i < per_wave; ++i) {
-        unsigned t = 0;
-        if (lane == 0) t = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        acc += __builtin_amdgcn_readfirstlane(t);
-    }
-    if (acc == 0xdeadbeefu) sink[0] = acc;
+// A kernel that does nothing: `waves` waves per workgroup start, end, and that is all.
+__global__ void tq_probe_empty_kernel(int* never) {
+    if (never && threadIdx.x == 0xffffff) never[0] = 1;
 }
 
 }  // namespace tq
@@ -143,35 +146,42 @@ int tq_probe_mfma_f16(int random_operands, int iterations, double* tflops) {
     return probe_mfma(true, random_operands, iterations, tflops);
 }
 
-int tq_probe_device_atomics(int addresses, int per_wave, double* per_microsecond) {
+int tq_probe_empty_launch(int workgroups, int threads, int launches, double* us_per_launch) {
     try {
-        if (!per_microsecond || addresses < 1 || addresses > 64 || per_wave < 1) { tq::set_error("tq_probe_device_atomics: bad argument"); return 1; }
-        int dev = 0; hipDeviceProp_t prop;
-        if (!tq::hip_ok(hipGetDevice(&dev), "hipGetDevice") || !tq::hip_ok(hipGetDeviceProperties(&prop, dev), "properties")) return 1;
-        const int cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-        unsigned* ctr = nullptr; unsigned* sink = nullptr;
-        hipEvent_t t0 = nullptr, t1 = nullptr;
-        bool ok = tq::hip_ok(hipMalloc((void**)&ctr, 64 * 64 * sizeof(unsigned)), "hipMalloc(counters)") &&
-                  tq::hip_ok(hipMalloc((void**)&sink, 4), "hipMalloc(sink)") &&
-                  tq::hip_ok(hipMemset(ctr, 0, 64 * 64 * sizeof(unsigned)), "hipMemset(counters)") &&
-                  tq::hip_ok(hipEventCreate(&t0), "event") && tq::hip_ok(hipEventCreate(&t1), "event");
-        float ms = 0.0f;
-        const int reps = 5;
-        if (ok) {
-            hipLaunchKernelGGL(tq::tq_probe_atomic_kernel, dim3(cus), dim3(1024), 0, nullptr, ctr, per_wave, addresses, sink);
-            (void)hipEventRecord(t0, nullptr);
-            for (int r = 0; r < reps; ++r)
-                hipLaunchKernelGGL(tq::tq_probe_atomic_kernel, dim3(cus), dim3(1024), 0, nullptr, ctr, per_wave, addresses, sink);
-            (void)hipEventRecord(t1, nullptr);
-            ok = tq::hip_ok(hipEventSynchronize(t1), "probe sync") && tq::hip_ok(hipEventElapsedTime(&ms, t0, t1), "elapsed");
+        if (!us_per_launch || workgroups < 1 || threads < 64 || threads > 1024 || launches < 1) {
+            tq::set_error("tq_probe_empty_launch: bad argument"); return 1;
         }
-        if (ok) *per_microsecond = (double)cus * 16.0 * per_wave * reps / (ms * 1e3);
+        hipStream_t st = nullptr;
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        hipEvent_t t0 = nullptr, t1 = nullptr;
+        bool ok = tq::hip_ok(hipStreamCreate(&st), "stream") && tq::hip_ok(hipEventCreate(&t0), "event") &&
+                  tq::hip_ok(hipEventCreate(&t1), "event") &&
+                  tq::hip_ok(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal), "begin capture");
+        if (ok) {
+            for (int i = 0; i < launches; ++i)
+                hipLaunchKernelGGL(tq::tq_probe_empty_kernel, dim3(workgroups), dim3(threads), 0, st, (int*)nullptr);
+            ok = tq::hip_ok(hipStreamEndCapture(st, &graph), "end capture") &&
+                 tq::hip_ok(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "instantiate");
+        }
+        float ms = 0.0f;
+        const int reps = 20;
+        if (ok) {
+            for (int r = 0; r < 3 && ok; ++r) ok = tq::hip_ok(hipGraphLaunch(exec, st), "graph launch");
+            ok = ok && tq::hip_ok(hipStreamSynchronize(st), "sync");
+            if (ok) (void)hipEventRecord(t0, st);
+            for (int r = 0; r < reps && ok; ++r) ok = tq::hip_ok(hipGraphLaunch(exec, st), "graph launch");
+            if (ok) (void)hipEventRecord(t1, st);
+            ok = ok && tq::hip_ok(hipEventSynchronize(t1), "probe sync") && tq::hip_ok(hipEventElapsedTime(&ms, t0, t1), "elapsed");
+        }
+        if (ok) *us_per_launch = (double)ms * 1e3 / ((double)reps * launches);
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (graph) (void)hipGraphDestroy(graph);
         if (t0) (void)hipEventDestroy(t0);
         if (t1) (void)hipEventDestroy(t1);
-        if (ctr) (void)hipFree(ctr);
-        if (sink) (void)hipFree(sink);
+        if (st) (void)hipStreamDestroy(st);
         return ok ? 0 : 1;
-    } catch (...) { tq::set_error("tq_probe_device_atomics: exception"); return 1; }
+    } catch (...) { tq::set_error("tq_probe_empty_launch: exception"); return 1; }
 }
 
 }  // extern "C"
