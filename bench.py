@@ -446,30 +446,32 @@ def main():
                 xp = torch.randn(M, inp, device="cuda", generator=g).to(torch.bfloat16)
                 yp = torch.empty(M, outp, device="cuda", dtype=torch.bfloat16)
                 L = tq.lib()
-                for _ in range(2):
+
+                def timed(call, reps=20):
+                    """Untimed calls until the chip has been under this load for 0.1 s (its clocks settle over tens
+                    of milliseconds: the first calls after a pause run up to 15 % slower), then one event bracket."""
+                    t_end = time.perf_counter() + 0.1
+                    while time.perf_counter() < t_end:
+                        for _ in range(5):
+                            call()
+                        torch.cuda.synchronize()
+                    st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    st.record()
+                    for _ in range(reps):
+                        call()
+                    en.record()
+                    torch.cuda.synchronize()
+                    return st.elapsed_time(en) * 1e3 / reps
+
+                def ours():
                     if L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None) != 0:
                         raise RuntimeError(tq.last_error())
-                torch.cuda.synchronize()
-                st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                reps = 10
-                st.record()
-                for _ in range(reps):
-                    L.tq_linear_forward(hp, xp.data_ptr(), tq.BF16, M, yp.data_ptr(), tq.BF16, None)
-                en.record()
-                torch.cuda.synchronize()
-                usp = st.elapsed_time(en) * 1e3 / reps
+                usp = timed(ours)
                 flops = 2.0 * M * outp * inp
                 # The vendor library's plain bf16 GEMM of the same shape on already dequantised weights
                 # (torch.matmul -> hipBLASLt): what a matrix kernel with no decode work reaches on this machine.
                 wv = (torch.randn(outp, inp, device="cuda", generator=g) * 0.01).to(torch.bfloat16)
-                for _ in range(3):
-                    torch.matmul(xp, wv.t(), out=yp)
-                st.record()
-                for _ in range(reps):
-                    torch.matmul(xp, wv.t(), out=yp)
-                en.record()
-                torch.cuda.synchronize()
-                usv = st.elapsed_time(en) * 1e3 / reps
+                usv = timed(lambda: torch.matmul(xp, wv.t(), out=yp))
                 del wv
                 extra[f"prefill_{outp}x{inp}_M{M}_bf16"] = {"us_per_layer": usp, "tflops": flops / usp / 1e6,
                                                           "vendor_plain_bf16_gemm_same_shape_us": usv,

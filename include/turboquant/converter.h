@@ -24,8 +24,8 @@ struct ConversionConfig {
 /// sensitive_layers_start and last sensitive_layers_end numbered layers; everything else is
 /// copied to "<shard>_passthrough.safetensors".  Other files of the directory are copied and
 /// config.json gains a "quantization_config" block.  Returns false if the input directory does
-/// not exist.  A weight this library's quantizer cannot take (width not a multiple of 32, more
-/// than 32768 columns, block size below 2) is passed through unchanged, with a line on stderr.
+/// not exist.  A weight with an odd number of columns (two columns share a byte of the 4-bit planes) is
+/// passed through unchanged, with a line on stderr.
 bool convert_model(const ConversionConfig& config);
 
 /// True if some safetensors file in the directory carries quantization_method=turboquant.

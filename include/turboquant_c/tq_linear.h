@@ -119,7 +119,10 @@ int tq_linear_reserve(tq_linear_t layer, int max_batch);
  * here into as many ranges as the array holds, so the last bits of a result can differ from
  * tq_linear_forward's by the order of those sums.)  Each GPU has one such array, shared
  * by every call on it and keeping the previous call's contents: calls that overlap on one GPU
- * (different streams or threads) race.  One row uses no workspace.
+ * (different streams or threads) race.  One row uses no part of the array (layers wider than 16384 columns,
+ * widths that are not a multiple of 32 and 5-bit layers that keep two planes use the handle's own rotated row
+ * at one row too: serialise calls per handle on those, as with tq_linear_forward).  The array's address on the
+ * current device is looked up when a layer is created, so the first call does no runtime work either.
  */
 #define TQ_STATIC_SCRATCH_BYTES (32u << 20)
 int tq_linear_forward_static(tq_linear_t layer, const void* x_dev, int x_dtype, int batch,

@@ -325,7 +325,10 @@ def test_cli_convert_then_dequant_model_directory(tmp_path, oracle, per_layer, s
     tensors = {"model.embed_tokens.weight": (rng.standard_normal((96, 64)) * 0.05).astype(np.float16),
                "lm_head.weight": (rng.standard_normal((96, 64)) * 0.05).astype(np.float32),
                "model.norm.weight": np.ones(64, np.float32),
-               "model.layers.1.mlp.odd.weight": (rng.standard_normal((8, 48)) * 0.05).astype(np.float32)}
+               # a width that is not a multiple of 32 (blocks of 16 columns) is quantized like any other; an odd
+               # width cannot share bytes between column pairs and is left as it is
+               "model.layers.1.mlp.narrow.weight": (rng.standard_normal((8, 48)) * 0.05).astype(np.float32),
+               "model.layers.2.mlp.odd.weight": (rng.standard_normal((8, 45)) * 0.05).astype(np.float32)}
     for n in range(4):
         tensors[f"model.layers.{n}.self_attn.q_proj.weight"] = (rng.standard_normal((64, 64)) * 0.05).astype(np.float32)
         tensors[f"model.layers.{n}.mlp.up_proj.weight"] = (rng.standard_normal((160, 1536)) * 0.02).astype(np.float16)
@@ -341,8 +344,9 @@ def test_cli_convert_then_dequant_model_directory(tmp_path, oracle, per_layer, s
         args.append("--shared-rotation")
     p = subprocess.run(args, capture_output=True, text=True, timeout=600)
     assert p.returncode == 0, p.stdout + p.stderr
-    assert "Sensitive layers: 4 weights kept at fp16, 6 weights quantized" in p.stdout
-    assert "model.layers.1.mlp.odd.weight [8, 48] left unquantized" in p.stderr
+    assert "Sensitive layers: 4 weights kept at fp16, 7 weights quantized" in p.stdout
+    assert "model.layers.2.mlp.odd.weight [8, 45] left unquantized" in p.stderr
+    assert "narrow" not in p.stderr
 
     cfg = json.loads((out / "config.json").read_text())
     assert cfg["model_type"] == "toy"
@@ -357,13 +361,13 @@ def test_cli_convert_then_dequant_model_directory(tmp_path, oracle, per_layer, s
     assert (meta.get("tq_per_layer_codebooks") == "true") == per_layer
     tq_t = load_file(str(out / "model.safetensors"))
     pt = load_file(str(out / "model_passthrough.safetensors"))
-    quantized = ["model.embed_tokens", "lm_head"] + [f"model.layers.{n}.{m}" for n in (1, 2)
-                                                      for m in ("self_attn.q_proj", "mlp.up_proj")]
+    quantized = ["model.embed_tokens", "lm_head", "model.layers.1.mlp.narrow"] + \
+                [f"model.layers.{n}.{m}" for n in (1, 2) for m in ("self_attn.q_proj", "mlp.up_proj")]
     assert sorted(k[:-len(".packed_primary")] for k in tq_t if k.endswith(".packed_primary")) == sorted(quantized)
     for name in quantized:
         w = tensors[name + ".weight"].astype(np.float32)
         o_f, i_f = w.shape
-        bs = 512 if i_f == 1536 else 64                              # largest power of two <= 512 dividing the width
+        bs = {1536: 512, 64: 64, 48: 16}[i_f]                       # largest power of two <= 512 dividing the width
         assert tq_t[name + ".packed_primary"].shape == (o_f, i_f // 2) and tq_t[name + ".packed_primary"].dtype == np.uint8
         assert tq_t[name + ".packed_residual"].shape == (o_f, i_f // 2)
         assert tq_t[name + ".norms"].shape == (o_f,) and tq_t[name + ".norms"].dtype == np.float32

@@ -341,3 +341,55 @@ def test_down_projection_5120x27648_prefill_few_output_tiles(tq, oracle, shared)
     yb = o.bf16_bits_to_f32(layer.forward(xbits[:512], tq.BF16, tq.BF16))
     assert _rel(yb[:, rows], want[:512]) < 5e-3
     layer.close()
+
+
+@pytest.mark.parametrize("shared", [True, False], ids=["shared_rotation", "dual_rotation"])
+def test_decoder_layer_projections_32b_batch_1_4_8(tq, oracle, shared):
+    """The 32B-shaped decoder layer as the benchmark launches it: q + k + v (5120 + 1024 + 1024 rows) and
+    gate + up (2 x 27648 rows) through tq_linear_forward_group, o alone, at 1, 4 and 8 rows of bf16
+    activations.  The host-computed row partition of a shared launch depends on every layer's row count, so
+    the full row counts are what is run: sampled rows of every layer against the oracle (recomputed from the
+    packed bytes of just those rows), first and last rows included, the grouped results equal bit for bit to
+    one call per layer, and q, o, k, v alone as well."""
+    o = oracle
+    hip = _Hip()
+    hidden, kv, inter, bs = 5120, 1024, 27648, 512
+    cb = o.generate_codebook(4)
+    shapes = {"q": hidden, "k": kv, "v": kv, "o": hidden, "gate": inter, "up": inter}
+    layers, qws = {}, {}
+    for i, (name, rows) in enumerate(shapes.items()):
+        w = _weights(rows, hidden, 0.01, 70 + i)
+        qws[name] = tq.quantize_weight(w, cb, cb, 4, 4, bs, shared)
+        del w
+        layers[name] = tq.TurboQuantLinear(hidden, rows, qws[name], cb, cb, bs)
+        assert layers[name].mode() == ("shared_lut" if shared else "dual")
+    rs = np.random.default_rng(77)
+    samples, w_rows = {}, {}
+    o.set_threads(8)
+    for name, rows in shapes.items():
+        pick = np.unique(np.concatenate([[0, 1, rows - 2, rows - 1], rs.choice(rows, 300, replace=False)]))
+        samples[name] = pick
+        w_rows[name] = o.dequantize_weight_cpu(_rows_subset(o, qws[name], pick), cb, cb, bs)
+    o.set_threads(1)
+    xbits = o.f32_to_bf16_bits(rs.standard_normal((8, hidden)).astype(np.float32))
+    x = o.bf16_bits_to_f32(xbits)
+    for batch in (1, 4, 8):
+        x_dev = hip.upload(xbits[:batch])
+        want = {name: o.matmul_xwT(x[:batch], w_rows[name], acc_double=True) for name in shapes}
+        alone = {name: layers[name].forward(xbits[:batch], tq.BF16, tq.F32) for name in shapes}
+        for name in shapes:                                              # every layer by itself
+            assert alone[name].shape == (batch, shapes[name]) and np.isfinite(alone[name]).all()
+            assert _rel(alone[name][:, samples[name]], want[name]) < 1e-3
+            for b in range(batch):
+                assert _rel(alone[name][b, samples[name]], want[name][b]) < 1e-3
+        for group in (("q", "k", "v"), ("gate", "up")):                  # the shared launches of the benchmark
+            outs = [hip.alloc(batch * shapes[n] * 4) for n in group]
+            tq.forward_group_device([layers[n] for n in group], x_dev, tq.BF16, batch, outs, tq.F32)
+            for n, ptr in zip(group, outs):
+                y = hip.download(ptr, (batch, shapes[n]), np.float32)
+                assert np.array_equal(y, alone[n])                       # same bits as one call per layer
+                assert _rel(y[:, samples[n]], want[n]) < 1e-3
+            hip.free(*outs)
+        hip.free(x_dev)
+    for l in layers.values():
+        l.close()

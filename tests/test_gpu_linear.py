@@ -421,6 +421,33 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     layer.close()
 
 
+@pytest.mark.parametrize("mode", ["shared", "dual"])
+@pytest.mark.parametrize("batch", [2, 4, 16, 40, 64])
+@pytest.mark.parametrize("scale", [1e-4, 1e3, 1e4])
+def test_matrix_core_paths_hold_their_tolerance_over_the_fp16_range(tq, oracle, mode, batch, scale):
+    """The matrix-core paths (2 rows and more) round the rotated activations, normalised by 1 / sqrt(block), to
+    fp16.  Activations of 1e-4 .. 1e4 times a standard normal stay inside fp16's normal range after the rotation
+    (a rotated value is bounded by the L2 norm of its block of the input), so the outputs keep 1e-3 against the
+    oracle for fp32 and bf16 activations alike and agree with the exact fp32 batch-1 kernel on the same row.
+    (Below about 1e-5 the rotated values become fp16 subnormals, beyond 65504 they saturate: the reference
+    casts its input itself to f16, src/dequantizer.cpp:691, and has the same limits.)"""
+    out, inf, bs = 300, 2048, 512
+    qw, cbp, cbr = _make(oracle, out, inf, bs, mode)
+    x32 = (np.random.default_rng(batch).standard_normal((batch, inf)) * scale).astype(np.float32)
+    layer = tq.TurboQuantLinear(inf, out, qw, cbp, cbr, bs)
+    want = oracle.linear_forward(qw, cbp, cbr, bs, x32)
+    y = layer.forward(x32)
+    assert np.isfinite(y).all() and _rel(y, want) < 1e-3
+    for b in range(batch):
+        assert _rel(y[b:b + 1], want[b:b + 1]) < 1e-3
+    xbits = oracle.f32_to_bf16_bits(x32)
+    yb = layer.forward(xbits, tq.BF16, tq.F32)
+    assert _rel(yb, oracle.linear_forward(qw, cbp, cbr, bs, oracle.bf16_bits_to_f32(xbits))) < 1e-3
+    y1 = layer.forward(x32[batch - 1:batch])                  # one row: the fp32 kernel
+    assert _rel(y[batch - 1:batch], y1) < 1e-3
+    layer.close()
+
+
 def _random_cases(n, seed):
     rng = np.random.default_rng(seed)
     cases = []

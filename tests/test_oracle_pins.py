@@ -110,6 +110,19 @@ def test_validate_codebook_rejects_bad(oracle):
     assert not oracle.validate_codebook(skew)     # analytical must be symmetric
     skew.analytical = False
     assert oracle.validate_codebook(skew)
+    # boundaries must be the midpoints to 1e-5 (src/codebook.cpp:337-340): 1e-4 off fails, 5e-6 off passes
+    off = oracle.Codebook(cb.centroids.copy(), 4, analytical=True)
+    off.boundaries = off.boundaries.copy()
+    off.boundaries[7] += np.float32(1e-4)
+    assert not oracle.validate_codebook(off)
+    near = oracle.Codebook(cb.centroids.copy(), 4, analytical=True)
+    near.boundaries = near.boundaries.copy()
+    near.boundaries[3] = np.float32(near.boundaries[3] + np.float32(5e-6))
+    assert abs(float(near.boundaries[3]) - float((cb.centroids[3] + cb.centroids[4]) * np.float32(0.5))) < 1e-5
+    assert oracle.validate_codebook(near)
+    short = oracle.Codebook(cb.centroids.copy(), 4, analytical=True)
+    short.boundaries = short.boundaries[:-1].copy()            # one boundary missing
+    assert not oracle.validate_codebook(short)
 
 
 def test_quantize_is_lower_bound(oracle):
@@ -195,6 +208,51 @@ def test_lloyd_max_fixed_point_and_normal_fit(oracle):
     idx0 = np.minimum(np.searchsorted(ref.boundaries, data, side="left"), 15)
     m0 = np.array([np.float32(data[idx0 == k].astype(np.float64).sum() / (idx0 == k).sum()) for k in range(16)])
     assert np.allclose(one.centroids, m0, rtol=0, atol=1e-7)
+
+
+def test_lloyd_max_runs_to_the_reference_stopping_rule(oracle):
+    """The whole fit by hand (src/codebook.cpp:99-143): bins by lower_bound on the midpoints of the current
+    centroids, means from double sums rounded once to float, a bin without data keeps its centroid, and the
+    loop ends after the first iteration in which no centroid moves by 1e-6 or more
+    (kLloydMaxShiftThreshold, src/codebook.cpp:68,132).  The oracle must stop in exactly the same iteration
+    and hold the same centroids; a looser threshold stops several iterations earlier on this data."""
+    rng = np.random.default_rng(23)
+    data = np.concatenate([rng.standard_normal(20000) * 0.7, rng.standard_normal(3333) * 2.5 + 0.4]).astype(np.float32)
+    for bits in (2, 3, 4):
+        n = 1 << bits
+        c = oracle.generate_codebook(bits).centroids.copy()
+        stops = {}                                             # threshold -> iteration at which it would stop
+        done = None
+        for it in range(1, 301):
+            b = ((c[:-1] + c[1:]) * np.float32(0.5)).astype(np.float32)
+            idx = np.minimum(np.searchsorted(b, data, side="left"), n - 1)
+            shift = np.float32(0.0)
+            for k in range(n):
+                sel = data[idx == k]
+                if sel.size:
+                    nv = np.float32(sel.astype(np.float64).sum() / sel.size)
+                    shift = max(shift, np.float32(abs(nv - c[k])))
+                    c[k] = nv
+            for thr in (1e-3, 1e-4, 1e-5):
+                if shift < np.float32(thr) and thr not in stops:
+                    stops[thr] = it
+            if shift < np.float32(1e-6):
+                done = it
+                break
+        assert done is not None and done < 300
+        got = oracle.generate_codebook_from_data(data, bits, 300)
+        assert got.iterations == done
+        assert np.abs(got.centroids - c).max() <= 1e-7
+        assert np.array_equal(got.boundaries, ((c[:-1] + c[1:]) * np.float32(0.5)).astype(np.float32))
+        # the test has teeth: looser thresholds would have stopped earlier, with other centroids (1e-5 cannot be
+        # told from 1e-6 on data of this size: the last shifts drop from about 1e-5 to exactly 0 in one step)
+        assert stops[1e-3] < done and stops[1e-4] <= done
+        if bits < 4:
+            assert stops[1e-3] < stops[1e-4] < done
+        early = oracle.generate_codebook_from_data(data, bits, stops[1e-3])
+        assert np.abs(early.centroids - c).max() > 1e-5
+        # the iteration cap is honoured as well
+        assert oracle.generate_codebook_from_data(data, bits, 2).iterations == 2
 
 
 def test_lloyd_max_thread_invariance(oracle):
@@ -317,6 +375,25 @@ def test_quantizer_properties_from_reference_tests(oracle):
     Wz = oracle.dequantize_weight_cpu(qz, cbp, cbr, 128)
     assert np.isfinite(Wz).all() and np.isfinite(qz.norms).all()
     assert np.abs(Wz[3]).max() < 1e-6
+
+
+def test_stored_residual_seed(oracle):
+    """seeds[1] is 0 only when both passes share the rotation AND there is a residual pass
+    (src/quantizer.cpp:255-256): a primary-only layer quantised with shared_rotation set keeps its derived
+    residual seed, which equals the one the dual-rotation call stores, and is never 0."""
+    w = oracle.lcg_matrix(16, 256, 7)
+    cb = oracle.generate_codebook(4)
+    shared44 = oracle.quantize_weight(w, cb, cb, 4, 4, 128, True)
+    dual44 = oracle.quantize_weight(w, cb, cb, 4, 4, 128, False)
+    shared40 = oracle.quantize_weight(w, cb, cb, 4, 0, 128, True)
+    dual40 = oracle.quantize_weight(w, cb, cb, 4, 0, 128, False)
+    assert shared44.seeds[1] == 0 and dual44.seeds[1] != 0
+    assert shared40.seeds[1] != 0 and shared40.seeds[1] == dual44.seeds[1] == dual40.seeds[1]
+    assert shared44.seeds[0] == dual44.seeds[0] == shared40.seeds[0] != 0
+    assert shared44.seeds[0] != dual44.seeds[1]                # two salts (src/quantizer.cpp:82-83)
+    assert all(q.seeds[2] == 128 for q in (shared44, dual44, shared40, dual40))
+    assert not shared40.packed_residual.any()                  # no residual pass: an all-zero plane
+    assert np.array_equal(shared40.packed_primary, dual40.packed_primary)
 
 
 def test_threads_do_not_change_results(oracle):

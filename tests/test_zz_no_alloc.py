@@ -51,6 +51,12 @@ class _Hip:
         for p in ptrs:
             self.rt.hipFree(p)
 
+    def free_bytes(self):
+        """Free device memory as the runtime reports it: any hipMalloc / hipFree in between changes it."""
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert self.rt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
 
 def _make(o, out, inf, bs, mode, seed=7):
     w = (np.random.default_rng(seed).standard_normal((out, inf)) * 0.05).astype(np.float32)
@@ -89,7 +95,10 @@ def test_static_forward_equals_forward_two_calls_in_a_row(tq, oracle, mode, out,
         y_ref_dev, y_dev = hip.alloc(batch * out * 4), hip.alloc(batch * out * 4)
         layer.forward_device(x_dev, tq.BF16, batch, y_ref_dev, tq.F32)
         want = hip.download(y_ref_dev, (batch, out), np.float32)
+        free_before = hip.free_bytes()
         layer.forward_static_device(x_dev, tq.BF16, batch, y_dev, tq.F32)
+        assert hip.rt.hipDeviceSynchronize() == 0
+        assert hip.free_bytes() == free_before, "the static entry point allocated or freed device memory"
         got = hip.download(y_dev, (batch, out), np.float32)
         assert np.array_equal(got, want), f"call {k}, batch {batch}"      # same kernels: bit-exact
         ref = o.matmul_xwT(o.bf16_bits_to_f32(xbits), w_ref, acc_double=True)
@@ -149,7 +158,10 @@ def test_static_forward_cuts_k_into_fewer_ranges_when_the_array_is_short(tq, ora
     layer.forward_device(x_dev, tq.BF16, batch, y_ref_dev, tq.F32)
     want = hip.download(y_ref_dev, (batch, out), np.float32)
     for _ in range(2):
+        free_before = hip.free_bytes()
         layer.forward_static_device(x_dev, tq.BF16, batch, y_dev, tq.F32)
+        assert hip.rt.hipDeviceSynchronize() == 0
+        assert hip.free_bytes() == free_before, "the static entry point allocated or freed device memory"
         got = hip.download(y_dev, (batch, out), np.float32)
         assert _rel(got, want) < 1e-5
         assert _rel(got, ref) < 1e-3

@@ -53,11 +53,11 @@ Codebook codebook_of(const float* centroids, int n, uint8_t bits) {
     return cb;
 }
 
-// The GPU quantizer works on 32-column lane chunks: widths that are a multiple of 32 (every block size the
-// block-size rule can then pick is fine).  Narrower multiples (a width of 48 gets blocks of 16) are left
-// unquantized and reported; files that hold such layers, written by the reference, still load and run.
+// What the layout can hold: an even width (two columns share a byte of the nibble planes) and a power-of-two
+// block of at most 2048 columns (the block rule of src/converter.cpp:228-240 never picks more than 512).  An
+// odd width is left unquantized and reported.
 bool quantizer_takes(int in_features, uint32_t block_size) {
-    return in_features % 32 == 0 && block_size >= 2 && block_size <= 2048;
+    return in_features % 2 == 0 && block_size >= 1 && block_size <= 2048 && in_features % (int)block_size == 0;
 }
 
 }  // namespace

@@ -106,6 +106,7 @@ struct QuantArgsHost {
 hipError_t launch_row_norms(const float* w, float* norms, int out, int in, hipStream_t stream);
 hipError_t launch_derive_seeds(const float* w, size_t n_floats, uint32_t* seeds_dev, hipStream_t stream);
 hipError_t launch_quantize_rows(const QuantArgsHost& h, hipStream_t stream);
+int quantize_partials_per_row(int in, uint32_t bs);      // doubles per row of recon_partial / launch_finish_norms' `slabs`
 hipError_t launch_finish_norms(const float* orig, const double* partial, float* norms, int out, int slabs,
                                hipStream_t stream);
 hipError_t launch_lloyd_pass(const float* data, size_t n, const float* bounds_dev, int nc, int subtract,

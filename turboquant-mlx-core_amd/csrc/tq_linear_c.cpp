@@ -112,6 +112,33 @@ struct tq_linear_s {
     }
 };
 
+// Workspace of the matrix-core paths for callers that cannot allocate (tq_linear_forward_static):
+// rotated activations (tile images) followed by the per-chunk partial products of the small-batch
+// kernels.  One copy per GPU, held until the process ends; every call on a GPU shares it, so calls
+// that overlap on one GPU race.  Nothing in it has to start at zero: the kernels write every element
+// they later read (rows past the batch are computed from whatever is there and never stored).
+static __device__ __align__(256) unsigned char scratch[TQ_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+// Device address of `scratch` on the current device (the array's name is only a host-side stand-in).
+void* static_scratch_ptr() {
+    static std::mutex mu;
+    static void* ptrs[64] = {};
+    int dev = 0;
+    if (!hip_ok(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+    if (dev < 0 || dev >= 64) { set_error("tq_linear_forward_static: device index out of range"); return nullptr; }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        if (!hip_ok(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+        ptrs[dev] = p;
+    }
+    return ptrs[dev];
+}
+
+}  // namespace
+
 namespace {
 
 // Decode tables as 256 floats.
@@ -186,6 +213,9 @@ tq_linear_t create_impl(int in_features, int out_features,
         return nullptr;
     }
 
+    // tq_linear_forward_static must not do runtime work on its first call (a caller may be capturing its
+    // stream): the address of the static workspace on this device is looked up here, once.
+    if (!static_scratch_ptr()) return nullptr;
     tq_linear_s* h = new (std::nothrow) tq_linear_s();
     if (!h) { set_error("tq_linear_create: out of host memory"); return nullptr; }
     const size_t pbytes = (size_t)out_features * primary_cols;
@@ -327,30 +357,7 @@ tq_linear_t create_impl(int in_features, int out_features,
 
 }  // namespace
 
-// Workspace of the matrix-core paths for callers that cannot allocate (tq_linear_forward_static):
-// rotated activations (tile images) followed by the per-chunk partial products of the small-batch
-// kernels.  One copy per GPU, held until the process ends; every call on a GPU shares it, so calls
-// that overlap on one GPU race.  Nothing in it has to start at zero: the kernels write every element
-// they later read (rows past the batch are computed from whatever is there and never stored).
-__device__ __align__(256) unsigned char scratch[TQ_STATIC_SCRATCH_BYTES];
-
 namespace {
-
-// Device address of `scratch` on the current device (the array's name is only a host-side stand-in).
-void* static_scratch_ptr() {
-    static std::mutex mu;
-    static void* ptrs[64] = {};
-    int dev = 0;
-    if (!hip_ok(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
-    if (dev < 0 || dev >= 64) { set_error("tq_linear_forward_static: device index out of range"); return nullptr; }
-    std::lock_guard<std::mutex> lock(mu);
-    if (!ptrs[dev]) {
-        void* p = nullptr;
-        if (!hip_ok(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
-        ptrs[dev] = p;
-    }
-    return ptrs[dev];
-}
 
 size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
@@ -515,10 +522,12 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
             size_t work = 0, part = 0;
             for (int k = 0; k < 2; ++k) {
                 const tq::LayerView& P = h->plane_view[k];
-                const size_t small = tq::skinny_workspace_bytes(P, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows);
+                const int rows = max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows;
+                const bool sk = tq::skinny_supported(P, tq::kBF16, rows);        // (layers the small-batch kernels never take need none of it)
+                const size_t small = sk ? tq::skinny_workspace_bytes(P, rows) : 0;
                 const size_t big = max_batch >= 16 ? tq::prefill_reserve_bytes(P, max_batch, device_cu_count()) : 0;
                 work = std::max(work, std::max(small, big));
-                part = std::max(part, tq::skinny_partial_bytes(P, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows));
+                if (sk) part = std::max(part, tq::skinny_partial_bytes(P, rows));
             }
             if (!ensure_stage(&h->d_work, &h->work_bytes, work, nullptr, &h->retired)) return 1;
             if (!ensure_stage(&h->d_partial, &h->partial_bytes, part, nullptr, &h->retired)) return 1;
@@ -526,10 +535,14 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
             return 0;
         }
         const tq::LayerView& V = h->has_fwd_view ? h->fwd_view : h->view;
-        const size_t small = tq::skinny_workspace_bytes(V, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows);
-        const size_t big = max_batch >= 16 ? tq::prefill_reserve_bytes(V, max_batch, device_cu_count()) : 0;
-        if (!ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big, nullptr, &h->retired)) return 1;
-        if (!ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows), nullptr, &h->retired)) return 1;
+        const int rows = max_batch < tq::kSkinnyMaxRows ? max_batch : tq::kSkinnyMaxRows;
+        // (a layer the small-batch kernels never take needs neither their tile images nor their partial products)
+        const bool sk = tq::lanes_supported(V.in_features, V.block_size) && tq::skinny_supported(V, tq::kBF16, rows);
+        const size_t small = sk ? tq::skinny_workspace_bytes(V, rows) : 0;
+        const bool pf = tq::lanes_supported(V.in_features, V.block_size) && max_batch >= 16 && tq::prefill_supported(V, tq::kBF16, max_batch);
+        const size_t big = pf ? tq::prefill_reserve_bytes(V, max_batch, device_cu_count()) : 0;
+        if ((small || big) && !ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big, nullptr, &h->retired)) return 1;
+        if (sk && !ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, rows), nullptr, &h->retired)) return 1;
         return 0;
     } catch (...) { set_error("tq_linear_reserve: exception"); return 1; }
 }

@@ -214,6 +214,143 @@ __global__ __launch_bounds__(kQWaves* kWave) void tq_quantize_kernel(QuantArgs a
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same pipeline for blocks of 1 to 16 columns, i.e. every width that is not a multiple of 32 (the block rule
+// of src/converter.cpp:228-240 then picks 16 columns at most) and blocks of one column: the reference quantises
+// whatever width is a multiple of its block (src/quantizer.cpp:41-79).  One thread per unit of max(BS, 2)
+// columns (whole bytes of the nibble planes), blocks entirely in registers; the butterfly is the in-register
+// part of fwht_lanes, so every fp32 operation and its order are those of the kernel above.  No tuning: these
+// shapes are small.
+// ---------------------------------------------------------------------------
+template <int BS>
+__device__ __forceinline__ void small_forward(float* x, uint32_t seed, float inv_sqrt_bs) {
+#pragma unroll
+    for (int k = 0; k < BS; ++k) x[k] *= sign_of(seed, (uint32_t)k);
+#pragma unroll
+    for (int h = 1; h < BS; h <<= 1)
+#pragma unroll
+        for (int i = 0; i < BS; i += 2 * h)
+#pragma unroll
+            for (int j = i; j < i + h; ++j) { const float p = x[j], q = x[j + h]; x[j] = p + q; x[j + h] = p - q; }
+#pragma unroll
+    for (int k = 0; k < BS; ++k) x[k] *= inv_sqrt_bs;
+}
+
+template <int BS>
+__device__ __forceinline__ void small_inverse(float* x, uint32_t seed, float inv_sqrt_bs) {
+#pragma unroll
+    for (int h = 1; h < BS; h <<= 1)
+#pragma unroll
+        for (int i = 0; i < BS; i += 2 * h)
+#pragma unroll
+            for (int j = i; j < i + h; ++j) { const float p = x[j], q = x[j + h]; x[j] = p + q; x[j + h] = p - q; }
+#pragma unroll
+    for (int k = 0; k < BS; ++k) x[k] *= inv_sqrt_bs * sign_of(seed, (uint32_t)k);
+}
+
+template <int BS>
+__global__ __launch_bounds__(256) void tq_quantize_small_kernel(QuantArgs a) {
+    constexpr int U = BS < 2 ? 2 : BS;              // columns of one thread
+    constexpr int NB = U / BS;                      // its blocks
+    __shared__ float tab[96];
+    for (int i = threadIdx.x; i < 96; i += blockDim.x) tab[i] = a.tables[i];
+    __syncthreads();
+    const float* cP = tab;
+    const float* bP = tab + 32;
+    const float* cR = tab + 64;
+    const float* bR = tab + 80;
+    const int units = a.in / U;                     // a.slabs == units: one partial sum of squares per unit
+    const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int row = (int)(id / units);
+    const int unit = (int)(id - (long long)row * units);
+    if (row >= a.out) return;
+    const size_t elem0 = (size_t)row * a.in + (size_t)unit * U;
+
+    float v[U];
+    const float nrm = a.orig_norm[row];
+    const float safe = nrm > 1e-10f ? nrm : 1e-10f;
+#pragma unroll
+    for (int k = 0; k < U; ++k) v[k] = a.w[elem0 + k] / safe;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) small_forward<BS>(v + b * BS, a.seed_p, a.inv_sqrt_bs);
+#pragma unroll
+    for (int k = 0; k < U; ++k) v[k] *= a.scale_factor;
+    if (a.scaled_out) {
+#pragma unroll
+        for (int k = 0; k < U; ++k) a.scaled_out[elem0 + k] = v[k];
+    }
+    if (!a.quantize) return;
+
+    uint32_t ip[U], ir[U];
+    const int nbp = a.n_primary - 1, nbr = a.n_residual - 1;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        const uint32_t idx = bin_of(v[k], bP, nbp);
+        ip[k] = idx >= (uint32_t)a.n_primary ? a.n_primary - 1 : idx;
+        ir[k] = 0;
+    }
+    float rec[U];
+    if (a.residual_bits > 0) {
+        float res[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) res[k] = v[k] - cP[ip[k]];
+        if (!a.shared_rotation) {
+#pragma unroll
+            for (int k = 0; k < U; ++k) res[k] *= a.inv_scale;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                small_inverse<BS>(res + b * BS, a.seed_p, a.inv_sqrt_bs);
+                small_forward<BS>(res + b * BS, a.seed_r, a.inv_sqrt_bs);
+            }
+#pragma unroll
+            for (int k = 0; k < U; ++k) res[k] *= a.scale_factor;
+        }
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            const uint32_t idx = bin_of(res[k], bR, nbr);
+            ir[k] = idx >= (uint32_t)a.n_residual ? a.n_residual - 1 : idx;
+        }
+    }
+    if (a.residual_bits > 0 && a.shared_rotation) {
+#pragma unroll
+        for (int k = 0; k < U; ++k) rec[k] = (cP[ip[k]] + cR[ir[k] & 15u]) * a.inv_scale;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) small_inverse<BS>(rec + b * BS, a.seed_p, a.inv_sqrt_bs);
+    } else {
+#pragma unroll
+        for (int k = 0; k < U; ++k) rec[k] = cP[ip[k]] * a.inv_scale;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) small_inverse<BS>(rec + b * BS, a.seed_p, a.inv_sqrt_bs);
+        if (a.residual_bits > 0) {
+            float r2[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) r2[k] = cR[ir[k] & 15u] * a.inv_scale;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) small_inverse<BS>(r2 + b * BS, a.seed_r, a.inv_sqrt_bs);
+#pragma unroll
+            for (int k = 0; k < U; ++k) rec[k] = rec[k] + r2[k];
+        }
+    }
+    double acc = 0.0;
+#pragma unroll
+    for (int k = 0; k < U; ++k) { const float sq = rec[k] * rec[k]; acc += (double)sq; }
+    a.recon_partial[(size_t)row * units + unit] = acc;
+
+    // pack: lo nibble = even column (src/quantizer.cpp:33-39); 5-bit primaries one index per byte
+    if (a.primary_bits <= 4) {
+        uint8_t* dst = a.packed_primary + (size_t)row * (a.in >> 1) + (size_t)unit * (U / 2);
+#pragma unroll
+        for (int k = 0; k < U; k += 2) dst[k >> 1] = (uint8_t)((ip[k] & 15u) | ((ip[k + 1] & 15u) << 4));
+    } else {
+        uint8_t* dst = a.packed_primary + elem0;
+#pragma unroll
+        for (int k = 0; k < U; ++k) dst[k] = (uint8_t)ip[k];
+    }
+    uint8_t* dstr = a.packed_residual + (size_t)row * (a.in >> 1) + (size_t)unit * (U / 2);
+#pragma unroll
+    for (int k = 0; k < U; k += 2) dstr[k >> 1] = (uint8_t)((ir[k] & 15u) | ((ir[k + 1] & 15u) << 4));
+}
+
 // corrected_norm = orig / max(||recon||, 1e-10)  (src/quantizer.cpp:237-248)
 __global__ void tq_finish_norms_kernel(const float* __restrict__ orig, const double* __restrict__ partial,
                                        float* __restrict__ norms, int out, int slabs) {
@@ -350,6 +487,14 @@ hipError_t launch_derive_seeds(const float* w, size_t n_floats, uint32_t* seeds_
     return hipGetLastError();
 }
 
+// Partial sums of squares per row that launch_quantize_rows writes (what recon_partial must hold and
+// launch_finish_norms is told): 2048-column slabs, or for blocks of at most 16 columns on widths the lane
+// kernel does not take, units of max(block, 2) columns.
+int quantize_partials_per_row(int in, uint32_t bs) {
+    if (lanes_supported(in, bs)) return (in / kChunk + kWave - 1) / kWave;
+    return in / (int)(bs < 2 ? 2 : bs);
+}
+
 hipError_t launch_quantize_rows(const QuantArgsHost& h, hipStream_t stream) {
     QuantArgs a{};
     a.w = h.w; a.orig_norm = h.orig_norm; a.recon_partial = h.recon_partial; a.scaled_out = h.scaled_out;
@@ -360,6 +505,22 @@ hipError_t launch_quantize_rows(const QuantArgsHost& h, hipStream_t stream) {
     a.bs = h.bs; a.seed_p = h.seed_p; a.seed_r = h.seed_r;
     a.scale_factor = h.scale_factor; a.inv_scale = h.inv_scale; a.inv_sqrt_bs = h.inv_sqrt_bs;
     a.quantize = h.quantize;
+    if (!lanes_supported(h.in, h.bs)) {                 // blocks of 1 to 16 columns, in registers
+        if (!layout_valid(h.in, h.bs) || h.bs > 16) return hipErrorInvalidValue;
+        a.slabs = quantize_partials_per_row(h.in, h.bs);
+        const long long threads = (long long)a.out * a.slabs;
+        const long long g = (threads + 255) / 256;
+        if (g > 0x7fffffffLL) return hipErrorInvalidValue;
+        const dim3 grid((unsigned)g), block(256);
+        switch (h.bs) {
+            case 1: hipLaunchKernelGGL(tq_quantize_small_kernel<1>, grid, block, 0, stream, a); break;
+            case 2: hipLaunchKernelGGL(tq_quantize_small_kernel<2>, grid, block, 0, stream, a); break;
+            case 4: hipLaunchKernelGGL(tq_quantize_small_kernel<4>, grid, block, 0, stream, a); break;
+            case 8: hipLaunchKernelGGL(tq_quantize_small_kernel<8>, grid, block, 0, stream, a); break;
+            default: hipLaunchKernelGGL(tq_quantize_small_kernel<16>, grid, block, 0, stream, a); break;
+        }
+        return hipGetLastError();
+    }
     const long long waves = (long long)a.out * a.slabs;
     const long long grid = (waves + kQWaves - 1) / kQWaves;
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;

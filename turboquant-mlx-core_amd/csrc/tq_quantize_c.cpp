@@ -42,9 +42,11 @@ bool check_shape(int out, int in, uint32_t bs, const char* who) {
     if (bs == 0 || in % (int)bs != 0) {
         set_error(std::string(who) + ": in_features must be divisible by block_size"); return false;
     }
-    if (!tq::lanes_supported(in, bs)) {
-        set_error(std::string(who) + ": unsupported shape (the quantizer needs in_features % 32 == 0 and a "
-                  "power-of-two block_size in [2, 2048])");
+    // (what the layout itself needs; widths that are not a multiple of 32 and blocks of one column run on the
+    // small-block kernel)
+    if (!tq::layout_valid(in, bs) || (!tq::lanes_supported(in, bs) && bs > 16)) {
+        set_error(std::string(who) + ": unsupported shape (need an even in_features and a power-of-two block_size "
+                  "in [1, 2048])");
         return false;
     }
     return true;
@@ -143,7 +145,7 @@ int tq_quantize_weight(const float* weight_dev, int out, int in,
             residual_bits < 0 || residual_bits > 4) {
             set_error("tq_quantize_weight: bad codebook sizes or bit widths"); return 1;
         }
-        const int slabs = (in / tq::kChunk + tq::kWave - 1) / tq::kWave;
+        const int slabs = tq::quantize_partials_per_row(in, block_size);
         DevBuf d_orig, d_partial, d_tables, d_seeds;
         float tables[96];
         fill_tables(cbp, np, cbr, nr, tables);
