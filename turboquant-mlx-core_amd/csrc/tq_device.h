@@ -254,6 +254,22 @@ __device__ __forceinline__ uint16_t float_to_f16_bits(float f) {
     return __builtin_bit_cast(uint16_t, (_Float16)c);
 }
 
+// Two fp32 values -> two fp16 in one register (first value in the low half), round to nearest even, saturating
+// like float_to_f16_bits: the packed conversion turns what lies beyond the largest finite fp16 into an infinity,
+// which becomes the largest finite value again (0x7c00 -> 0x7bff, sign kept); NaN stays NaN.
+__device__ __forceinline__ uint32_t pack_f16_saturating(float lo, float hi) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t p = {lo, hi};
+    const uint32_t h = __builtin_bit_cast(uint32_t, __builtin_convertvector(p, f16x2_t));
+    typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+    const u16x2_t hv = __builtin_bit_cast(u16x2_t, h);
+    const u16x2_t m = __builtin_bit_cast(u16x2_t, (h & 0x7fff7fffu) ^ 0x7c007c00u);   // a half is 0 exactly where it holds an infinity
+    const u16x2_t one = {1, 1}, fifteen = {15, 15};
+    const u16x2_t is_inf = (u16x2_t)(m - one) >> fifteen;             // m <= 0x7fff: only m == 0 wraps to 0xffff (packed 16-bit ops)
+    return __builtin_bit_cast(uint32_t, (u16x2_t)(hv - is_inf));
+}
+
 // Load the 32 consecutive activations a lane owns and widen them to fp32.
 __device__ __forceinline__ void load_chunk(const void* base, int dtype, size_t elem_offset,
                                            float (&v)[kChunk]) {

@@ -397,7 +397,11 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 // Rotate activations [M, K] (f32 / f16 / bf16) -> fp16 tile images: X~ = H (s (.) X) / sqrt(bs) per block,
 // stored as [M/256][K/32] images of 256 rows x 64 bytes in the exact byte order the GEMM keeps
 // them in LDS (16-byte slots permuted by a_slot), so a tile is one contiguous 16 KB copy.
-// One wave per (row, 2048-column slab), 32 consecutive columns per lane, fp32 butterfly.
+// One wave per 64 consecutive 32-column chunks of the row-major input (whole blocks: no half-empty wave at the end
+// of a row), 32 consecutive columns per lane, fp32 butterfly.  (Measured and not kept: 32 rows x 512 columns per
+// workgroup with 1 KB loads and the images written in 1 KB runs through LDS, 21-27 us against 21-26 us for 2048
+// rows of 5120 columns and 10.9 against 8.5 us for 512 rows: the kernel is bound by neither its 64-byte accesses
+// nor, since the signs come from a table, its arithmetic.)
 // PANEL: fragment images for tq_prefill_panel_kernel instead, [M/512][K/16][4 waves][4 row blocks][64 lanes x 16 B]:
 // the 8 columns [16 u + 8 g, +8) of row r sit where lane 32 g + r % 32 of wave (r % 512) / 128 expects the
 // A operand of row block (r % 128) / 32 in sub-step u.
@@ -405,20 +409,32 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 template <bool PANEL>
 __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restrict__ x, int x_dtype,
                                                              uint16_t* __restrict__ out, int rows, int cols,
-                                                             int chunks, int slabs, uint32_t seed, uint32_t bs,
-                                                             float scale) {
-    const int lane = threadIdx.x & 63;
-    const int row = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);     // grid = row quads x slabs
-    const int slab = blockIdx.y;
-    if (row >= rows) return;
-    const int chunk = slab * kWave + lane;
-    const bool active = chunk < chunks;
-    const uint32_t col0 = ((uint32_t)chunk * kChunk) & (bs - 1);
+                                                             int chunks, uint32_t seed, uint32_t bs, float scale) {
+    // The signs of one block as +-1.0f, hashed once per workgroup instead of once per value (the hash is two
+    // 32-bit multiplications per index): entry (32 j + k) at float index 36 j + k, so that the 16-byte reads
+    // of lanes with neighbouring j fall on different banks.
+    __shared__ __align__(16) float signs[64 * 36];
+    const int tid = threadIdx.x;
+    const uint32_t span = bs < 32 ? 32 : bs;                          // (blocks below 32 columns repeat inside a chunk)
+    for (uint32_t i = tid; i < span; i += 256) signs[(i >> 5) * 36 + (i & 31)] = sign_of(seed, i & (bs - 1));
+    __syncthreads();
+
+    // The (row, 32-column chunk) pairs of the whole input in row-major order, 64 to a wave: whole blocks (a row
+    // holds a whole number of them, and 64 chunks are a multiple of every block size up to 2048 columns).
+    const int lane = tid & 63;
+    const long long c = ((long long)blockIdx.x * 4 + (tid >> 6)) * kWave + lane;
+    const bool active = c < (long long)rows * chunks;
+    const int row = active ? (int)(c / chunks) : 0;
+    const int chunk = active ? (int)(c - (long long)row * chunks) : 0;
     float v[kChunk];
     if (active) {
         load_chunk(x, x_dtype, (size_t)row * cols + (size_t)chunk * kChunk, v);
+        const float4* sg = reinterpret_cast<const float4*>(signs + (chunk & (int)((span >> 5) - 1)) * 36);
 #pragma unroll
-        for (int k = 0; k < kChunk; ++k) v[k] *= sign_of(seed, (col0 + k) & (bs - 1));
+        for (int q = 0; q < 8; ++q) {
+            const float4 t = sg[q];
+            v[4 * q] *= t.x; v[4 * q + 1] *= t.y; v[4 * q + 2] *= t.z; v[4 * q + 3] *= t.w;
+        }
     } else {
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) v[k] = 0.0f;
@@ -433,8 +449,7 @@ __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restri
         for (int i = 0; i < 4; ++i) {
             uint32_t w[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                w[j] = (uint32_t)float_to_f16_bits(v[8 * i + 2 * j] * scale) | ((uint32_t)float_to_f16_bits(v[8 * i + 2 * j + 1] * scale) << 16);
+            for (int j = 0; j < 4; ++j) w[j] = pack_f16_saturating(v[8 * i + 2 * j] * scale, v[8 * i + 2 * j + 1] * scale);
             if constexpr (PANEL) pdst[(i >> 1) * 1024 + (i & 1) * 32] = make_uint4(w[0], w[1], w[2], w[3]);
             else dst[a_slot(r, i)] = make_uint4(w[0], w[1], w[2], w[3]);
         }
@@ -530,23 +545,22 @@ hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, i
     const int K = L.in_features, M = batch;
     uint16_t* xt = static_cast<uint16_t*>(workspace);
     const int chunks = K / kChunk;
-    const int slabs = (chunks + kWave - 1) / kWave;
-    const dim3 rgrid((unsigned)((M + 3) / 4), (unsigned)slabs);
+    const dim3 rgrid((unsigned)(((long long)M * chunks + 4 * kWave - 1) / (4 * kWave)));   // 256 chunks per workgroup
     const int tile_m = panel ? kPanelM : kBM;                      // rows of one image
     uint16_t* const xt2 = xt + (size_t)((M + tile_m - 1) / tile_m) * tile_m * K;
     if (panel) {
-        hipLaunchKernelGGL(tq_rotate_f16_kernel<true>, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
+        hipLaunchKernelGGL(tq_rotate_f16_kernel<true>, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks,
                            L.seed_primary, L.block_size, L.inv_sqrt_bs);
         if (L.mode == kDual)
             hipLaunchKernelGGL(tq_rotate_f16_kernel<true>, rgrid, dim3(256), 0, stream, x, x_dtype, xt2, M, K, chunks,
-                               slabs, L.seed_residual, L.block_size, L.inv_sqrt_bs);
+                               L.seed_residual, L.block_size, L.inv_sqrt_bs);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(tq_rotate_f16_kernel<false>, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks, slabs,
+    hipLaunchKernelGGL(tq_rotate_f16_kernel<false>, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks,
                        L.seed_primary, L.block_size, L.inv_sqrt_bs);
     if (L.mode == kDual)
         hipLaunchKernelGGL(tq_rotate_f16_kernel<false>, rgrid, dim3(256), 0, stream, x, x_dtype, xt2, M, K, chunks,
-                           slabs, L.seed_residual, L.block_size, L.inv_sqrt_bs);
+                           L.seed_residual, L.block_size, L.inv_sqrt_bs);
     return hipGetLastError();
 }
 
