@@ -191,11 +191,14 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     const int r_last = r_end > r_begin ? r_end - 1 : r_base;
 
     // The weight plane is read through a buffer descriptor based at the first row of the stream
-    // (offsets inside a stream's rows stay far below 2 GB; the host checks).  Idle runs re-read a
-    // valid address; their rotated activations are 0.
+    // (offsets inside a stream's rows stay far below 2 GB; the host checks).  Idle runs (columns past the row in
+    // its last slab) ask for an offset beyond the descriptor's 2 GB: the hardware returns zeros without touching
+    // memory (with a valid address instead, half a wave re-read the first bytes of its row on every load: 3584-
+    // column rows fetched 9 % more than they hold); their rotated activations are 0.
+    constexpr uint32_t kNoFetch = 0x80000000u;
     const uint8_t* pp = combined ? a.L.packed_combined : (plane ? a.L.packed_residual : a.L.packed_primary);
-    const uint32_t off_p = combined ? (uint32_t)(act_a ? col_a : 0) : (uint32_t)(act_a ? (col_a >> 1) : 0);
-    const uint32_t off_q = (uint32_t)(act_b ? col_b : 0);          // combined plane only (PAIR: same columns, next row)
+    const uint32_t off_p = act_a ? (combined ? (uint32_t)col_a : (uint32_t)(col_a >> 1)) : kNoFetch;
+    const uint32_t off_q = act_b ? (uint32_t)col_b : kNoFetch;      // combined plane only (PAIR: same columns, next row)
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(pp) + (size_t)r_base * row_bytes, 0, 0x7fffffff, 0x00020000);
     const int row_stride = (int)row_bytes;
@@ -216,17 +219,21 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
         gte[buf] = gsrc[rc];
 #pragma unroll
         for (int i = 0; i < R; ++i) {
+            // Rows past the stream's range are requested like the others (the number of loads in flight must not
+            // depend on a branch) but beyond the descriptor: nothing is fetched for them.  (They used to re-read
+            // the range's last row: with 18.5 rows per stream and groups of two, 8 % more bytes than the plane holds.)
             const int ra = PAIR ? r0 + 2 * i : r0 + i;
             const int r = ra < r_last ? ra : r_last;
             const int soff = (r - r_base) * row_stride;
-            P[buf][i] = load_stream16(rs, off_p, soff);
+            const uint32_t vp = ra > r_last ? kNoFetch : off_p;           // wave-uniform condition
+            P[buf][i] = load_stream16(rs, vp, soff);
             if constexpr (PAIR) {
                 const int rq = ra + 1 < r_last ? ra + 1 : r_last;
-                Q[buf][i] = load_stream16(rs, off_q, (rq - r_base) * row_stride);
+                Q[buf][i] = load_stream16(rs, ra + 1 > r_last ? kNoFetch : off_q, (rq - r_base) * row_stride);
             } else if constexpr (BOTH) {
-                Q[buf][i] = load_stream16(rs2, off_p, soff);
+                Q[buf][i] = load_stream16(rs2, vp, soff);
             } else if constexpr (use_res) {
-                Q[buf][i] = load_stream16(rs, off_q, soff);
+                Q[buf][i] = load_stream16(rs, ra > r_last ? kNoFetch : off_q, soff);
             }
         }
     };
