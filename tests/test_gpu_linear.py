@@ -353,11 +353,11 @@ def test_prefill_panel_kernel_matches_dequant_matmul(tq, oracle, mode, out, inf,
 
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("out,inf,bs,batch,ydt", [(8448, 2048, 512, 2000, "f32"),    # 4 x 66 tiles: 8 left after one round of 256
-                                                  (8400, 2304, 256, 1600, "bf16"),   # ragged last tile, 144 sub-steps in 4 parts
+                                                  (8400, 2304, 256, 1600, "bf16"),   # ragged last tile, 144 sub-steps in parts of 32 (the last one 16)
                                                   (16500, 2048, 128, 1025, "f16")])  # 3 x 129 tiles: 131 left after one round -> 1 part, whole
 def test_prefill_panel_kernel_tail_tiles_in_k_ranges(tq, oracle, mode, out, inf, bs, batch, ydt):
-    """Tiles left over after the last full round of the chip (at most half a round of them, rows of 2048 columns
-    or more) are cut into 2..4 K ranges (dual rotation: one per plane) whose fp32 products a second kernel adds:
+    """Tiles left over after the last full round of the chip are cut into K ranges (dual rotation: one part per
+    plane and range) where that is cheaper by the library's count of rounds; a second kernel adds their fp32 products:
     sampled rows of every panel against the oracle, in particular rows of the last panel, whose last tiles are
     the ones that are cut."""
     qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf + batch)
@@ -379,6 +379,40 @@ def test_prefill_panel_kernel_tail_tiles_in_k_ranges(tq, oracle, mode, out, inf,
         assert _rel(y[rows][:, c0:c0 + 128], want[:, c0:c0 + 128]) < tol
     y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)
     assert _rel(y[batch - 1:batch], y1) < tol
+    layer.close()
+
+
+@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
+@pytest.mark.parametrize("out,inf,bs,batch,ydt", [(5100, 8192, 256, 2048, "f32"),   # 160 tiles, each in 3 ranges: two rounds of parts
+                                                  (4400, 9216, 128, 2048, "f16"),   # 140 tiles, 576 sub-steps in 3 ranges, ragged last tile
+                                                  (5000, 8192, 512, 1600, "bf16")])  # 160 tiles, the last panel 64 rows
+def test_prefill_panel_kernel_less_than_a_round_all_tiles_cut_along_k(tq, oracle, mode, out, inf, bs, batch, ydt):
+    """Calls with fewer 512 x 128 tiles than the chip has CUs (but more than half as many) and long rows: every
+    tile is cut into K ranges (dual rotation: one part per plane and range, here two ranges) so that the parts
+    fill the chip; more parts than CUs run in rounds, and the sum kernel adds them.  Sampled rows of every panel
+    against the oracle."""
+    qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf + batch)
+    x32 = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
+    xbits = oracle.f32_to_bf16_bits(x32)
+    last = (batch - 1) // 512 * 512
+    rows = sorted(r for r in {0, 127, 128, 255, 256, 511, 512, last, (last + batch) // 2, batch - 1} if 0 <= r < batch)
+    want = oracle.linear_forward(qw, cb, cb, bs, oracle.bf16_bits_to_f32(xbits[rows]))
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    code = {"f32": tq.F32, "bf16": tq.BF16, "f16": tq.F16}[ydt]
+    y = layer.forward(xbits, tq.BF16, code)
+    y = oracle.bf16_bits_to_f32(y) if ydt == "bf16" else y.astype(np.float32)
+    assert y.shape == (batch, out) and np.isfinite(y).all()
+    tol = 5e-3 if ydt == "bf16" else 1e-3
+    assert _rel(y[rows], want) < tol
+    for k, r in enumerate(rows):
+        assert _rel(y[r:r + 1], want[k:k + 1]) < tol
+    for c0 in range(0, out, 128):                            # every tile of weights
+        assert _rel(y[rows][:, c0:c0 + 128], want[:, c0:c0 + 128]) < tol
+    y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)
+    assert _rel(y[batch - 1:batch], y1) < tol
+    y2 = layer.forward(xbits, tq.BF16, code)                 # the parts are added in a fixed order
+    y2 = oracle.bf16_bits_to_f32(y2) if ydt == "bf16" else y2.astype(np.float32)
+    assert np.array_equal(y, y2)
     layer.close()
 
 

@@ -456,6 +456,105 @@ __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restri
     }
 }
 
+// Fragment images for blocks of at most 512 columns, the whole call in one launch: a wave takes R consecutive rows
+// of one 512-column segment, 8 columns per lane, so a load instruction reads 1 KB of one row (the kernel above
+// reads 64 bytes per lane with the lanes 64 bytes apart: every line passes through the CU's cache four times, and
+// 2048 rows of 27648 columns took 132 us against 72-99 us here).  R = 8: the 8 rows of a lane's 8 columns are 128
+// consecutive bytes of the image (rows r % 32 = 8 j .. 8 j + 7 of lane group g); they change lanes through a
+// wave-private piece of LDS so that a store instruction writes eight whole 128-byte lines.  R = 2, for calls
+// with few rows (less than two waves of 8 rows per SIMD): the launch is as long as one wave's chain of loads,
+// butterflies and stores, so the waves are kept short and store their 2 x 16 bytes themselves.
+// planes = 2: both rotations of the dual layout from one read of the activations (images out and out2).
+constexpr int kRotPitch = 144;                 // bytes of a lane's 8 x 16 B in LDS, padded: 16-byte accesses spread over the banks
+template <int R>
+__global__ __launch_bounds__(256) void tq_rotate_panel_kernel(const void* __restrict__ x, int x_dtype,
+                                                               uint16_t* __restrict__ out, uint16_t* __restrict__ out2,
+                                                               int rows, int cols, int segs, int planes,
+                                                               uint32_t seed, uint32_t seed2, uint32_t bs, float scale) {
+    __shared__ __align__(16) char stage_all[R == 8 ? 4 * kWave * kRotPitch : 16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    char* const stage = stage_all + (R == 8 ? wave * (kWave * kRotPitch) : 0);
+    const long long task = (long long)blockIdx.x * 4 + wave;           // (row group, segment), segment fastest
+    const int rg = (int)(task / segs), seg = (int)(task - (long long)rg * segs);
+    const int row0 = rg * R;
+    if (row0 >= rows) return;                                          // wave-uniform; no workgroup barrier below
+    const int col = seg * 512 + lane * 8;
+    const bool active = col < cols;                                    // (the last segment of a width that is no multiple of 512)
+
+    uint4 raw[R][2];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row = row0 + r < rows ? row0 + r : rows - 1;
+        const size_t e = (size_t)row * cols + (active ? col : 0);
+        if (x_dtype == kF32) {
+            const uint4* p = reinterpret_cast<const uint4*>(static_cast<const float*>(x) + e);
+            raw[r][0] = p[0]; raw[r][1] = p[1];
+        } else {
+            raw[r][0] = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + e);
+        }
+    }
+    const int U_all = cols >> 4;
+    const int g_own = seg * 64 + lane;                                 // this lane's 8-column group of the row
+    for (int plane = 0; plane < planes; ++plane) {
+        const uint32_t sd = plane ? seed2 : seed;
+        uint4* const img = reinterpret_cast<uint4*>(plane ? out2 : out);
+        float sg[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sg[j] = active ? sign_of(sd, (uint32_t)(col + j) & (bs - 1)) : 0.0f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float v[8];
+            if (x_dtype == kF32) {
+                const uint32_t w[8] = {raw[r][0].x, raw[r][0].y, raw[r][0].z, raw[r][0].w, raw[r][1].x, raw[r][1].y, raw[r][1].z, raw[r][1].w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = __builtin_bit_cast(float, w[j]);
+            } else {
+                const uint32_t w[4] = {raw[r][0].x, raw[r][0].y, raw[r][0].z, raw[r][0].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (x_dtype == kBF16) {
+                        v[2 * j] = bf16_bits_to_float(w[j] & 0xffffu);
+                        v[2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+                    } else {
+                        v[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] & 0xffffu));
+                        v[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] >> 16));
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] *= sg[j];
+            fwht_lanes<8>(v, bs, lane);
+            uint4 o;
+            o.x = pack_f16_saturating(v[0] * scale, v[1] * scale); o.y = pack_f16_saturating(v[2] * scale, v[3] * scale);
+            o.z = pack_f16_saturating(v[4] * scale, v[5] * scale); o.w = pack_f16_saturating(v[6] * scale, v[7] * scale);
+            if constexpr (R == 8) {
+                *reinterpret_cast<uint4*>(stage + lane * kRotPitch + r * 16) = o;
+            } else {
+                const int row = row0 + r;
+                if (active)
+                    img[((size_t)(row >> 9) * U_all + (g_own >> 1)) * 1024 + (size_t)(((row >> 7) & 3) * 4 + ((row >> 5) & 3)) * 64 +
+                        (row & 31) + (g_own & 1) * 32] = o;
+            }
+        }
+        if constexpr (R == 8) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            // Store instruction i: lane -> (column group 8 i + lane / 8, row lane % 8): eight lanes write one line.
+            const int r = lane & 7, row = row0 + r;
+            const size_t row_unit = (size_t)(((row >> 7) & 3) * 4 + ((row >> 5) & 3)) * 64 + (row & 31);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int g_in_seg = 8 * i + (lane >> 3);
+                const uint4 o = *reinterpret_cast<const uint4*>(stage + g_in_seg * kRotPitch + r * 16);
+                const int g = seg * 64 + g_in_seg;                      // 8-column group of the row
+                if (g * 8 < cols)
+                    img[((size_t)(row >> 9) * U_all + (g >> 1)) * 1024 + row_unit + (g & 1) * 32] = o;
+            }
+            __builtin_amdgcn_wave_barrier();                           // (the next plane writes the piece again)
+        }
+    }
+}
+
 // Sum of the K ranges: y[m, n] = out_scale * norm[n] * (partial[0][m, n] + partial[1][m, n] + ...), ranges added
 // in their order.  One thread per four neighbouring outputs (QUAD: N is a multiple of 4) or per output.
 template <bool QUAD>
@@ -548,6 +647,20 @@ hipError_t launch_rotate_tiles(const LayerView& L, const void* x, int x_dtype, i
     const dim3 rgrid((unsigned)(((long long)M * chunks + 4 * kWave - 1) / (4 * kWave)));   // 256 chunks per workgroup
     const int tile_m = panel ? kPanelM : kBM;                      // rows of one image
     uint16_t* const xt2 = xt + (size_t)((M + tile_m - 1) / tile_m) * tile_m * K;
+    if (panel && L.block_size <= 512) {
+        const int segs = (K + 511) / 512;
+        const int planes = L.mode == kDual ? 2 : 1;
+        const long long tasks8 = (long long)((M + 7) / 8) * segs;
+        if (tasks8 >= 2048) {
+            hipLaunchKernelGGL(tq_rotate_panel_kernel<8>, dim3((unsigned)((tasks8 + 3) / 4)), dim3(256), 0, stream, x, x_dtype,
+                               xt, xt2, M, K, segs, planes, L.seed_primary, L.seed_residual, L.block_size, L.inv_sqrt_bs);
+        } else {
+            const long long tasks2 = (long long)((M + 1) / 2) * segs;
+            hipLaunchKernelGGL(tq_rotate_panel_kernel<2>, dim3((unsigned)((tasks2 + 3) / 4)), dim3(256), 0, stream, x, x_dtype,
+                               xt, xt2, M, K, segs, planes, L.seed_primary, L.seed_residual, L.block_size, L.inv_sqrt_bs);
+        }
+        return hipGetLastError();
+    }
     if (panel) {
         hipLaunchKernelGGL(tq_rotate_f16_kernel<true>, rgrid, dim3(256), 0, stream, x, x_dtype, xt, M, K, chunks,
                            L.seed_primary, L.block_size, L.inv_sqrt_bs);

@@ -63,10 +63,11 @@ struct PanelArgs {
     int M, N, K;
     int panels, n_tiles, n_per_xcd;
     float out_scale;
-    // The last `tail_tiles` tiles (in panel-major order) do not fill a round of the chip: each is cut into `parts`
-    // K ranges of part_subs sub-steps (dual rotation: two parts, one per plane), run by the workgroups
-    // [first_part_wg, first_part_wg + tail_tiles * parts) of the grid, which write their raw fp32 products to
-    // partial[(tile, part)][512][128]; tq_prefill_panel_sum_kernel adds the parts.  tail_tiles == 0: no such tiles.
+    // The last `tail_tiles` tiles (in panel-major order; all tiles where the call has fewer tiles than the chip has
+    // CUs) are cut into `parts` parts: K ranges of part_subs sub-steps, with the dual rotation one per (plane, K
+    // range), plane = part & 1.  They are run by the workgroups [first_part_wg, first_part_wg + tail_tiles * parts),
+    // which write their raw fp32 products to partial[(tile, part)][512][128]; tq_prefill_panel_sum_kernel adds the
+    // parts.  tail_tiles == 0: no such tiles.
     int tail_tiles, parts, part_subs, first_part_wg;
     float* partial;
 };
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
     constexpr int kPlanes = (MODE == kDual) ? 2 : 1;
     const int U_all = a.K / kSubK;                         // sub-steps of a row (a multiple of kUnroll)
     const int id = blockIdx.x;
-    int panel, n_tile, part = -1;
+    int panel, n_tile, part = -1, part_slot = 0;            // part_slot: index of the part's fp32 product
     int u_begin = 0, u_end = U_all, plane_begin = 0, plane_end = kPlanes;
     if (id < a.first_part_wg) {
         const int xcd = id & 7, slot = id >> 3;
@@ -107,18 +108,26 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
         if (n_tile >= a.n_tiles) return;                   // whole workgroup leaves together
         if (panel * a.n_tiles + n_tile >= a.panels * a.n_tiles - a.tail_tiles) return;     // a tail tile: run in parts
     } else {
-        const int k = id - a.first_part_wg;
-        const int t = a.panels * a.n_tiles - a.tail_tiles + k / a.parts;
-        part = k - (k / a.parts) * a.parts;
+        // Workgroup ids go round the XCDs: XCD x takes the x-th eighth of the (part, tile) pairs in part-major
+        // order, so that the workgroups it runs side by side walk the same K range of the same panel and its L2
+        // fetches that range of the activations once.
+        const int k0 = id - a.first_part_wg, units = a.tail_tiles * a.parts;
+        const int x = k0 & 7, per = units >> 3, extra = units & 7;
+        const int k = x * per + (x < extra ? x : extra) + (k0 >> 3);
+        part = k / a.tail_tiles;
+        const int part_tile = k - part * a.tail_tiles;
+        part_slot = part_tile * a.parts + part;
+        const int t = a.panels * a.n_tiles - a.tail_tiles + part_tile;
         panel = t / a.n_tiles;
         n_tile = t - panel * a.n_tiles;
+        int range = part;
         if constexpr (MODE == kDual) {
-            plane_begin = part;
-            plane_end = part + 1;
-        } else {
-            u_begin = part * a.part_subs;
-            u_end = u_begin + a.part_subs < U_all ? u_begin + a.part_subs : U_all;
+            plane_begin = part & 1;
+            plane_end = plane_begin + 1;
+            range = part >> 1;
         }
+        u_begin = range * a.part_subs;
+        u_end = u_begin + a.part_subs < U_all ? u_begin + a.part_subs : U_all;
     }
     const int m0 = panel * kPanelM, n0 = n_tile * kPN;
     const int tiles_end = u_end / 4;                       // 64-column weight tiles end here
@@ -385,7 +394,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
         return;
     }
     const bool is_part = part >= 0;
-    void* const y_out = is_part ? static_cast<void*>(a.partial + (size_t)(id - a.first_part_wg) * (kPanelM * kPN)) : a.y;
+    void* const y_out = is_part ? static_cast<void*>(a.partial + (size_t)part_slot * (kPanelM * kPN)) : a.y;
     const int y_type = is_part ? (int)kF32 : a.y_dtype;
     const int yN = is_part ? kPN : a.N, yM = is_part ? kPanelM : a.M;          // row pitch / row limit of y_out
     const int col0 = (is_part ? 0 : n0) + (lane >> 5) * 4;
@@ -547,6 +556,7 @@ __global__ __launch_bounds__(256) void tq_prefill_panel_sum_kernel(PanelArgs a) 
         if (row >= a.M || col >= a.N) continue;
         const float* src = a.partial + ((size_t)tile_k * a.parts) * (kPanelM * kPN) + (size_t)(r + rr) * kPN + c4;
         float4 s = *reinterpret_cast<const float4*>(src);
+#pragma unroll 4
         for (int k = 1; k < a.parts; ++k) {
             const float4 v = *reinterpret_cast<const float4*>(src + (size_t)k * (kPanelM * kPN));
             s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
@@ -561,29 +571,45 @@ __global__ __launch_bounds__(256) void tq_prefill_panel_sum_kernel(PanelArgs a) 
 namespace {
 
 // How a call is cut: all tiles whole (tail_tiles == 0), or the tiles that are left after the last full round of
-// the chip in `parts` K ranges each.  Worth it where those tiles are at most half a round (two parts or more fit
-// on the CUs) and long enough to pay for the hand-over through memory; the fp32 parts follow the fragment images
-// in the workspace.
+// the chip (every tile, where the call has fewer tiles than the chip has CUs) in `parts` parts each; the fp32
+// parts follow the fragment images in the workspace.  The cut is the cheapest by a count in sub-steps of one
+// workgroup: rounds of whole tiles and of parts on the CUs, a fixed cost per workgroup (table, first requests,
+// epilogue), and the hand-over of the parts through memory.
 struct PanelPlan { int tail_tiles, parts, part_subs; size_t xt_bytes, total_bytes; };
+
+constexpr double kWorkgroupCost = 20.0;        // prologue + epilogue of a workgroup, in sub-steps (0.4 us each)
+constexpr double kSumFixedCost = 5.0;          // the launch of the sum kernel
+constexpr double kSumCostPerPart = 0.19;       // 256 KB written and read again, at the rate the sum kernel reaches
+constexpr size_t kMaxPartBytes = (size_t)512 << 20;
+
 
 PanelPlan panel_plan(const LayerView& L, int batch, int num_cus, size_t capacity) {
     PanelPlan p{};
-    const size_t planes = (L.mode == kDual) ? 2 : 1;
+    const int planes = (L.mode == kDual) ? 2 : 1;
     const size_t panels = ((size_t)batch + kPanelM - 1) / kPanelM;     // whole fragment images
-    p.xt_bytes = (planes * panels * kPanelM * L.in_features * sizeof(uint16_t) + 255) & ~(size_t)255;
+    p.xt_bytes = ((size_t)planes * panels * kPanelM * L.in_features * sizeof(uint16_t) + 255) & ~(size_t)255;
     p.total_bytes = p.xt_bytes;
     const long long tiles = (long long)panels * ((L.out_features + kPN - 1) / kPN);
     const int subs = L.in_features / kSubK;
-    const int tail = (int)(tiles % num_cus);
-    if (tiles < num_cus || tail == 0 || tail * 2 > num_cus || L.in_features < 2048) return p;
-    int parts = num_cus / tail;
-    if (parts > 4) parts = 4;
-    if (L.mode == kDual) parts = 2;                                    // one part per plane
-    int per = ((subs + parts - 1) / parts + kUnroll - 1) / kUnroll * kUnroll;
-    if (L.mode != kDual) parts = (subs + per - 1) / per;
-    const size_t need = p.xt_bytes + (size_t)tail * parts * kPanelM * kPN * sizeof(float);
-    if (parts < 2 || need > capacity) return p;
-    p.tail_tiles = tail; p.parts = parts; p.part_subs = per; p.total_bytes = need;
+    const long long cut = tiles < num_cus ? tiles : tiles % num_cus;   // tiles that would be cut
+    if (cut == 0) return p;
+    const double whole = (double)subs * planes + kWorkgroupCost;
+    double best = 0.97 * (double)((tiles + num_cus - 1) / num_cus) * whole;        // (of no cut at all)
+    for (int ranges = 1; ranges <= 8; ++ranges) {
+        const int per = ((subs + ranges - 1) / ranges + kUnroll - 1) / kUnroll * kUnroll;
+        const int parts = (subs + per - 1) / per * planes;
+        if (parts < 2 || (ranges > 1 && (subs + per - 1) / per != ranges)) continue;
+        const long long units = cut * parts;
+        const size_t bytes = (size_t)units * kPanelM * kPN * sizeof(float);
+        if (bytes > kMaxPartBytes || p.xt_bytes + bytes > capacity) continue;
+        const double cost = (double)((tiles - cut) / num_cus) * whole +
+                            (double)((units + num_cus - 1) / num_cus) * (per + kWorkgroupCost) +
+                            kSumFixedCost + kSumCostPerPart * (double)units;
+        if (cost < best) {
+            best = cost;
+            p.tail_tiles = (int)cut; p.parts = parts; p.part_subs = per; p.total_bytes = p.xt_bytes + bytes;
+        }
+    }
     return p;
 }
 
@@ -594,8 +620,10 @@ size_t prefill_panel_workspace_bytes(const LayerView& L, int batch, int num_cus,
 }
 
 // More than 256 rows (up to 256 the 256-row tiles of the other kernel multiply half as many padding rows), a
-// width that fills the unrolled loop, and enough 512 x 128 tiles for the chip (with few tiles the other kernel
-// cuts K into ranges).
+// width that fills the unrolled loop, and 512 x 128 tiles for more than half the CUs.  (With fewer tiles the other
+// kernel, which cuts K with 256 x 256 tiles, is as fast or faster even when every tile here is cut along K so
+// that the parts fill the chip: 512 and 1024 rows of 3584 x 18944, 4096 x 14336 and 8192 x 8192 took 4-12 % longer
+// that way, 5120 x 27648 the same at 512 rows and 4 % less at 1024.)
 bool prefill_panel_supported(const LayerView& L, int batch, int num_cus) {
     if (batch <= 256) return false;
     if (L.mode != kSharedLut && L.mode != kDual && L.mode != kPrimaryOnly) return false;
@@ -627,7 +655,8 @@ hipError_t launch_prefill_panel(const LayerView& L, const void* x, int x_dtype, 
     a.n_per_xcd = (a.n_tiles + 7) / 8;
     a.out_scale = L.inv_scale;
     a.tail_tiles = plan.tail_tiles; a.parts = plan.parts; a.part_subs = plan.part_subs;
-    a.first_part_wg = 8 * a.n_per_xcd * a.panels;
+    // (all tiles cut: no workgroups for whole tiles)
+    a.first_part_wg = plan.tail_tiles == a.panels * a.n_tiles ? 0 : 8 * a.n_per_xcd * a.panels;
     a.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + plan.xt_bytes);
     const dim3 grid((unsigned)(a.first_part_wg + a.tail_tiles * a.parts));
     switch (L.mode) {
