@@ -465,6 +465,9 @@ __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restri
 // with few rows (less than two waves of 8 rows per SIMD): the launch is as long as one wave's chain of loads,
 // butterflies and stores, so the waves are kept short and store their 2 x 16 bytes themselves.
 // planes = 2: both rotations of the dual layout from one read of the activations (images out and out2).
+// (The same kernel writing the 256-row tile images of tq_prefill_gemm_kernel was measured and not kept: there a lane of
+// tq_rotate_f16_kernel already stores the 64 contiguous bytes of its chunk; 512 x 27648 took 25.5 us instead of 19.8,
+// 1024 x 5120 9.4 instead of 10.0.)
 constexpr int kRotPitch = 144;                 // bytes of a lane's 8 x 16 B in LDS, padded: 16-byte accesses spread over the banks
 template <int R>
 __global__ __launch_bounds__(256) void tq_rotate_panel_kernel(const void* __restrict__ x, int x_dtype,
