@@ -140,7 +140,7 @@ def test_forward_fp32(tq, oracle, mode, out, inf, bs, batch):
                                         (130, 16384, 512), (3, 5120, 512), (2049, 12288, 64)])
 def test_forward_batch1_wide_rows(tq, oracle, mode, out, inf, bs):
     """One activation row on rows of 3 to 8 slabs (and, shared rotation, of an odd number of
-    1024-column halves, which are served two rows at a time; dual rotation up to 4 slabs, the waves
+    1024-column halves, which are served two rows at a time; dual rotation with the waves
     of a row split by plane): the one-workgroup-per-CU kernel.
     Row counts are chosen so that streams get ragged, empty and single-row ranges; fp32 and bf16
     activations; every output against the oracle within the fp32 tolerance."""

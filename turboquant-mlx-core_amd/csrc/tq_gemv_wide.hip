@@ -54,7 +54,8 @@ __device__ unsigned long long g_timeline[256 * 16 * 16];
 namespace {
 
 constexpr int kMaxImageCols = 16384;             // widest rotated-activation image in LDS (64 KB)
-constexpr int kPairDualSlabs = 3;                // dual rotation with byte-pair tables: 2 x 64 KB of tables leave 24 KB
+constexpr int kPairDualSlabs = 8;                // dual rotation with byte-pair tables: rows of up to 8 slabs
+constexpr int kTwoImageSlabs = 5;                // ... of which up to 5 keep an image per rotation side by side (80 KB)
 
 // Marks a loaded value as consumed here.  A load whose result is only read on some paths stays
 // "possibly in flight" for the compiler on the others, and it then waits for it (and, as loads
@@ -144,7 +145,8 @@ template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, boo
 __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     static_assert(!BOTH || (MODE == kDual && PT && (DYN != PRE) && !PAIR && R <= 2), "both planes per wave: dual rotation, pair tables");
     static_assert(!PT || MODE != kSharedLut, "pair tables serve the nibble planes");
-    constexpr int kRegion = (PT && MODE == kDual) ? 2 * kLut256Bytes : kRegionBytes;   // decode tables
+    constexpr int kRegion = kRegionBytes;           // decode tables
+    constexpr bool kTwoPlaneTable = PT && MODE == kDual;    // both planes' byte-pair tables in one region (below)
     static_assert(!PRE || (!PAIR && !DYN && (MODE != kDual || BOTH) && TILES == 1), "pre-rotated rows: plain slab streams");
     static_assert(!PAIR || MODE == kSharedLut, "row pairs need the one-byte-per-weight plane");
     static_assert(!DYN || (!PAIR && (MODE != kDual || BOTH)), "the group counter serves one-wave row streams");
@@ -154,7 +156,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     // tables | cross-wave partial sums | activation image.  A static array: its address is a constant
     // the compiler folds into the LDS instructions (with a dynamic one every table read carried an
     // address addition of its own, a third of the vector instructions of the decode).
-    constexpr int kImageBytes = PRE ? 0 : ((PT && MODE == kDual) ? kPairDualSlabs * kSlab : kMaxImageCols) * (int)sizeof(float);
+    constexpr int kImageBytes = PRE ? 0 : (kTwoPlaneTable ? 2 * kTwoImageSlabs * kSlab : kMaxImageCols) * (int)sizeof(float);
     __shared__ __align__(16) char smem[kRegion + kPartialBytes + kImageBytes];
     float* partial = reinterpret_cast<float*>(smem + kRegion);   // [2][waves][V]
 
@@ -173,11 +175,14 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     const int col_a = PAIR ? slab * (kSlab / 2) + 16 * lane : slab * kSlab + (combined ? 16 * lane : 32 * lane);
     const int col_b = PAIR ? col_a : (combined ? col_a + 1024 : col_a + 16);
     const bool act_a = col_a < a.L.in_features, act_b = col_b < a.L.in_features;
-    const uint32_t laneoff = (uint32_t)lane << 2;
-    [[maybe_unused]] const uint32_t laneoff_plane = laneoff | ((uint32_t)plane << 16);   // kLut256Bytes = 1 << 16
+    // Table entries are 256 bytes apart and a lane reads its own 4-byte column of an entry.  One table: 64 columns.
+    // Byte-pair tables of both planes: an entry holds 32 columns of the primary plane's value, then 32 of the
+    // residual plane's; lanes l and l + 32 share a column (the LDS serves a wave's 32-bit reads in two halves of
+    // 32 lanes, so they never meet), and both tables take the 64 KB that one took.
+    const uint32_t laneoff = kTwoPlaneTable ? (uint32_t)(lane & 31) << 2 : (uint32_t)lane << 2;
+    [[maybe_unused]] const uint32_t laneoff_plane = kTwoPlaneTable ? laneoff | ((uint32_t)plane << 7) : laneoff;
     [[maybe_unused]] const uint32_t table_bits = plane ? 0x10101010u : 0u;               // 16-entry tables: kTab16Bytes = 16 entries
-    [[maybe_unused]] const uint32_t laneoff_res = laneoff | (1u << 16);                   // BOTH: the residual plane's table
-    static_assert(kLut256Bytes == (1 << 16), "the table number sits in bits 16.. of a table address");
+    [[maybe_unused]] const uint32_t laneoff_res = laneoff | 128u;                        // BOTH: the residual plane's columns
     const int out = a.L.out_features;
     const size_t row_bytes = combined ? (size_t)a.L.in_features : ((size_t)a.L.in_features >> 1);
     constexpr bool use_res = (MODE == kSharedLut) || BOTH;  // second 16-byte load per row
@@ -242,7 +247,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     // tiles, then the weights.  (Every vector memory instruction of a wave occupies the CU's
     // address unit for 16 cycles, and 16 waves share it: the table values, which are the same for
     // all lanes, come through scalar loads instead.)
-    constexpr int kEntries = PT ? (MODE == kDual ? 512 : 256) : (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
+    constexpr int kEntries = PT ? 256 : (MODE == kSharedLut) ? 256 : (MODE == kDual ? 32 : 16);
     // Wave w writes table entries 16 w .. 16 w + 15 (then 16 (w + nwaves) ..); the first 16 values
     // are requested here.
     typedef const __attribute__((address_space(4))) float cfloat;     // uniform address: scalar load
@@ -291,14 +296,28 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     if (DYN && tid == 0) *next_group = 2 * nwaves;              // (groups w and w + nwaves are wave w's first two)
     if constexpr (PT) {
         // Entry e of a plane's table: fp16 centroid of nibble e & 15 in the low half, of nibble e >> 4
-        // in the high half.  Chunk c = 16 entries with the same high nibble; chunks 16.. are plane 1.
+        // in the high half.  Chunk c = 16 entries with the same high nibble.  Both planes: lanes 0..31 write
+        // the primary plane's columns, lanes 32..63 the residual plane's (16 table values further on).
         uint32_t* const dst = reinterpret_cast<uint32_t*>(smem) + lane;
+        const bool second = kTwoPlaneTable && lane >= 32;
+        // (both planes' entries are made from scalar loads and chosen per lane afterwards: a choice between the
+        // two addresses instead becomes a vector load, which queues behind the weight requests above)
+        auto pair_entry = [&](int base, int c, int e) {
+            const uint32_t h = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)tab[base + c]);
+            const uint32_t l = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)tab[base + e]);
+            return (uint32_t)__builtin_amdgcn_readfirstlane((int)((h << 16) | l));
+        };
         for (int c = wave; c * 16 < kEntries; c += nwaves) {
-            const int pl = c >> 4;
-            const uint32_t hi = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)tab[16 * pl + (c & 15)]) << 16;
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
-                dst[(c * 16 + e) * kWave] = hi | (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)tab[16 * pl + e]);
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t u0 = pair_entry(0, c, e);
+                if constexpr (kTwoPlaneTable) {
+                    const uint32_t u1 = pair_entry(16, c, e);
+                    dst[(c * 16 + e) * kWave] = second ? u1 : u0;
+                } else {
+                    dst[(c * 16 + e) * kWave] = u0;
+                }
+            }
         }
     } else {
         // Lane l stores each entry's value into its own column, 4 l bytes into the entry's 256.
@@ -327,12 +346,27 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
     float* const image = reinterpret_cast<float*>(smem + kRegion + kPartialBytes);
     rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_primary, a.L.block_size, image, wave,
                                      nwaves, lane);
+    // (byte-pair tables of both planes leave room for a second image of rows up to 5 slabs wide: both rotations
+    // before the one barrier)
+    [[maybe_unused]] float* const image2 = image + a.img_cols;
+    const bool two_images = kTwoPlaneTable && a.img_cols <= kTwoImageSlabs * kSlab;      // uniform over the launch
+    if (two_images)
+        rotate_to_image<combined, TILES>(raw, a.x_dtype, a.L.in_features, a.L.seed_residual, a.L.block_size, image2,
+                                         wave, nwaves, lane);
     TQ_MARK(3);
     __syncthreads();                  // image and tables (and the group counter) visible to every wave
     TQ_MARK(4);
     // The second stage of the ring is requested behind the barrier: a wave whose requests queue up
     // in the memory pipeline would otherwise keep the whole workgroup waiting there.
     fetch(1, DYN ? r_begin + (wave + nwaves) * V : r_begin + V);
+    if (two_images) {
+        if constexpr (BOTH) {
+            take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xt);
+            take_from_image<PAIR, NX>(image2, lane, slab, act_a, act_b, xr);
+        } else {
+            take_from_image<PAIR, NX>(plane ? image2 : image, lane, slab, act_a, act_b, xt);
+        }
+    } else {
     if (plane == 0) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xt);
     if constexpr (MODE == kDual) {
         __syncthreads();                                      // everyone has read the first rotation
@@ -341,6 +375,7 @@ __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
         __syncthreads();
         if constexpr (BOTH) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xr);
         else if (plane == 1) take_from_image<PAIR, NX>(image, lane, slab, act_a, act_b, xt);
+    }
     }
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { consumed(raw[t].a); consumed(raw[t].b); }
