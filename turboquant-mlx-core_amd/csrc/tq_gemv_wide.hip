@@ -143,7 +143,7 @@ __device__ __forceinline__ void take_from_image(const float* image, int lane, in
 // their rows from the LDS counter like the other one-slab layers.
 template <int MODE, int R, int TILES, bool PAIR, bool DYN, bool PRE = false, bool PT = false, bool BOTH = false>
 __device__ __forceinline__ void wide_body(const GemvArgs& a, const int block) {
-    static_assert(!BOTH || (MODE == kDual && PT && (DYN != PRE) && !PAIR && R <= 2), "both planes per wave: dual rotation, pair tables");
+    static_assert(!BOTH || (MODE == kDual && PT && !(DYN && PRE) && !PAIR && R <= 2), "both planes per wave: dual rotation, pair tables");
     static_assert(!PT || MODE != kSharedLut, "pair tables serve the nibble planes");
     constexpr int kRegion = kRegionBytes;           // decode tables
     constexpr bool kTwoPlaneTable = PT && MODE == kDual;    // both planes' byte-pair tables in one region (below)
@@ -569,17 +569,26 @@ struct GemvGroup {
     GemvArgs a[3];
     int first[4];          // layer j owns workgroups first[j] .. first[j + 1] - 1
 };
-template <int MODE, int R, bool PAIR, bool PT>
+template <int MODE, int R, bool PAIR, bool PT, bool BOTH = false>
 __global__ __launch_bounds__(1024) void tq_gemv_wide_group_kernel(GemvGroup g) {
     const int b = (int)blockIdx.x;
     const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
-    wide_body<MODE, R, 1, PAIR, false, false, PT>(g.a[j], b - g.first[j]);
+    wide_body<MODE, R, 1, PAIR, false, false, PT, BOTH>(g.a[j], b - g.first[j]);
 }
 
 template <int MODE, int R, int TILES, bool PAIR, bool DYN = false, bool PRE = false, bool PT = false, bool BOTH = false>
 hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t stream) {
     hipLaunchKernelGGL((tq_gemv_wide_kernel<MODE, R, TILES, PAIR, DYN, PRE, PT, BOTH>), dim3(grid), dim3(threads), 0, stream, a);
     return hipGetLastError();
+}
+
+// Dual rotation on pair tables, rows of 3 to 5 slabs: one wave per slab that decodes both planes (two images of
+// the row, one per rotation) instead of a wave per (slab, plane).  Measured, eager launches on one box, both
+// planes per wave against one: 10240 x 10240 27.0 against 29.5 us, 27648 x 5120 32.8 / 33.9; rows of two slabs:
+// 18944 x 3584 18.8 / 19.0-20.0, 8192 x 8192 equal, 4096 x 4096 8.8 / 8.5: they stay with a wave per plane.  (A
+// property of the layer's width alone: a grouped launch must take the kernel a launch of its own would.)
+bool wants_both_planes(int slabs, bool fp16_ok) {
+    return fp16_ok && slabs >= 3 && slabs <= kTwoImageSlabs;
 }
 
 // Row pairs are used where the width is an odd number of 1024-column halves.
@@ -616,7 +625,8 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
     if (PAIR) a.W = a.L.in_features / (kSlab / 2);           // halves per row
     // Dual rotation: (slab, plane) pairs per row; rows of one slab whose centroids fit fp16 keep both
     // planes in one wave instead.
-    const bool both = MODE == kDual && (slabs == 1 || a.pre_rotated) && a.L.fp16_centroids_ok;
+    const bool both = MODE == kDual && a.L.fp16_centroids_ok &&
+                      (slabs == 1 || a.pre_rotated || wants_both_planes(slabs, true));
     if (MODE == kDual && !both) a.W = 2 * slabs;
     a.S = 16 / a.W;                                          // row streams sharing the CU
     const int threads = a.W * a.S * kWave;
@@ -644,6 +654,16 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
             return R == 2 ? launch_wide_one<kDual, 2, 1, false, false, true, true, true>(a, grid, threads, stream)
                           : launch_wide_one<kDual, 1, 1, false, false, true, true, true>(a, grid, threads, stream);
         }
+        if (both && slabs > 1) {      // 2 to 5 slabs: one wave per slab, both planes per wave, an image per rotation
+            const int ntiles = (a.L.in_features + kTile - 1) / kTile;
+            const bool two = ntiles > threads / kWave;
+            const int Rb = max_rows >= 2 ? 2 : 1;
+            a.iters = (max_rows + Rb - 1) / Rb;
+            if (Rb == 2) return two ? launch_wide_one<kDual, 2, 2, false, false, false, true, true>(a, grid, threads, stream)
+                                    : launch_wide_one<kDual, 2, 1, false, false, false, true, true>(a, grid, threads, stream);
+            return two ? launch_wide_one<kDual, 1, 2, false, false, false, true, true>(a, grid, threads, stream)
+                       : launch_wide_one<kDual, 1, 1, false, false, false, true, true>(a, grid, threads, stream);
+        }
         if (both) {
             const int rows_wg = (out + grid - 1) / grid;
             if (rows_wg >= 4 * a.S) return launch_wide_one<kDual, 2, 1, false, true, false, true, true>(a, grid, threads, stream);
@@ -661,17 +681,18 @@ hipError_t launch_wide_mode(GemvArgs a, int num_cus, hipStream_t stream) {
                     : launch_wide_shape<MODE, PAIR, false>(a, grid, threads, R, two, out, stream);
 }
 
-template <int MODE, int R, bool PAIR, bool PT>
+template <int MODE, int R, bool PAIR, bool PT, bool BOTH = false>
 hipError_t launch_group_one(const GemvGroup& g, int grid, int threads, hipStream_t stream) {
-    hipLaunchKernelGGL((tq_gemv_wide_group_kernel<MODE, R, PAIR, PT>), dim3(grid), dim3(threads), 0, stream, g);
+    hipLaunchKernelGGL((tq_gemv_wide_group_kernel<MODE, R, PAIR, PT, BOTH>), dim3(grid), dim3(threads), 0, stream, g);
     return hipGetLastError();
 }
 
-template <int MODE, bool PAIR, bool PT>
+// BOTH (dual rotation on pair tables, rows of up to 5 slabs): one wave per slab decodes both planes.
+template <int MODE, bool PAIR, bool PT, bool BOTH = false>
 hipError_t launch_group_mode(GemvGroup& g, int n, int num_cus, hipStream_t stream) {
     const int in = g.a[0].L.in_features;
     const int slabs = (in / kChunk + kWave - 1) / kWave;
-    const int W = PAIR ? in / (kSlab / 2) : (MODE == kDual ? 2 * slabs : slabs);
+    const int W = PAIR ? in / (kSlab / 2) : ((MODE == kDual && !BOTH) ? 2 * slabs : slabs);
     const int S = 16 / W;
     const int threads = W * S * kWave;
     long long total = 0;
@@ -700,7 +721,7 @@ hipError_t launch_group_mode(GemvGroup& g, int n, int num_cus, hipStream_t strea
         const int max_rows = a.rows_q + (a.rows_rem ? 1 : 0);
         if (max_rows < min_rows) min_rows = max_rows;
     }
-    const int R = (MODE != kSharedLut && min_rows >= 4) ? 4 : min_rows >= 2 * per_r ? 2 : 1;
+    const int R = (MODE != kSharedLut && !BOTH && min_rows >= 4) ? 4 : min_rows >= 2 * per_r ? 2 : 1;
     g.first[0] = 0;
     for (int j = 0; j < 3; ++j) g.first[j + 1] = g.first[j] + (j < n ? blocks[j] : 0);
     for (int j = n; j < 3; ++j) g.first[j + 1] = 1 << 30;        // no workgroup reaches an unused slot
@@ -709,11 +730,11 @@ hipError_t launch_group_mode(GemvGroup& g, int n, int num_cus, hipStream_t strea
         const int max_rows = g.a[j].rows_q + (g.a[j].rows_rem ? 1 : 0);
         g.a[j].iters = (max_rows + R * per_r - 1) / (R * per_r);
     }
-    if constexpr (MODE != kSharedLut) {
+    if constexpr (MODE != kSharedLut && !BOTH) {
         if (R == 4) return launch_group_one<MODE, 4, PAIR, PT>(g, used, threads, stream);
     }
-    if (R == 2) return launch_group_one<MODE, 2, PAIR, PT>(g, used, threads, stream);
-    return launch_group_one<MODE, 1, PAIR, PT>(g, used, threads, stream);
+    if (R == 2) return launch_group_one<MODE, 2, PAIR, PT, BOTH>(g, used, threads, stream);
+    return launch_group_one<MODE, 1, PAIR, PT, BOTH>(g, used, threads, stream);
 }
 
 }  // namespace
@@ -726,7 +747,10 @@ bool gemv_wide_group_supported(const LayerView* Ls, int n, int num_cus) {
     const LayerView& L0 = Ls[0];
     if (L0.mode != kSharedLut && L0.mode != kDual) return false;
     const int slabs = (L0.in_features / kChunk + kWave - 1) / kWave;
-    const int W = wants_pairs(L0) ? L0.in_features / (kSlab / 2) : (L0.mode == kDual ? 2 * slabs : slabs);
+    bool fp16_all = true;
+    for (int j = 0; j < n; ++j) fp16_all = fp16_all && Ls[j].fp16_centroids_ok;
+    const bool both = L0.mode == kDual && wants_both_planes(slabs, fp16_all);     // as launch_gemv_wide_group decides
+    const int W = wants_pairs(L0) ? L0.in_features / (kSlab / 2) : ((L0.mode == kDual && !both) ? 2 * slabs : slabs);
     if (W < 2 || W > 16) return false;
     if (L0.mode == kDual && slabs == 1) return false;       // one-slab dual rows: one wave per row (both planes), no sharing
     const int threads = W * (16 / W) * kWave;
@@ -749,6 +773,7 @@ hipError_t launch_gemv_wide_group(const GemvArgs* as, int n, int num_cus, hipStr
                               : launch_group_mode<kSharedLut, false, false>(g, n, num_cus, stream);
     bool fp16_ok = true;
     for (int j = 0; j < n; ++j) fp16_ok = fp16_ok && g.a[j].L.fp16_centroids_ok;
+    if (wants_both_planes(slabs, fp16_ok)) return launch_group_mode<kDual, false, true, true>(g, n, num_cus, stream);
     return (slabs <= kPairDualSlabs && fp16_ok) ? launch_group_mode<kDual, false, true>(g, n, num_cus, stream)
                                                 : launch_group_mode<kDual, false, false>(g, n, num_cus, stream);
 }
