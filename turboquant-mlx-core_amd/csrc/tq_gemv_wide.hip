@@ -587,6 +587,8 @@ hipError_t launch_wide_one(const GemvArgs& a, int grid, int threads, hipStream_t
 // planes per wave against one: 10240 x 10240 27.0 against 29.5 us, 27648 x 5120 32.8 / 33.9; rows of two slabs:
 // 18944 x 3584 18.8 / 19.0-20.0, 8192 x 8192 equal, 4096 x 4096 8.8 / 8.5: they stay with a wave per plane.  (A
 // property of the layer's width alone: a grouped launch must take the kernel a launch of its own would.)
+// (Also measured and not kept: a wave per 1024-column half at 5120 columns, 8 bytes per lane, plane and row, so
+// that no wave carries the half-empty third slab: 27648 x 5120 33.1 us, 5120 x 5120 12.4, no better than the above.)
 bool wants_both_planes(int slabs, bool fp16_ok) {
     return fp16_ok && slabs >= 3 && slabs <= kTwoImageSlabs;
 }
