@@ -320,13 +320,19 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
 # ------------------------------------------------------------------ prefill, 512-row activation panels
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("out,inf,bs,batch", [(16500, 256, 256, 257),      # one ragged panel, ragged last weight tile
+                                              (16500, 512, 256, 33),       # one row block per wave, one token in wave 0's
+                                              (16640, 256, 128, 128),      # one whole row block per wave
+                                              (16500, 512, 512, 129),      # two row blocks per wave
+                                              (16640, 768, 256, 256),
+                                              (16500, 256, 64, 300),       # three row blocks per wave
                                               (16640, 512, 128, 600),      # two panels, the second with 88 rows
                                               (33000, 768, 256, 1030),     # three panels
                                               (8300, 1024, 512, 1537)])    # four panels, 65 tiles each
 def test_prefill_panel_kernel_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, batch):
-    """More than 256 rows on a layer with enough 512 x 128 output tiles for the chip and a width that is a
+    """More than 32 rows on a layer with enough 512 x 128 output tiles for the chip and a width that is a
     multiple of 256 take tq_prefill_panel_kernel (activations as MFMA-operand images read straight from
-    global memory, 128 x 128 accumulators per wave): same tolerances as the other prefill kernel, every
+    global memory, 128 x 128 accumulators per wave; up to 384 rows the kernel instances that multiply one,
+    two or three of a wave's four row blocks): same tolerances as the other prefill kernel, every
     output dtype, and a row of the batch equal to its batch-1 result."""
     qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf + batch)
     x32 = np.random.default_rng(batch).standard_normal((batch, inf)).astype(np.float32)
@@ -336,7 +342,7 @@ def test_prefill_panel_kernel_matches_dequant_matmul(tq, oracle, mode, out, inf,
     y = layer.forward(xbits, tq.BF16, tq.F32)
     assert y.shape == (batch, out) and np.isfinite(y).all()
     assert _rel(y, want) < 1e-3
-    for b in (0, 255, 256, batch - 1):                       # no row leaks into another
+    for b in sorted({0, 31, 32, 127, 128, 255, 256, batch - 1} & set(range(batch))):      # no row leaks into another
         assert _rel(y[b:b + 1], want[b:b + 1]) < 1e-3
     for c in (0, 127, 128, out - 1):                         # nor a column
         assert _rel(y[:, c:c + 1], want[:, c:c + 1]) < 1e-3

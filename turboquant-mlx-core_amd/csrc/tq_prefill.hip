@@ -403,8 +403,9 @@ __global__ __launch_bounds__(kGemmThreads) void tq_prefill_gemm_kernel(PrefillAr
 // rows of 5120 columns and 10.9 against 8.5 us for 512 rows: the kernel is bound by neither its 64-byte accesses
 // nor, since the signs come from a table, its arithmetic.)
 // PANEL: fragment images for tq_prefill_panel_kernel instead, [M/512][K/16][4 waves][4 row blocks][64 lanes x 16 B]:
-// the 8 columns [16 u + 8 g, +8) of row r sit where lane 32 g + r % 32 of wave (r % 512) / 128 expects the
-// A operand of row block (r % 128) / 32 in sub-step u.
+// the 8 columns [16 u + 8 g, +8) of row r sit where lane 32 g + r % 32 of wave (r % 128) / 32 expects the
+// A operand of its row block (r % 512) / 128 in sub-step u (the first 128 rows of a panel are the first row block of
+// all four waves: a call of few rows keeps every SIMD busy with its first blocks).
 // ---------------------------------------------------------------------------
 template <bool PANEL>
 __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restrict__ x, int x_dtype,
@@ -444,7 +445,7 @@ __global__ __launch_bounds__(256) void tq_rotate_f16_kernel(const void* __restri
         const int m_tile = row >> 8, r = row & 255;
         uint4* dst = reinterpret_cast<uint4*>(out + (((size_t)m_tile * chunks + chunk) * 256 + r) * kBK);
         // (PANEL: 16-byte units; sub-step 2 chunk + i / 2 of panel row >> 9, block of (wave, row block), lane)
-        uint4* pdst = reinterpret_cast<uint4*>(out) + ((((size_t)(row >> 9) * chunks + chunk) * 2 * 4 + ((row >> 7) & 3)) * 4 + ((row >> 5) & 3)) * 64 + (row & 31);
+        uint4* pdst = reinterpret_cast<uint4*>(out) + ((((size_t)(row >> 9) * chunks + chunk) * 2 * 4 + ((row >> 5) & 3)) * 4 + ((row >> 7) & 3)) * 64 + (row & 31);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t w[4];
@@ -535,7 +536,7 @@ __global__ __launch_bounds__(256) void tq_rotate_panel_kernel(const void* __rest
             } else {
                 const int row = row0 + r;
                 if (active)
-                    img[((size_t)(row >> 9) * U_all + (g_own >> 1)) * 1024 + (size_t)(((row >> 7) & 3) * 4 + ((row >> 5) & 3)) * 64 +
+                    img[((size_t)(row >> 9) * U_all + (g_own >> 1)) * 1024 + (size_t)(((row >> 5) & 3) * 4 + ((row >> 7) & 3)) * 64 +
                         (row & 31) + (g_own & 1) * 32] = o;
             }
         }
@@ -544,7 +545,7 @@ __global__ __launch_bounds__(256) void tq_rotate_panel_kernel(const void* __rest
             __builtin_amdgcn_wave_barrier();
             // Store instruction i: lane -> (column group 8 i + lane / 8, row lane % 8): eight lanes write one line.
             const int r = lane & 7, row = row0 + r;
-            const size_t row_unit = (size_t)(((row >> 7) & 3) * 4 + ((row >> 5) & 3)) * 64 + (row & 31);
+            const size_t row_unit = (size_t)(((row >> 5) & 3) * 4 + ((row >> 7) & 3)) * 64 + (row & 31);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int g_in_seg = 8 * i + (lane >> 3);

@@ -83,7 +83,11 @@ template <> struct TileBytes<false> { u32x4v v[1]; };
 
 }  // namespace
 
-template <int MODE>
+// NBLK: row blocks of 32 tokens per wave.  4: whole panels.  1..3: a call of at most 128 NBLK rows (one panel, of
+// which the first NBLK blocks of every wave hold tokens: rows 128 i + 32 w + l are block i of wave w); the matrix
+// instructions, activation loads and stores of the other blocks are not compiled, the decode of the weight tile,
+// which the four waves share, is the same.
+template <int MODE, int NBLK>
 __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a) {
     __shared__ __align__(16) char smem[kPSmem];
 
@@ -140,9 +144,9 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
     // Fragment reads: lane -> (row lane % 32 of a 32-row block, 8 columns (lane / 32) of the sub-step).
     const char* const bfrag = smem + kPLut + (lane & 31) * kWPitch + (lane >> 5) * 16;
 
-    f32x16 acc[4][4];
+    f32x16 acc[NBLK][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NBLK; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
         const uint8_t* const bp = combined ? a.plane0 + (size_t)b_row * a.K + dh * 32
                                            : (plane == 0 ? a.plane0 : a.plane1) + (size_t)b_row * (a.K >> 1) + dh * 16;
 
-        f16x8 A[8][4];                                     // ring of eight sub-steps of this wave's 128 rows
+        f16x8 A[8][NBLK];                                  // ring of eight sub-steps of this wave's 32 NBLK rows
         f16x8 Bf[2][4];                                    // weight fragments of the current and the next sub-step
         Bytes By[4];                                       // ring of four tiles of index bytes
 
@@ -164,7 +168,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
             constexpr int s = decltype(Sc)::value;
             const char* p = ap + (size_t)(u < u_end ? u : u_end - 1) * kSubImage;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) A[s][i] = *reinterpret_cast<const f16x8*>(p + i * 1024);
+            for (int i = 0; i < NBLK; ++i) A[s][i] = *reinterpret_cast<const f16x8*>(p + i * 1024);
         };
         auto load_bytes = [&](auto Sc, int tile) {
             constexpr int s = decltype(Sc)::value;
@@ -291,7 +295,8 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
                 constexpr int i = k >> 2, j = k & 3;
                 // (weights as the first operand: a lane's 16 results are then 4 x 4 consecutive output columns of
                 // one token, which the epilogue stores without a transposition)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Bf[sb][j], A[sa][i], acc[i][j], 0, 0, 0);
+                if constexpr (i < NBLK)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Bf[sb][j], A[sa][i], acc[i][j], 0, 0, 0);
                 if constexpr (k < 4 && !(PANEL_ABL & 16))
                     Bf[sbn][k] = *reinterpret_cast<const f16x8*>(bfrag + fbuf * kWTile + k * 32 * kWPitch + fks * 32);
                 if constexpr (!(PANEL_ABL & 2)) {
@@ -326,7 +331,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
                         }
                     }
                 }
-                if constexpr (k >= 8 && k < 12 && !(PANEL_ABL & 1))
+                if constexpr (k >= 8 && k < 8 + NBLK && !(PANEL_ABL & 1))
                     A[san][k - 8] = *reinterpret_cast<const f16x8*>(pa + (k - 8) * 1024);
                 if constexpr (k == 14 && q == 3 && !(PANEL_ABL & 8)) {
                     const int tile = (ub >> 2) + dtile + 4;
@@ -376,7 +381,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
     lds_barrier();                                         // LDS is free for the epilogue
 
     // Epilogue: * norm[n] / sqrt(in) (1 / sqrt(bs) is in the rotated activations), convert, store.  Block (i, j) of
-    // a lane holds token m0 + 128 wave + 32 i + lane % 32 and, in registers 4 g .. 4 g + 3, the four consecutive
+    // a lane holds token m0 + 128 i + 32 wave + lane % 32 and, in registers 4 g .. 4 g + 3, the four consecutive
     // output columns n0 + 32 j + 8 g + 4 (lane / 32) + (0..3): one 8-byte (16-bit outputs) or 16-byte (fp32) store
     // each, straight from the accumulators.  The whole workgroup does nothing else meanwhile (one wave per SIMD,
     // one workgroup per CU), so the epilogue is kept to a read, a multiply, a packed conversion and a store.
@@ -385,7 +390,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
     if constexpr (PANEL_ABL & 32) {       // no epilogue: one value per lane keeps the accumulators alive
         float t = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < NBLK; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -398,7 +403,7 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
     const int y_type = is_part ? (int)kF32 : a.y_dtype;
     const int yN = is_part ? kPN : a.N, yM = is_part ? kPanelM : a.M;          // row pitch / row limit of y_out
     const int col0 = (is_part ? 0 : n0) + (lane >> 5) * 4;
-    const int row0 = (is_part ? 0 : m0) + wave * 128 + (lane & 31);
+    const int row0 = (is_part ? 0 : m0) + wave * 32 + (lane & 31);
     // Stores go through a buffer descriptor that ends with the output: rows and columns past the end are given an
     // offset beyond it and dropped by the hardware, so the loop nest carries no branches.
     // (all scales first: a load issued between stores would wait for every store before it, the memory counter
@@ -408,9 +413,9 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(y_out, 0, (int)((uint32_t)yM * (uint32_t)yN * es), 0x00020000);
     constexpr uint32_t kDropped = 0xfffffff0u;
     float4 scs[4][4];
-    uint32_t coff[4][4], roff[4];
+    uint32_t coff[4][4], roff[NBLK];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) roff[i] = (uint32_t)(row0 + 32 * i) * (uint32_t)yN * es;
+    for (int i = 0; i < NBLK; ++i) roff[i] = (uint32_t)(row0 + 128 * i) * (uint32_t)yN * es;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -444,10 +449,10 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
                 const int col = col0 + 32 * j + 8 * g;
                 const float4 sc = scs[j][g];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
+                for (int i = 0; i < NBLK; ++i) {
                     const float v0 = acc[i][j][4 * g] * sc.x, v1 = acc[i][j][4 * g + 1] * sc.y;
                     const float v2 = acc[i][j][4 * g + 2] * sc.z, v3 = acc[i][j][4 * g + 3] * sc.w;
-                    const bool row_ok = row0 + 32 * i < yM;
+                    const bool row_ok = row0 + 128 * i < yM;
                     const uint32_t at = (row_ok && col < yN) ? roff[i] + coff[j][g] : kDropped;
                     if constexpr (kVec) {
                         if constexpr (T == kF32) {
@@ -498,9 +503,9 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
         const uint32_t cbyte = (uint32_t)(n0 + (lane & 15) * 8) * 2u;
         const bool col_ok = n0 + (lane & 15) * 8 < yN;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
+        for (int half = 0; half < (NBLK + 1) / 2; ++half) {
 #pragma unroll
-            for (int ii = 0; ii < 2; ++ii)
+            for (int ii = 0; ii < (2 * half + 1 < NBLK ? 2 : 1); ++ii)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -520,9 +525,10 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
                         *reinterpret_cast<u32x2v*>(wr + ii * 32 * kPitch + (32 * j + 8 * g) * 2) = o;
                     }
 #pragma unroll
-            for (int it = 0; it < 16; ++it) {
+            for (int it = 0; it < (2 * half + 1 < NBLK ? 16 : 8); ++it) {
                 const u32x4v v = *reinterpret_cast<const u32x4v*>(rd + it * 4 * kPitch);
-                const int row = m0 + wave * 128 + half * 64 + it * 4 + (lane >> 4);
+                // (row it * 4 + lane / 16 of the stage: row block 2 half + it / 8, row (it % 8) * 4 + lane / 16 of it)
+                const int row = m0 + wave * 32 + (lane >> 4) + (2 * half + (it >> 3)) * 128 + (it & 7) * 4;
                 const uint32_t at = (row < yM && col_ok) ? (uint32_t)row * (uint32_t)yN * 2u + cbyte : kDropped;
                 __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)at, 0, 0);
             }
@@ -625,7 +631,7 @@ size_t prefill_panel_workspace_bytes(const LayerView& L, int batch, int num_cus,
 // that the parts fill the chip: 512 and 1024 rows of 3584 x 18944, 4096 x 14336 and 8192 x 8192 took 4-12 % longer
 // that way, 5120 x 27648 the same at 512 rows and 4 % less at 1024.)
 bool prefill_panel_supported(const LayerView& L, int batch, int num_cus) {
-    if (batch <= 256) return false;
+    if (batch <= kSkinnyMaxRows) return false;                 // (up to 32 rows: the small-batch kernels)
     if (L.mode != kSharedLut && L.mode != kDual && L.mode != kPrimaryOnly) return false;
     if (!L.fp16_centroids_ok) return false;
     if (!lanes_supported(L.in_features, L.block_size)) return false;
@@ -659,13 +665,22 @@ hipError_t launch_prefill_panel(const LayerView& L, const void* x, int x_dtype, 
     a.first_part_wg = plan.tail_tiles == a.panels * a.n_tiles ? 0 : 8 * a.n_per_xcd * a.panels;
     a.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + plan.xt_bytes);
     const dim3 grid((unsigned)(a.first_part_wg + a.tail_tiles * a.parts));
+    // Row blocks per wave: a single panel of at most 384 rows is run by the kernel that multiplies only the blocks
+    // that hold tokens.
+    const int nblk = batch > 3 * 128 ? 4 : (batch + 127) / 128;
+    auto launch = [&](auto Mode) {
+        constexpr int M = decltype(Mode)::value;
+        switch (nblk) {
+            case 1: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 1>), grid, dim3(kPThreads), 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 2>), grid, dim3(kPThreads), 0, stream, a); break;
+            case 3: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 3>), grid, dim3(kPThreads), 0, stream, a); break;
+            default: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 4>), grid, dim3(kPThreads), 0, stream, a); break;
+        }
+    };
     switch (L.mode) {
-        case kSharedLut:
-            hipLaunchKernelGGL(tq_prefill_panel_kernel<kSharedLut>, grid, dim3(kPThreads), 0, stream, a); break;
-        case kDual:
-            hipLaunchKernelGGL(tq_prefill_panel_kernel<kDual>, grid, dim3(kPThreads), 0, stream, a); break;
-        default:
-            hipLaunchKernelGGL(tq_prefill_panel_kernel<kPrimaryOnly>, grid, dim3(kPThreads), 0, stream, a); break;
+        case kSharedLut: launch(std::integral_constant<int, kSharedLut>{}); break;
+        case kDual: launch(std::integral_constant<int, kDual>{}); break;
+        default: launch(std::integral_constant<int, kPrimaryOnly>{}); break;
     }
     e = hipGetLastError();
     if (e != hipSuccess || a.tail_tiles == 0) return e;
