@@ -322,6 +322,7 @@ def test_prefill_bf16_matches_dequant_matmul(tq, oracle, mode, out, inf, bs, bat
 @pytest.mark.parametrize("out,inf,bs,batch", [(16500, 256, 256, 257),      # one ragged panel, ragged last weight tile
                                               (16500, 512, 256, 33),       # one row block per wave, one token in wave 0's
                                               (16640, 256, 128, 128),      # one whole row block per wave
+                                              (16500, 2048, 512, 100),     # ... and two wave groups that halve the row (widths that are multiples of 512)
                                               (16500, 512, 512, 129),      # two row blocks per wave
                                               (16640, 768, 256, 256),
                                               (16500, 256, 64, 300),       # three row blocks per wave

@@ -87,13 +87,22 @@ template <> struct TileBytes<false> { u32x4v v[1]; };
 // which the first NBLK blocks of every wave hold tokens: rows 128 i + 32 w + l are block i of wave w); the matrix
 // instructions, activation loads and stores of the other blocks are not compiled, the decode of the weight tile,
 // which the four waves share, is the same.
-template <int MODE, int NBLK>
-__global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a) {
-    __shared__ __align__(16) char smem[kPSmem];
+// KG = 2 (one row block per wave, whole tiles of a width that is a multiple of 512 columns): eight waves, two per
+// SIMD.  Waves 4..7 are a second group that walks the second half of the sub-steps with tile buffers of its own
+// and hands its products to the first group through LDS at the end: with one block of matrix instructions per
+// sub-step a lone wave per SIMD spends its time waiting for its own table reads, and a second wave fills the gaps.
+// Both groups run the same number of sub-steps, so they meet at every barrier.
+template <int MODE, int NBLK, int KG = 1>
+__global__ __launch_bounds__(kPThreads * KG) void tq_prefill_panel_kernel(PanelArgs a) {
+    static_assert(KG == 1 || (KG == 2 && NBLK == 1), "a second wave group: one row block per wave");
+    constexpr int kExchange = 4 * 64 * 272;            // past the epilogue's stage: the second group's products
+    __shared__ __align__(16) char smem[KG == 2 ? (kPLut + 4 * kWTile) : kPSmem];
+    static_assert(KG == 1 || kExchange + 4 * 64 * 64 * 4 <= kPLut + 4 * kWTile, "exchange area inside the workgroup's LDS");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);          // wave of its group
+    const int kg = KG == 2 ? __builtin_amdgcn_readfirstlane(tid >> 8) : 0;    // wave group
     const uint32_t laneoff = (uint32_t)lane << 2;
 
     // Workgroup ids go round the XCDs (id % 8).  The workgroups an XCD runs side by side share a panel of
@@ -133,6 +142,10 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
         u_begin = range * a.part_subs;
         u_end = u_begin + a.part_subs < U_all ? u_begin + a.part_subs : U_all;
     }
+    if constexpr (KG == 2) {                              // (the host sends only whole tiles of 32 k sub-steps here)
+        const int half = (u_end - u_begin) >> 1;
+        if (kg == 0) u_end = u_begin + half; else u_begin += half;
+    }
     const int m0 = panel * kPanelM, n0 = n_tile * kPN;
     const int tiles_end = u_end / 4;                       // 64-column weight tiles end here
 
@@ -140,9 +153,9 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
     // hold 16 consecutive rows, which the 144-byte pitch spreads over all 16 slot phases.
     const int drow = wave * 32 + (lane & 31), dh = lane >> 5;
     const int b_row = (n0 + drow < a.N) ? n0 + drow : a.N - 1;
-    char* const wdst = smem + kPLut + drow * kWPitch + dh * 64;
+    char* const wdst = smem + kPLut + kg * (2 * kWTile) + drow * kWPitch + dh * 64;
     // Fragment reads: lane -> (row lane % 32 of a 32-row block, 8 columns (lane / 32) of the sub-step).
-    const char* const bfrag = smem + kPLut + (lane & 31) * kWPitch + (lane >> 5) * 16;
+    const char* const bfrag = smem + kPLut + kg * (2 * kWTile) + (lane & 31) * kWPitch + (lane >> 5) * 16;
 
     f32x16 acc[NBLK][4];
 #pragma unroll
@@ -235,8 +248,8 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
             cfloat* const src = (cfloat*)(a.tables + (plane == 0 ? 0 : 16));
             uint32_t* const dst = reinterpret_cast<uint32_t*>(smem) + lane;
 #pragma unroll 8
-            for (int e = 0; e < 64; ++e) {
-                const int entry = wave * 64 + e;
+            for (int e = 0; e < 64 / KG; ++e) {
+                const int entry = (kg * 4 + wave) * (64 / KG) + e;
                 uint32_t v;
                 if constexpr (combined) v = (uint32_t)float_to_f16_bits(src[entry]) << 16;
                 else v = (uint32_t)float_to_f16_bits(src[entry & 15]) | ((uint32_t)float_to_f16_bits(src[entry >> 4]) << 16);
@@ -379,6 +392,23 @@ __global__ __launch_bounds__(kPThreads) void tq_prefill_panel_kernel(PanelArgs a
         }
     }
     lds_barrier();                                         // LDS is free for the epilogue
+    if constexpr (KG == 2) {
+        // The second group's products go to the first: [wave][register][lane] floats, past the stage the epilogue
+        // uses, so that no further barrier is needed.
+        float* const ex = reinterpret_cast<float*>(smem + kExchange) + wave * (64 * 64) + lane;
+        if (kg == 1) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ex[(j * 16 + r) * 64] = acc[0][j][r];
+        }
+        lds_barrier();
+        if (kg == 1) return;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[0][j][r] += ex[(j * 16 + r) * 64];
+    }
 
     // Epilogue: * norm[n] / sqrt(in) (1 / sqrt(bs) is in the rotated activations), convert, store.  Block (i, j) of
     // a lane holds token m0 + 128 i + 32 wave + lane % 32 and, in registers 4 g .. 4 g + 3, the four consecutive
@@ -671,7 +701,13 @@ hipError_t launch_prefill_panel(const LayerView& L, const void* x, int x_dtype, 
     auto launch = [&](auto Mode) {
         constexpr int M = decltype(Mode)::value;
         switch (nblk) {
-            case 1: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 1>), grid, dim3(kPThreads), 0, stream, a); break;
+            case 1:
+                // (whole tiles whose sub-steps halve into multiples of the unrolled loop: two wave groups)
+                if (a.tail_tiles == 0 && a.K % (2 * kSubK * kUnroll) == 0)
+                    hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 1, 2>), grid, dim3(2 * kPThreads), 0, stream, a);
+                else
+                    hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 1>), grid, dim3(kPThreads), 0, stream, a);
+                break;
             case 2: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 2>), grid, dim3(kPThreads), 0, stream, a); break;
             case 3: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 3>), grid, dim3(kPThreads), 0, stream, a); break;
             default: hipLaunchKernelGGL((tq_prefill_panel_kernel<M, 4>), grid, dim3(kPThreads), 0, stream, a); break;
