@@ -392,10 +392,12 @@ def test_prefill_panel_kernel_tail_tiles_in_k_ranges(tq, oracle, mode, out, inf,
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("out,inf,bs,batch,ydt", [(5100, 8192, 256, 2048, "f32"),   # 160 tiles, each in 3 ranges: two rounds of parts
                                                   (4400, 9216, 128, 2048, "f16"),   # 140 tiles, 576 sub-steps in 3 ranges, ragged last tile
-                                                  (5000, 8192, 512, 1600, "bf16")])  # 160 tiles, the last panel 64 rows
+                                                  (5000, 8192, 512, 1600, "bf16"),  # 160 tiles, the last panel 64 rows
+                                                  (1280, 8192, 512, 100, "bf16"),   # 10 tiles of long rows, up to 128 tokens: 8 ranges each
+                                                  (2000, 9216, 128, 40, "f32")])    # 16 tiles, ragged last one, one row block per wave
 def test_prefill_panel_kernel_less_than_a_round_all_tiles_cut_along_k(tq, oracle, mode, out, inf, bs, batch, ydt):
-    """Calls with fewer 512 x 128 tiles than the chip has CUs (but more than half as many) and long rows: every
-    tile is cut into K ranges (dual rotation: one part per plane and range, here two ranges) so that the parts
+    """Calls with fewer 512 x 128 tiles than the chip has CUs (more than half as many, or, up to 128 tokens of rows
+    of 8192 columns and more, any number) and long rows: every tile is cut into K ranges (dual rotation: one part per plane and range, here two ranges) so that the parts
     fill the chip; more parts than CUs run in rounds, and the sum kernel adds them.  Sampled rows of every panel
     against the oracle."""
     qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf + batch)

@@ -384,7 +384,7 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
     float* partial = nullptr;
     tq::PrefillPlan plan{};
     // (more than 256 rows and enough output tiles: 512-row activation panels, tq_prefill_panel.hip)
-    const bool panel = prefill && tq::prefill_panel_supported(V, batch, device_cu_count());
+    const bool panel = prefill && tq::prefill_panel_supported(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0);
     if (prefill && !panel) plan = tq::prefill_plan(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0);
     if (prefill || skinny) {
         const size_t work_need = panel ? tq::prefill_panel_workspace_bytes(V, batch, device_cu_count(), static_ws ? static_cap : ~(size_t)0)

@@ -619,16 +619,19 @@ PrefillPlan prefill_plan(const LayerView& L, int batch, int num_cus, size_t capa
     return p;
 }
 
-// Largest workspace any call of 16 .. max_batch rows needs (fewer rows can mean more ranges).
+// Largest workspace any call of 16 .. max_batch rows needs (fewer rows can mean more ranges, and the two kernels
+// cut differently: every row count at which the choice of kernel or the number of tiles changes is looked at).
 size_t prefill_reserve_bytes(const LayerView& L, int max_batch, int num_cus) {
     size_t need = 0;
-    for (int m_tiles = 1; (m_tiles - 1) * kBM < max_batch; ++m_tiles) {
-        const int rows = m_tiles * kBM < max_batch ? m_tiles * kBM : max_batch;
-        if (rows < 16) continue;
-        const size_t n = prefill_panel_supported(L, rows, num_cus) ? prefill_panel_workspace_bytes(L, rows, num_cus, ~(size_t)0)
-                                                                   : prefill_plan(L, rows, num_cus, ~(size_t)0).total_bytes;
+    auto look = [&](int rows) {
+        if (rows < 16 || rows > max_batch) return;
+        const size_t n = prefill_panel_supported(L, rows, num_cus, ~(size_t)0) ? prefill_panel_workspace_bytes(L, rows, num_cus, ~(size_t)0)
+                                                                             : prefill_plan(L, rows, num_cus, ~(size_t)0).total_bytes;
         if (n > need) need = n;
-    }
+    };
+    look(16); look(kSkinnyMaxRows); look(kSkinnyMaxRows + 1); look(128); look(129);
+    for (int rows = kBM; rows < max_batch + kBM; rows += kBM) { look(rows); look(rows + 1); }
+    look(max_batch);
     return need;
 }
 

@@ -30,7 +30,7 @@ __device__ __forceinline__ uint32_t pack_half2(uint32_t lo_val, uint32_t hi_val)
 // The panel kernel (tq_prefill_panel.hip): 512-row activation panels, activations read from global memory in
 // MFMA operand order.  Its rotated activations are "fragment images" (rotate_panel_kernel writes them).
 constexpr int kPanelM = 512;
-bool prefill_panel_supported(const LayerView& L, int batch, int num_cus);
+bool prefill_panel_supported(const LayerView& L, int batch, int num_cus, size_t capacity);
 // Workspace of a call: fragment images, then the fp32 parts of the tiles that are cut along K (none if that would
 // exceed `capacity`).  launch_prefill_panel derives the same cut from the bytes it is given.
 size_t prefill_panel_workspace_bytes(const LayerView& L, int batch, int num_cus, size_t capacity);

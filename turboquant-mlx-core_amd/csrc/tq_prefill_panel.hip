@@ -655,12 +655,14 @@ size_t prefill_panel_workspace_bytes(const LayerView& L, int batch, int num_cus,
     return panel_plan(L, batch, num_cus, capacity).total_bytes;
 }
 
-// More than 256 rows (up to 256 the 256-row tiles of the other kernel multiply half as many padding rows), a
-// width that fills the unrolled loop, and 512 x 128 tiles for more than half the CUs.  (With fewer tiles the other
-// kernel, which cuts K with 256 x 256 tiles, is as fast or faster even when every tile here is cut along K so
-// that the parts fill the chip: 512 and 1024 rows of 3584 x 18944, 4096 x 14336 and 8192 x 8192 took 4-12 % longer
-// that way, 5120 x 27648 the same at 512 rows and 4 % less at 1024.)
-bool prefill_panel_supported(const LayerView& L, int batch, int num_cus) {
+// More than 32 rows (up to there: the small-batch kernels), a width that fills the unrolled loop, and 512 x 128
+// tiles for more than half the CUs.  With fewer tiles the other kernel, which cuts K with 256 x 256 tiles, is as
+// fast or faster even when every tile here is cut along K so that the parts fill the chip (512 and 1024 rows of
+// 3584 x 18944, 4096 x 14336 and 8192 x 8192 took 4-12 % longer that way) - except up to 128 rows of long rows,
+// where the instance with one row block per wave and every tile cut wins (33 / 64 / 128 rows: 5120 x 27648 62 / 64 /
+// 71 us against 70 / 74 / 82, 8192 x 8192 41 / 42 / 44 against 42 / 45 / 50).  capacity: the workspace bytes the
+// caller can give (the cut needs room for its parts).
+bool prefill_panel_supported(const LayerView& L, int batch, int num_cus, size_t capacity) {
     if (batch <= kSkinnyMaxRows) return false;                 // (up to 32 rows: the small-batch kernels)
     if (L.mode != kSharedLut && L.mode != kDual && L.mode != kPrimaryOnly) return false;
     if (!L.fp16_centroids_ok) return false;
@@ -670,7 +672,8 @@ bool prefill_panel_supported(const LayerView& L, int batch, int num_cus) {
     // (the epilogue addresses the output with 32-bit byte offsets through a buffer descriptor)
     if ((unsigned long long)batch * (unsigned long long)L.out_features * 4ull >= (1ull << 31)) return false;
     const long long tiles = (long long)((batch + kPanelM - 1) / kPanelM) * ((L.out_features + kPN - 1) / kPN);
-    return tiles * 2 > num_cus;
+    if (tiles * 2 > num_cus) return true;
+    return batch <= 128 && L.in_features >= 8192 && panel_plan(L, batch, num_cus, capacity).tail_tiles > 0;
 }
 
 hipError_t launch_prefill_panel(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
