@@ -121,10 +121,15 @@ def _bits(o, rng, batch, inf):
 BATCHES = (1, 4, 15, 24, 40)      # batch-1 kernel, small-batch kernels (one and two sets of rows), prefill kernel
 
 
-@pytest.mark.parametrize("mode", ["shared", "dual", "primary_only", "dual_5bit"])
-def test_reserved_layer_is_captured_and_replayed(tq, oracle, mode):
+# (a layer with tiles for more than half the CUs: the panel kernel with one, two, three row blocks per wave, whole panels)
+PANEL_BATCHES = (40, 130, 300, 600)
+
+
+@pytest.mark.parametrize("mode,out,inf,bs,BATCHES", [("shared", 640, 2048, 512, BATCHES), ("dual", 640, 2048, 512, BATCHES),
+                                                     ("primary_only", 640, 2048, 512, BATCHES), ("dual_5bit", 640, 2048, 512, BATCHES),
+                                                     ("shared", 16500, 512, 256, PANEL_BATCHES), ("dual", 16500, 512, 256, PANEL_BATCHES)])
+def test_reserved_layer_is_captured_and_replayed(tq, oracle, mode, out, inf, bs, BATCHES):
     o, hip = oracle, _Hip()
-    out, inf, bs = 640, 2048, 512
     layer, qw, cb = _layer(tq, o, out, inf, bs, mode)
     layer.reserve(max(BATCHES))
     rng = np.random.default_rng(5)

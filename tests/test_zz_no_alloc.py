@@ -77,7 +77,8 @@ def _rel(a, b):
 # (out, in, block, first batch, second and smaller batch): small-batch kernels with the rotation inside
 # (blocks <= 512) and behind the separate rotation kernel (block 1024), and the prefill kernels
 CASES = [(300, 1024, 256, 8, 3), (513, 2048, 1024, 15, 2), (257, 1536, 512, 100, 20), (64, 512, 512, 300, 40),
-         (1000, 5120, 512, 9, 1)]
+         (1000, 5120, 512, 9, 1),
+         (16500, 512, 256, 300, 100)]     # enough tiles for the panel kernel: three row blocks per wave, then one (two wave groups)
 
 
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
