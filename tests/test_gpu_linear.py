@@ -361,7 +361,8 @@ def test_prefill_panel_kernel_matches_dequant_matmul(tq, oracle, mode, out, inf,
 @pytest.mark.parametrize("mode", ["shared", "dual", "primary_only"])
 @pytest.mark.parametrize("out,inf,bs,batch,ydt", [(8448, 2048, 512, 2000, "f32"),    # 4 x 66 tiles: 8 left after one round of 256
                                                   (8400, 2304, 256, 1600, "bf16"),   # ragged last tile, 144 sub-steps in parts of 32 (the last one 16)
-                                                  (16500, 2048, 128, 1025, "f16")])  # 3 x 129 tiles: 131 left after one round -> 1 part, whole
+                                                  (16500, 2048, 128, 1025, "f16"),   # 3 x 129 tiles: 131 left after one round -> 1 part, whole
+                                                  (33000, 2048, 256, 200, "bf16")])  # 258 tiles of two row blocks per wave, the last 2 cut
 def test_prefill_panel_kernel_tail_tiles_in_k_ranges(tq, oracle, mode, out, inf, bs, batch, ydt):
     """Tiles left over after the last full round of the chip are cut into K ranges (dual rotation: one part per
     plane and range) where that is cheaper by the library's count of rounds; a second kernel adds their fp32 products:
