@@ -173,13 +173,17 @@ __global__ __launch_bounds__(kPThreads * KG) void tq_prefill_panel_kernel(PanelA
         const uint8_t* const bp = combined ? a.plane0 + (size_t)b_row * a.K + dh * 32
                                            : (plane == 0 ? a.plane0 : a.plane1) + (size_t)b_row * (a.K >> 1) + dh * 16;
 
+        // One row block per wave and no token among this wave's 32 rows: the wave re-reads the first image it was
+        // given (one KB, in L1 after the first read) instead of pulling K x 64 bytes of padding through L2.  Its
+        // products are never stored.
+        const size_t a_step = (NBLK == 1 && m0 + wave * 32 >= a.M) ? 0 : (size_t)kSubImage;
         f16x8 A[8][NBLK];                                  // ring of eight sub-steps of this wave's 32 NBLK rows
         f16x8 Bf[2][4];                                    // weight fragments of the current and the next sub-step
         Bytes By[4];                                       // ring of four tiles of index bytes
 
         auto load_a = [&](auto Sc, int u) {
             constexpr int s = decltype(Sc)::value;
-            const char* p = ap + (size_t)(u < u_end ? u : u_end - 1) * kSubImage;
+            const char* p = ap + (size_t)(u < u_end ? u : u_end - 1) * a_step;
 #pragma unroll
             for (int i = 0; i < NBLK; ++i) A[s][i] = *reinterpret_cast<const f16x8*>(p + i * 1024);
         };
@@ -299,7 +303,7 @@ __global__ __launch_bounds__(kPThreads * KG) void tq_prefill_panel_kernel(PanelA
                 w0 = By[sby].v[0][q];
             }
             const int un = ub + U + 7;
-            const char* const pa = ap + (size_t)(un < u_end ? un : u_end - 1) * kSubImage;
+            const char* const pa = ap + (size_t)(un < u_end ? un : u_end - 1) * a_step;
             // One matrix instruction, then the k-th share of the side work, fenced: a single wave per SIMD has
             // nobody to fill the matrix pipe while it issues a run of other instructions, so they go out two or
             // three at a time in the shadow of the instruction before them.
