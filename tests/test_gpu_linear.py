@@ -465,6 +465,49 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     layer.close()
 
 
+# ------------------------------------------------------------------ two to four rows, whole weight rows per stream
+@pytest.mark.parametrize("out,inf,bs,batch", [
+    # the workgroups rotate the activation rows themselves: 2..7 segments of 256 columns per wave, one wave per row
+    # quad (no cross-wave sum) or several
+    (64, 256, 64, 2), (70, 1536, 512, 3), (64, 768, 256, 4), (66, 2048, 512, 2), (61, 1024, 64, 3),
+    (64, 2560, 512, 4), (63, 1280, 256, 2), (65, 4352, 256, 3), (64, 3328, 256, 4), (67, 1792, 256, 2),
+    # fewer rows than a quad, ragged quads, widths that are not a multiple of a segment, many streams per workgroup
+    (3, 1024, 64, 4), (1281, 5120, 512, 3), (6913, 5120, 512, 4), (130, 2816, 256, 4), (77, 1344, 64, 2),
+    (3000, 2848, 32, 3), (16500, 2304, 256, 4),
+    # four to six tiles of the rotation per wave
+    (6000, 11520, 256, 2), (10000, 6400, 256, 4), (10000, 6656, 512, 4),
+    # rows wider than 16384 columns come rotated from a kernel of their own
+    (4096, 17408, 512, 3), (3500, 24576, 512, 4), (2600, 27648, 512, 4), (2600, 32768, 512, 2)])
+def test_two_to_four_rows_whole_row_kernel(tq, oracle, out, inf, bs, batch):
+    """2..4 rows on a shared-rotation layer: the kernel that reads whole weight rows per stream (four rows and four
+    activation rows per v_mfma_f32_4x4x4_16b_f16 block, fp16 weights and rotated activations, fp32 sums, the
+    cross-wave sum inside the workgroup).  1e-3 relative L2 against the oracle for every activation type (5e-3 with a
+    bf16 output), every row by itself, every row equal to its batch-1 result within the same bound, and the same
+    bits on a second call."""
+    qw, cb = _packed_layer(oracle, out, inf, bs, "shared", out + inf + batch)
+    x32 = np.random.default_rng(batch + inf).standard_normal((batch, inf)).astype(np.float32)
+    xbits = oracle.f32_to_bf16_bits(x32)
+    w = oracle.dequantize_weight_cpu(qw, cb, cb, bs)
+    want = oracle.matmul_xwT(oracle.bf16_bits_to_f32(xbits), w, True)
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    y = layer.forward(xbits, tq.BF16, tq.F32)
+    assert y.shape == (batch, out) and np.isfinite(y).all()
+    assert _rel(y, want) < 1e-3
+    for b in range(batch):                                   # no row leaks into another
+        assert _rel(y[b:b + 1], want[b:b + 1]) < 1e-3
+    for c0 in range(0, out, max(1, out // 7)):               # nor a weight row into another
+        assert _rel(y[:, c0:c0 + 3], want[:, c0:c0 + 3]) < 2e-3
+    assert np.array_equal(y, layer.forward(xbits, tq.BF16, tq.F32))
+    yb = oracle.bf16_bits_to_f32(layer.forward(xbits, tq.BF16, tq.BF16))
+    assert _rel(yb, want) < 5e-3
+    y1 = layer.forward(xbits[batch - 1:batch], tq.BF16, tq.F32)      # exact fp32 batch-1 kernel
+    assert _rel(y[batch - 1:batch], y1) < 1e-3
+    x16 = x32.astype(np.float16)
+    assert _rel(layer.forward(x16, tq.F16, tq.F32), oracle.matmul_xwT(x16.astype(np.float32), w, True)) < 1e-3
+    assert _rel(layer.forward(x32), oracle.matmul_xwT(x32, w, True)) < 1e-3
+    layer.close()
+
+
 @pytest.mark.parametrize("mode", ["shared", "dual"])
 @pytest.mark.parametrize("batch", [2, 4, 16, 40, 64])
 @pytest.mark.parametrize("scale", [1e-4, 1e3, 1e4])

@@ -1,0 +1,508 @@
+// Fused TQ8 dequant + matrix-vector products for gfx950, two to four activation rows, shared-rotation layers
+// (one byte per weight), blocks of at most 512 columns.
+//
+// The batch-1 kernel (tq_gemv_wide.hip) reads the plane in whole rows and runs at the rate of its table reads.  The
+// small-batch kernel (tq_skinny.hip) puts the activation rows on v_mfma_f32_16x16x32_f16, whose operand layout
+// wants 16 weight rows per load instruction, 64 bytes of each; it cuts K over the workgroups and adds the parts in a
+// second kernel.  Up to four activation rows fit v_mfma_f32_4x4x4_16b_f16 instead: 16 independent 4 x 4 x 4 blocks
+// per instruction, block = lane / 4.  The four lanes of a block hold the same 16 columns of four consecutive weight
+// rows (A operand: four decoded weights per step) and of the four activation rows (B operand), so
+//   * a load instruction of a wave fetches 256 contiguous bytes of each of four rows (whole cache lines), a wave
+//     covers U such segments of its four rows, and the waves of a row stream cover the whole row: no cut along K,
+//     the cross-wave sum stays inside the workgroup and there is no second kernel;
+//   * a decoded weight costs one address permute, one table read and half a pack (as in the small-batch kernel)
+//     whatever the number of activation rows; the products are four matrix instructions per 16 bytes of a lane;
+//   * the kernel keeps the batch-1 kernel's shape: one workgroup of up to 16 waves per CU, lane-private table
+//     in LDS, the rotated activations of a lane's columns in registers (fp16 pairs, scaled by 1 / sqrt(bs) before
+//     they are rounded, as in the small-batch and prefill kernels), every load slot requested again as soon as it
+//     has been decoded.
+// The activation rows are rotated once per CU (the waves share out the 512-column tiles of all rows and hand the
+// result over through fp16 images in LDS), or, where the images do not fit, by a small kernel of its own.
+// Sums are fp32.  The reference has no batched path (src/dequantizer.cpp:545-549: batch is a grid dimension of its
+// per-row kernel).
+#include "tq_device.h"
+#include "tq_gemv_common.h"
+
+namespace tq {
+
+namespace {
+
+constexpr int kSegCols = 256;                    // columns of a segment: 16 blocks x 16 columns
+constexpr int kFewMaxBatch = 4;
+constexpr int kFewImageBytes = 88 * 1024;        // fp16 images of the activation rows in LDS
+constexpr int kFewMaxU = 8;
+constexpr int kFewPartialBytes = 2 * 16 * 32 * 4;   // [2 buffers][<= 16 waves][<= 32 sums]
+
+// Quads of weight rows per trip of the main loop.  (Two, for twice the loads in flight and half the cross-wave sums,
+// measured no faster on the large layers and slower on the small ones, whose streams have one or two quads.)
+constexpr int few_quads(int) { return 1; }
+
+struct FewArgs {
+    LayerView L;
+    const void* x;       // activations [batch, in] (x_dtype), or PRE: rotated, scaled fp16 [batch, in]
+    void* y;
+    int x_dtype, y_dtype;
+    int batch;
+    int W, S;            // waves per row quad, quad streams per workgroup
+    int w_inv;           // (w * w_inv) >> 8 == w / W
+    int iters;           // uniform trip count: the longest range of a stream, in trips of the main loop
+    int quads_q, quads_rem;
+    int ntiles, nt_inv;  // 512-column tiles of a row; (i * nt_inv) >> 16 == i / ntiles for the job numbers in use
+};
+
+typedef _Float16 few_h4 __attribute__((ext_vector_type(4)));
+typedef float few_f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t few_u2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint4 few_load16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, int row_off) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, row_off, 2);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ uint4 few_pack8(const float (&v)[8], float s) {
+    uint4 o;
+    o.x = (uint32_t)float_to_f16_bits(v[0] * s) | ((uint32_t)float_to_f16_bits(v[1] * s) << 16);
+    o.y = (uint32_t)float_to_f16_bits(v[2] * s) | ((uint32_t)float_to_f16_bits(v[3] * s) << 16);
+    o.z = (uint32_t)float_to_f16_bits(v[4] * s) | ((uint32_t)float_to_f16_bits(v[5] * s) << 16);
+    o.w = (uint32_t)float_to_f16_bits(v[6] * s) | ((uint32_t)float_to_f16_bits(v[7] * s) << 16);
+    return o;
+}
+
+// rotate_tile() with the signs handed in: blocks are at most one tile wide and tiles start at multiples of 512, so
+// the sign of a column depends on its position inside the tile alone, and a wave computes its eight once for all
+// the tiles it rotates (the hash is a quarter of the instructions of a rotation).
+__device__ __forceinline__ void few_rotate(const TileRaw& raw, int x_dtype, bool active, const float (&sg)[8],
+                                           uint32_t bs, int lane, float (&v)[8]) {
+    if (active) {
+        if (x_dtype == kF32) {
+            const uint32_t w[8] = {raw.a.x, raw.a.y, raw.a.z, raw.a.w, raw.b.x, raw.b.y, raw.b.z, raw.b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = __builtin_bit_cast(float, w[j]);
+        } else {
+            const uint32_t w[4] = {raw.a.x, raw.a.y, raw.a.z, raw.a.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (x_dtype == kBF16) {
+                    v[2 * j]     = bf16_bits_to_float(w[j] & 0xffffu);
+                    v[2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+                } else {
+                    v[2 * j]     = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] & 0xffffu));
+                    v[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] >> 16));
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] *= sg[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = 0.0f;
+    }
+    fwht_lanes<8>(v, bs, lane);
+}
+
+// U segments per wave (wave w of a quad stream owns segments U w .. U w + U - 1 of its rows), Q quads of weight
+// rows per trip of the main loop, TL tile jobs of the rotation per wave (PRE: none, the rows come rotated).
+template <int U, int Q, int TL, bool PRE>
+__device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
+    constexpr int kImage = PRE ? 0 : kFewImageBytes;
+    constexpr int kSums = 16 * Q;                  // (weight row of the trip, activation row) pairs
+    __shared__ __align__(16) char smem[kLut256Bytes + kFewPartialBytes + kImage];
+    float* const partial = reinterpret_cast<float*>(smem + kLut256Bytes);     // [2][waves][32]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int stream = (wave * a.w_inv) >> 8;
+    const int unit = wave - stream * a.W;
+    const uint32_t laneoff = (uint32_t)lane << 2;
+    const int out = a.L.out_features, K = a.L.in_features;
+    const int blk = lane >> 2, q = lane & 3;      // block of the matrix instruction; weight row of the quad and activation row
+
+    int col[U];
+    bool act[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        col[u] = (unit * U + u) * kSegCols + 16 * blk;
+        act[u] = col[u] < K;
+    }
+
+    // Quads of this stream: a contiguous range, one more for the first quads_rem streams.
+    const int gs = block * a.S + stream;
+    const int q_begin = gs * a.quads_q + (gs < a.quads_rem ? gs : a.quads_rem);
+    const int q_end = q_begin + a.quads_q + (gs < a.quads_rem ? 1 : 0);
+    const int r_begin = 4 * q_begin;
+    const int r_end = 4 * q_end < out ? 4 * q_end : out;
+    const int r_base = r_begin < out ? r_begin : out - 1;
+
+    // The plane through a buffer descriptor based at the stream's first row.  Segments past the row and rows past
+    // the range ask for an offset beyond the descriptor and fetch nothing (zeros: entry 0 of the table, times
+    // activations that are zero, or sums that are not stored).
+    constexpr uint32_t kNoFetch = 0x80000000u;
+    uint32_t off[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) off[u] = act[u] ? (uint32_t)q * (uint32_t)K + (uint32_t)col[u] : kNoFetch;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(a.L.packed_combined) + (size_t)r_base * (size_t)K, 0, 0x7fffffff, 0x00020000);
+    uint4 P[Q][U];                            // one load slot per quad and segment, requested again as soon as it is decoded
+    auto fetch = [&](auto Uc, int r0) {
+        constexpr int u = decltype(Uc)::value;
+#pragma unroll
+        for (int k = 0; k < Q; ++k)
+            P[k][u] = few_load16(rs, r0 + 4 * k + q < r_end ? off[u] : kNoFetch, (r0 + 4 * k - r_base) * K);
+    };
+    auto norm_of = [&](int r0) {
+        const int rn = r0 + ((lane >> 2) & (4 * Q - 1));
+        return a.L.norms[rn < out ? rn : out - 1];
+    };
+
+    // Small requests first (loads complete in order): the activation tiles this wave rotates, or its columns of
+    // the rotated rows; then the norms of the first quad and the first weights.
+    uint32_t xh[U][8];                        // fp16 pairs of activation row q: columns 2 j, 2 j + 1 of segment u
+    TileRaw raw[PRE ? 1 : TL];
+    const int jobs = a.batch * a.ntiles;
+    if constexpr (PRE) {
+        const char* xr = static_cast<const char*>(a.x);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool on = act[u] && q < a.batch;
+            const uint4* p = reinterpret_cast<const uint4*>(xr + ((size_t)(on ? q : 0) * K + (on ? col[u] : 0)) * 2);
+            const uint4 lo = p[0], hi = p[1];
+            xh[u][0] = lo.x; xh[u][1] = lo.y; xh[u][2] = lo.z; xh[u][3] = lo.w;
+            xh[u][4] = hi.x; xh[u][5] = hi.y; xh[u][6] = hi.z; xh[u][7] = hi.w;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < TL; ++k) {            // jobs past the last re-read the start of the first row and are not used
+            const int job = wave + k * nwaves;
+            const int tok = (job * a.nt_inv) >> 16;
+            const int c = (job - tok * a.ntiles) * kTile + lane * 8;
+            const bool on = job < jobs && c < K;
+            raw[k] = load_tile_raw(a.x, a.x_dtype, (size_t)(on ? tok : 0) * K, on ? c : 0);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    float nrm = norm_of(r_begin);
+    fetch(std::integral_constant<int, 0>{}, r_begin);
+    if constexpr (U > 1) fetch(std::integral_constant<int, 1>{}, r_begin);
+    if constexpr (U > 2) fetch(std::integral_constant<int, 2>{}, r_begin);
+    if constexpr (U > 3) fetch(std::integral_constant<int, 3>{}, r_begin);
+
+    // Decode table -> LDS, one private column per lane: fp16 value in the upper half of the entry.  Values through
+    // scalar loads (a vector memory instruction holds the CU's address unit for 16 cycles, and 16 waves share it).
+    {
+        typedef const __attribute__((address_space(4))) float cfloat;
+        cfloat* const tab = (cfloat*)a.L.tables;
+        uint32_t* const dst = reinterpret_cast<uint32_t*>(smem) + lane;
+        for (int c = wave; c < 16; c += nwaves) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) dst[(c * 16 + e) * kWave] = (uint32_t)float_to_f16_bits(tab[c * 16 + e]) << 16;
+        }
+    }
+
+    if constexpr (PRE) {
+        __syncthreads();                                       // table visible to every wave
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xh[u][j] = (act[u] && q < a.batch) ? xh[u][j] : 0u;     // idle lanes contribute 0
+    } else {
+        char* const image = smem + kLut256Bytes + kFewPartialBytes;               // [batch][K] fp16
+        float sg[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sg[j] = sign_of(a.L.seed_primary, (uint32_t)(lane * 8 + j) & (a.L.block_size - 1));
+#pragma unroll
+        for (int k = 0; k < TL; ++k) {
+            const int job = wave + k * nwaves;
+            if (job < jobs) {                                  // wave-uniform
+                const int tok = (job * a.nt_inv) >> 16;
+                const int c = (job - tok * a.ntiles) * kTile + lane * 8;
+                float v[8];
+                few_rotate(raw[k], a.x_dtype, c < K, sg, a.L.block_size, lane, v);
+                if (c < K) *reinterpret_cast<uint4*>(image + ((size_t)tok * K + c) * 2) = few_pack8(v, a.L.inv_sqrt_bs);
+            }
+        }
+        __syncthreads();                                       // images and table visible to every wave
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool on = act[u] && q < a.batch;
+            const uint4* p = reinterpret_cast<const uint4*>(image + ((size_t)(on ? q : 0) * K + (on ? col[u] : 0)) * 2);
+            const uint4 lo = p[0], hi = p[1];
+            xh[u][0] = on ? lo.x : 0u; xh[u][1] = on ? lo.y : 0u; xh[u][2] = on ? lo.z : 0u; xh[u][3] = on ? lo.w : 0u;
+            xh[u][4] = on ? hi.x : 0u; xh[u][5] = on ? hi.y : 0u; xh[u][6] = on ? hi.z : 0u; xh[u][7] = on ? hi.w : 0u;
+        }
+    }
+    // The other load slots are requested behind the barrier: a wave whose requests queue up in the memory pipeline
+    // would otherwise keep the whole workgroup waiting there.
+    if constexpr (U > 4) fetch(std::integral_constant<int, 4>{}, r_begin);
+    if constexpr (U > 5) fetch(std::integral_constant<int, 5>{}, r_begin);
+    if constexpr (U > 6) fetch(std::integral_constant<int, 6>{}, r_begin);
+    if constexpr (U > 7) fetch(std::integral_constant<int, 7>{}, r_begin);
+
+    // Four weights of this lane's row -> one A operand (entries are fp32 patterns with the fp16 value in the upper half).
+    auto operand = [&](uint32_t w) {
+        const uint32_t v0 = *reinterpret_cast<const uint32_t*>(smem + entry_addr<0>(w, laneoff));
+        const uint32_t v1 = *reinterpret_cast<const uint32_t*>(smem + entry_addr<1>(w, laneoff));
+        const uint32_t v2 = *reinterpret_cast<const uint32_t*>(smem + entry_addr<2>(w, laneoff));
+        const uint32_t v3 = *reinterpret_cast<const uint32_t*>(smem + entry_addr<3>(w, laneoff));
+        const few_u2 r = {__builtin_amdgcn_perm(v1, v0, 0x07060302u), __builtin_amdgcn_perm(v3, v2, 0x07060302u)};
+        return __builtin_bit_cast(few_h4, r);
+    };
+
+    for (int it = 0; it < a.iters; ++it) {
+        const int r0 = r_begin + 4 * Q * it;
+        const float nrm_next = norm_of(r0 + 4 * Q);
+        few_f4 acc[Q];                                         // results D[i][q] of the lane's block: weight rows r0 + 4 k + i
+#pragma unroll
+        for (int k = 0; k < Q; ++k) acc[k] = few_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        auto segment = [&](auto Uc) {
+            constexpr int u = decltype(Uc)::value;
+            uint4 p[Q];
+#pragma unroll
+            for (int k = 0; k < Q; ++k) p[k] = P[k][u];
+            fetch(Uc, r0 + 4 * Q);
+#pragma unroll
+            for (int k = 0; k < Q; ++k) {
+                const uint32_t pw[4] = {p[k].x, p[k].y, p[k].z, p[k].w};
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const few_u2 xb = {xh[u][2 * d], xh[u][2 * d + 1]};
+                    acc[k] = __builtin_amdgcn_mfma_f32_4x4x4f16(operand(pw[d]), __builtin_bit_cast(few_h4, xb), acc[k], 0, 0, 0);
+                }
+            }
+        };
+        segment(std::integral_constant<int, 0>{});
+        if constexpr (U > 1) segment(std::integral_constant<int, 1>{});
+        if constexpr (U > 2) segment(std::integral_constant<int, 2>{});
+        if constexpr (U > 3) segment(std::integral_constant<int, 3>{});
+        if constexpr (U > 4) segment(std::integral_constant<int, 4>{});
+        if constexpr (U > 5) segment(std::integral_constant<int, 5>{});
+        if constexpr (U > 6) segment(std::integral_constant<int, 6>{});
+        if constexpr (U > 7) segment(std::integral_constant<int, 7>{});
+
+        // Sum over the 16 blocks (the columns of the wave): afterwards every lane holds the wave total of weight row
+        // (lane / 4) % (4 Q) of the trip and activation row lane % 4.
+        float v[4 * Q];
+#pragma unroll
+        for (int k = 0; k < Q; ++k)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[4 * k + i] = acc[k][i];
+        const float total = reduce_rec<4 * Q, 4>(v, lane);
+        const int r = r0 + ((lane >> 2) & (4 * Q - 1));
+        const bool owner = lane < kSums && q < a.batch && r < r_end;
+        float t = total;
+        bool store = owner;
+        if (a.W > 1) {                                         // cross-wave sum of the row's segments
+            float* const buf_base = partial + (it & 1) * (16 * 32);
+            if (lane < kSums) buf_base[wave * 32 + lane] = total;
+            __syncthreads();
+            store = owner && unit == 0;
+            if (store) {
+                t = 0.0f;
+                for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * 32 + lane];
+            }
+        }
+        if (store) store_scalar(a.y, a.y_dtype, (size_t)q * out + r, t * (a.L.inv_scale * nrm));
+        nrm = nrm_next;
+    }
+}
+
+template <int U, int Q, int TL, bool PRE>
+__global__ __launch_bounds__(1024) void tq_gemv_few_kernel(FewArgs a) {
+    few_body<U, Q, TL, PRE>(a, (int)blockIdx.x);
+}
+
+// Two or three layers of equal width on the same activation rows (q, k, v or gate, up), one launch: the
+// workgroups are shared out over the layers by rows.
+struct FewGroup {
+    FewArgs a[3];
+    int first[4];          // layer j owns workgroups first[j] .. first[j + 1] - 1
+};
+template <int U, int TL>
+__global__ __launch_bounds__(1024) void tq_gemv_few_group_kernel(FewGroup g) {
+    const int b = (int)blockIdx.x;
+    const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
+    few_body<U, few_quads(U), TL, false>(g.a[j], b - g.first[j]);
+}
+
+// Rotated, scaled activation rows as fp16 [batch, in] for the layers whose images do not fit LDS: one wave per
+// 512-column tile and row.
+__global__ __launch_bounds__(64) void tq_rotate_rows_f16_kernel(const void* x, int x_dtype, int K, uint32_t seed,
+                                                                 uint32_t bs, float scale, uint16_t* out) {
+    const int lane = threadIdx.x, t = blockIdx.y;
+    const int c = blockIdx.x * kTile + lane * 8;
+    const TileRaw raw = load_tile_raw(x, x_dtype, (size_t)t * K, c < K ? c : 0);
+    float v[8];
+    rotate_tile(raw, x_dtype, c, c < K, seed, bs, lane, v);
+    if (c < K) *reinterpret_cast<uint4*>(out + (size_t)t * K + c) = few_pack8(v, scale);
+}
+
+// The shape of a launch: segments per wave, waves per row quad, quad streams, rotation jobs per wave, whether the
+// rows come rotated.  Among the splits of the row's segments over 1 to 16 waves with at most kFewMaxU segments each,
+// the one that keeps most lanes busy (segments that exist, waves that exist; on a tie the one nearest four
+// segments per wave: streams short enough for layers of a few thousand rows, long enough between two barriers).  A function
+// of the width and the batch alone: the order in which a row's products are added depends on it, and a layer must
+// give the same bits in a launch of its own and in one it shares.
+struct FewShape { int U, W, S, threads, tl; bool pre; };
+FewShape few_shape(int K, int batch) {
+    FewShape s{};
+    const int segs = (K + kSegCols - 1) / kSegCols;
+    double best = -1.0;
+    for (int W = 1; W <= 16; ++W) {
+        int U = (segs + W - 1) / W;
+        if (U > kFewMaxU) continue;
+        if (U < 2) U = 2;
+        const int S = 16 / W;
+        const double eff = (double)segs / (W * U) * (W * S) / 16.0;
+        const bool tie = eff > best - 1e-9 && (U - 4) * (U - 4) < (s.U - 4) * (s.U - 4);
+        if (eff > best + 1e-9 || tie) { best = eff; s.U = U; s.W = W; s.S = S; }
+    }
+    s.threads = s.W * s.S * kWave;
+    const int ntiles = (K + kTile - 1) / kTile, waves = s.W * s.S;
+    const int per_wave = (batch * ntiles + waves - 1) / waves;
+    s.pre = (size_t)batch * K * 2 > (size_t)kFewImageBytes || per_wave > 6;
+    s.tl = per_wave <= 3 ? 3 : 6;
+    return s;
+}
+
+void few_ranges(FewArgs& a, const FewShape& s, int grid, int batch) {
+    const int quads = (a.L.out_features + 3) / 4, ts = grid * s.S;
+    a.batch = batch;
+    a.W = s.W; a.S = s.S;
+    a.w_inv = (256 + s.W - 1) / s.W;
+    a.quads_q = quads / ts;
+    a.quads_rem = quads % ts;
+    a.iters = (a.quads_q + (a.quads_rem ? 1 : 0) + few_quads(s.U) - 1) / few_quads(s.U);
+    a.ntiles = (a.L.in_features + kTile - 1) / kTile;
+    a.nt_inv = 65536 / a.ntiles + 1;       // exact quotients for job numbers below 16 x 6 (at most 64 tiles per row)
+}
+
+template <int U>
+hipError_t launch_few_u(const FewArgs& a, const FewShape& s, int grid, hipStream_t stream) {
+    const dim3 g(grid), b(s.threads);
+    if (s.pre) hipLaunchKernelGGL((tq_gemv_few_kernel<U, few_quads(U), 1, true>), g, b, 0, stream, a);
+    else if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_kernel<U, few_quads(U), 3, false>), g, b, 0, stream, a);
+    else hipLaunchKernelGGL((tq_gemv_few_kernel<U, few_quads(U), 6, false>), g, b, 0, stream, a);
+    return hipGetLastError();
+}
+
+template <int U>
+hipError_t launch_few_group_u(const FewGroup& g, const FewShape& s, int grid, hipStream_t stream) {
+    const dim3 gr(grid), b(s.threads);
+    if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_group_kernel<U, 3>), gr, b, 0, stream, g);
+    else hipLaunchKernelGGL((tq_gemv_few_group_kernel<U, 6>), gr, b, 0, stream, g);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+namespace {
+// What the kernel asks of a layer whatever the launch: shared rotation, centroid sums that fit fp16, blocks of at
+// most 512 columns (a block never leaves the tile a wave rotates), rows of at most 64 tiles.
+bool few_layer_ok(const LayerView& L, int batch) {
+    if (batch < 2 || batch > kFewMaxBatch) return false;
+    if (L.mode != kSharedLut || !L.packed_combined || !L.fp16_centroids_ok) return false;
+    if (!lanes_supported(L.in_features, L.block_size) || L.block_size > (uint32_t)kTile) return false;
+    return L.in_features <= 16 * kFewMaxU * kSegCols;
+}
+// A stream's share of the plane stays below the 2 GB of its buffer descriptor (one stream per CU at least).
+bool few_share_ok(const LayerView& L, int num_cus) {
+    const long long cus = num_cus > 0 ? num_cus : 1;
+    const long long max_rows = (L.out_features + cus - 1) / cus + 24;
+    return (unsigned long long)max_rows * (unsigned long long)L.in_features < (1ull << 31);
+}
+// Every workgroup rotates all the activation rows for itself: about 0.15 us per 512-column tile and row, whatever
+// the size of the plane, where the small-batch kernel pays 4 us for its second kernel and loses about 0.06 us per MB
+// of plane to its load pattern (same-box comparisons of the two on eleven shapes, weight copies cycled).  Few rows
+// of a wide plane go to the small-batch kernel.  (Up to 40 tiles whatever the plane: the layers of a group, large
+// and small, should agree on the kernel, or the group is run layer by layer.)
+bool few_worth_it(int batch, int K, long long plane_bytes) {
+    const long long jobs = (long long)batch * ((K + kTile - 1) / kTile);
+    return jobs <= 40 || jobs * 5 <= 135 + plane_bytes / 500000;           // jobs <= 27 + 0.4 per MB
+}
+}  // namespace
+
+// Two to four rows of any activation type.
+bool gemv_few_supported(const LayerView& L, int batch, int num_cus) {
+    if (!few_layer_ok(L, batch) || !few_share_ok(L, num_cus)) return false;
+    const FewShape s = few_shape(L.in_features, batch);
+    // (rows that come rotated: the scratch row holds them, 2 x in floats = 4 rows of fp16; the rotation is a
+    // kernel of its own, which only a plane of some size repays)
+    if (s.pre) return L.xrot_work != nullptr && (long long)L.out_features * L.in_features >= (64ll << 20);
+    return few_worth_it(batch, L.in_features, (long long)L.out_features * L.in_features);
+}
+
+namespace {
+template <typename F>
+hipError_t few_dispatch_u(int U, F&& f) {
+    switch (U) {
+        case 2: return f(std::integral_constant<int, 2>{});
+        case 3: return f(std::integral_constant<int, 3>{});
+        case 4: return f(std::integral_constant<int, 4>{});
+        case 5: return f(std::integral_constant<int, 5>{});
+        case 6: return f(std::integral_constant<int, 6>{});
+        case 7: return f(std::integral_constant<int, 7>{});
+        case 8: return f(std::integral_constant<int, 8>{});
+        default: return hipErrorInvalidValue;
+    }
+}
+}  // namespace
+
+hipError_t launch_gemv_few(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
+                           int num_cus, hipStream_t stream) {
+    const FewShape s = few_shape(L.in_features, batch);
+    FewArgs a{};
+    a.L = L; a.x = x; a.y = y; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+    if (s.pre) {
+        uint16_t* const xr = reinterpret_cast<uint16_t*>(L.xrot_work);
+        hipLaunchKernelGGL(tq_rotate_rows_f16_kernel, dim3((L.in_features + kTile - 1) / kTile, batch), dim3(64), 0, stream,
+                           x, x_dtype, L.in_features, L.seed_primary, L.block_size, L.inv_sqrt_bs, xr);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        a.x = xr;
+    }
+    const int quads = (L.out_features + 3) / 4;
+    int grid = (quads + s.S - 1) / s.S;
+    if (grid > num_cus) grid = num_cus;
+    if (grid < 1) grid = 1;
+    few_ranges(a, s, grid, batch);
+    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value>(a, s, grid, stream); });
+}
+
+// Layers that can share a launch: two or three of equal width, each taken by the kernel in a launch of its own, whose
+// rows the workgroups rotate themselves.
+bool gemv_few_group_supported(const LayerView* Ls, int n, int batch, int num_cus) {
+    if (n < 2 || n > 3 || num_cus < n) return false;
+    for (int j = 0; j < n; ++j) {
+        if (Ls[j].in_features != Ls[0].in_features) return false;
+        if (!gemv_few_supported(Ls[j], batch, 1)) return false;      // (1 CU: the strictest bound on a stream's share)
+    }
+    return !few_shape(Ls[0].in_features, batch).pre;
+}
+
+hipError_t launch_gemv_few_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
+                                 int y_dtype, int num_cus, hipStream_t stream) {
+    long long total = 0;
+    for (int j = 0; j < n; ++j) total += Ls[j].out_features;
+    const FewShape s = few_shape(Ls[0].in_features, batch);
+    // Workgroups per layer in proportion to its rows.
+    int blocks[3] = {0, 0, 0}, used = 0;
+    for (int j = 0; j < n; ++j) {
+        blocks[j] = (int)((long long)num_cus * Ls[j].out_features / total);
+        if (blocks[j] < 1) blocks[j] = 1;
+        used += blocks[j];
+    }
+    for (int j = 0; used < num_cus; j = (j + 1) % n) { ++blocks[j]; ++used; }
+    for (int j = 0; used > num_cus; j = (j + 1) % n) if (blocks[j] > 1) { --blocks[j]; --used; }
+    FewGroup g{};
+    g.first[0] = 0;
+    for (int j = 0; j < 3; ++j) g.first[j + 1] = g.first[j] + (j < n ? blocks[j] : 0);
+    for (int j = n; j < 3; ++j) { g.first[j] = 1 << 30; g.first[j + 1] = 1 << 30; }     // no workgroup reaches an unused slot
+    for (int j = 0; j < n; ++j) {
+        FewArgs& a = g.a[j];
+        a.L = Ls[j]; a.x = x; a.y = ys[j]; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+        few_ranges(a, s, blocks[j], batch);
+    }
+    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_group_u<decltype(Uc)::value>(g, s, used, stream); });
+}
+
+}  // namespace tq

@@ -373,6 +373,10 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
                  void* y_dev, int y_dtype, hipStream_t stream, const float* gate, void* static_ws, size_t static_cap) {
     const bool lanes = !generic_only && tq::lanes_supported(V.in_features, V.block_size);
     // (the gated store is a feature of the one-row kernels; 16..32 rows: the small-batch kernel where it takes the layer)
+    // (two to four rows on a shared-rotation layer: whole rows per stream, products on the vector ALU, no workspace)
+    if (lanes && !gate && tq::gemv_few_supported(V, batch, device_cu_count()))
+        return hip_ok(tq::launch_gemv_few(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream),
+                      "tq_gemv_few launch") ? 0 : 1;
     const bool skinny = lanes && !gate && tq::skinny_supported(V, x_dtype, batch);
     const bool prefill = lanes && !skinny && !gate && tq::prefill_supported(V, x_dtype, batch);
     if (!prefill && !skinny && (generic_only || !tq::shape_supported(V.in_features, V.block_size))) {
@@ -587,7 +591,13 @@ int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int
             }
             return hip_ok(tq::launch_gemv_wide_group(as, n, device_cu_count(), st), "tq_gemv group launch") ? 0 : 1;
         }
-        if (plain && tq::skinny_group_supported(views, n, x_dtype, batch, device_cu_count())) {
+        if (plain && tq::gemv_few_group_supported(views, n, batch, device_cu_count()))
+            return hip_ok(tq::launch_gemv_few_group(views, n, x_dev, x_dtype, batch, y_devs, y_dtype, device_cu_count(), st),
+                          "tq_gemv_few group launch") ? 0 : 1;
+        // (a layer that a call of its own would send to the kernel above keeps it: the group is then run layer by layer)
+        bool any_few = false;
+        for (int j = 0; j < n; ++j) any_few = any_few || tq::gemv_few_supported(views[j], batch, device_cu_count());
+        if (plain && !any_few && tq::skinny_group_supported(views, n, x_dtype, batch, device_cu_count())) {
             // 2..32 rows on the matrix cores; the per-chunk partial products are per layer and allocated
             // on the first such call (not capturable in a graph), as in tq_linear_forward.
             float* partials[3] = {nullptr, nullptr, nullptr};
@@ -775,7 +785,14 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
                                        m->up->has_fwd_view ? m->up->fwd_view : m->up->view};
         const bool plain = !(m->gate->view.mode >= tq::kShared5 && !m->gate->has_fwd_view) &&
                            !(m->up->view.mode >= tq::kShared5 && !m->up->has_fwd_view);
-        if (plain && tq::skinny_group_supported(both, 2, x_dtype, batch, device_cu_count())) {
+        const bool any_few = tq::gemv_few_supported(both[0], batch, device_cu_count()) ||
+                             tq::gemv_few_supported(both[1], batch, device_cu_count());
+        if (plain && tq::gemv_few_group_supported(both, 2, batch, device_cu_count())) {
+            // two to four rows: gate and up share one launch of the kernel that reads whole rows
+            void* outs[2] = {m->d_gate, m->d_up};
+            if (!hip_ok(tq::launch_gemv_few_group(both, 2, x_dev, x_dtype, batch, outs, tq::kF32, device_cu_count(), st),
+                        "tq_gemv_few group launch")) return 1;
+        } else if (plain && !any_few && tq::skinny_group_supported(both, 2, x_dtype, batch, device_cu_count())) {
             // gate and up share the small-batch kernel and its reduction (workspaces sized by tq_mlp_create)
             void* outs[2] = {m->d_gate, m->d_up};
             float* partials[2] = {static_cast<float*>(m->gate->d_partial), static_cast<float*>(m->up->d_partial)};
