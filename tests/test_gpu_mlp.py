@@ -304,6 +304,44 @@ def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):
         layer.close()
 
 
+@pytest.mark.parametrize("outs,in_f,bs,batch", [((9900, 9850), 10240, 512, 8),     # two sets of four rows: 96 MB and more per layer
+                                                ((4700, 4800, 4690), 14336, 256, 4)])   # images that do not fit LDS
+def test_forward_group_rows_rotated_by_a_kernel_of_their_own(tq, oracle, outs, in_f, bs, batch):
+    """tq_linear_forward_group where the two-to-eight-row kernel takes rows that come rotated: one rotation launch
+    writes every layer's rotation (each layer has a seed of its own) into its part of the first layer's workspace.
+    Bit-identical to separate calls, twice in a row; a sample of the rows against the dense product."""
+    hip = _Hip()
+    cb = oracle.generate_codebook(4)
+    layers, qws = [], []
+    for j, o in enumerate(outs):
+        rng = np.random.default_rng(900 + j)
+        pp = rng.integers(0, 256, size=(o, in_f // 2)).astype(np.uint8)
+        pr = rng.integers(0, 256, size=(o, in_f // 2)).astype(np.uint8)
+        norms = (rng.random(o) + 0.5).astype(np.float32)
+        qw = oracle.QuantizedWeight(pp, pr, norms, np.array([rng.integers(1, 2 ** 32), 0, bs], np.uint32))
+        qws.append(qw)
+        layers.append(tq.TurboQuantLinear(in_f, o, qw, cb, cb, bs))
+    xbits = oracle.f32_to_bf16_bits(np.random.default_rng(batch).standard_normal((batch, in_f)).astype(np.float32))
+    xin = oracle.bf16_bits_to_f32(xbits)
+    dx = hip.upload(xbits)
+    ys_group = [hip.alloc(batch * o * 4) for o in outs]
+    ys_single = [hip.alloc(batch * o * 4) for o in outs]
+    for _ in range(2):
+        tq.forward_group_device(layers, dx, tq.BF16, batch, ys_group, tq.F32)
+    for layer, yp in zip(layers, ys_single):
+        layer.forward_device(dx, tq.BF16, batch, yp, tq.F32)
+    for j, o in enumerate(outs):
+        yg = hip.download(ys_group[j], (batch, o), np.float32)
+        y1 = hip.download(ys_single[j], (batch, o), np.float32)
+        assert np.isfinite(yg).all() and np.array_equal(yg, y1)
+        rows = np.unique(np.concatenate([np.arange(5), np.arange(o - 5, o), np.arange(0, o, 211)]))
+        sub = oracle.QuantizedWeight(qws[j].packed_primary[rows], qws[j].packed_residual[rows], qws[j].norms[rows], qws[j].seeds)
+        assert _rel(yg[:, rows], xin @ oracle.dequantize_weight_cpu(sub, cb, cb, bs).T) < 1e-3
+    hip.free(dx, *ys_group, *ys_single)
+    for layer in layers:
+        layer.close()
+
+
 def _random_groups(n, seed):
     rng = np.random.default_rng(seed)
     cases = []

@@ -83,14 +83,17 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
 bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, int num_cus);
 hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
                                int y_dtype, float* const* partials, int num_cus, hipStream_t stream);
-// Two to four rows on shared-rotation layers (tq_gemv_few.hip): the batch-1 kernel's shape, the products of a
-// decoded weight with every row on the vector ALU.  No workspace (rows wider than 16384 columns use xrot_work).
+// Two to eight rows on shared-rotation layers (tq_gemv_few.hip): the batch-1 kernel's shape (whole weight rows per
+// stream, no cut along K, no second kernel), four weight rows by four activation rows per 4x4x4 matrix block.
+// workspace: gemv_few_workspace_bytes() (0 for most calls of up to four rows: the workgroups rotate the rows
+// themselves); a group needs that of its first layer once per layer.
 bool gemv_few_supported(const LayerView& L, int batch, int num_cus);
+size_t gemv_few_workspace_bytes(const LayerView& L, int batch);
 hipError_t launch_gemv_few(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
-                           int num_cus, hipStream_t stream);
+                           void* workspace, int num_cus, hipStream_t stream);
 bool gemv_few_group_supported(const LayerView* Ls, int n, int batch, int num_cus);
 hipError_t launch_gemv_few_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
-                                 int y_dtype, int num_cus, hipStream_t stream);
+                                 int y_dtype, void* workspace, int num_cus, hipStream_t stream);
 hipError_t launch_wht(const float* in, float* out, int rows, int cols, uint32_t seed,
                       uint32_t block_size, float inv_sqrt_bs, int inverse, hipStream_t stream);
 hipError_t launch_any_nonzero(const uint8_t* data, size_t n, int* flag_dev, hipStream_t stream);

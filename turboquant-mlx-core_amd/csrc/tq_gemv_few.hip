@@ -1,11 +1,11 @@
-// Fused TQ8 dequant + matrix-vector products for gfx950, two to four activation rows, shared-rotation layers
+// Fused TQ8 dequant + matrix-vector products for gfx950, two to eight activation rows, shared-rotation layers
 // (one byte per weight), blocks of at most 512 columns.
 //
 // The batch-1 kernel (tq_gemv_wide.hip) reads the plane in whole rows and runs at the rate of its table reads.  The
 // small-batch kernel (tq_skinny.hip) puts the activation rows on v_mfma_f32_16x16x32_f16, whose operand layout
 // wants 16 weight rows per load instruction, 64 bytes of each; it cuts K over the workgroups and adds the parts in a
-// second kernel.  Up to four activation rows fit v_mfma_f32_4x4x4_16b_f16 instead: 16 independent 4 x 4 x 4 blocks
-// per instruction, block = lane / 4.  The four lanes of a block hold the same 16 columns of four consecutive weight
+// second kernel.  Four activation rows fit v_mfma_f32_4x4x4_16b_f16 instead (five to eight: two such sets on the
+// same decoded weights): 16 independent 4 x 4 x 4 blocks per instruction, block = lane / 4.  The four lanes of a block hold the same 16 columns of four consecutive weight
 // rows (A operand: four decoded weights per step) and of the four activation rows (B operand), so
 //   * a load instruction of a wave fetches 256 contiguous bytes of each of four rows (whole cache lines), a wave
 //     covers U such segments of its four rows, and the waves of a row stream cover the whole row: no cut along K,
@@ -17,7 +17,8 @@
 //     they are rounded, as in the small-batch and prefill kernels), every load slot requested again as soon as it
 //     has been decoded.
 // The activation rows are rotated once per CU (the waves share out the 512-column tiles of all rows and hand the
-// result over through fp16 images in LDS), or, where the images do not fit, by a small kernel of its own.
+// result over through fp16 images in LDS), or, where the images do not fit or there are more than four rows (every
+// CU rotating every row costs 0.15 us per tile and row), by a small kernel of its own into a workspace.
 // Sums are fp32.  The reference has no batched path (src/dequantizer.cpp:545-549: batch is a grid dimension of its
 // per-row kernel).
 #include "tq_device.h"
@@ -28,14 +29,13 @@ namespace tq {
 namespace {
 
 constexpr int kSegCols = 256;                    // columns of a segment: 16 blocks x 16 columns
-constexpr int kFewMaxBatch = 4;
+constexpr int kFewMaxBatch = 8;
 constexpr int kFewImageBytes = 88 * 1024;        // fp16 images of the activation rows in LDS
 constexpr int kFewMaxU = 8;
-constexpr int kFewPartialBytes = 2 * 16 * 32 * 4;   // [2 buffers][<= 16 waves][<= 32 sums]
+constexpr int kFewPartialBytes = 2 * 16 * 32 * 4;   // [2 buffers][<= 16 waves][16 sums x 2 sets of activation rows]
 
-// Quads of weight rows per trip of the main loop.  (Two, for twice the loads in flight and half the cross-wave sums,
+// (Two quads of weight rows per trip of the main loop, for twice the loads in flight and half the cross-wave sums,
 // measured no faster on the large layers and slower on the small ones, whose streams have one or two quads.)
-constexpr int few_quads(int) { return 1; }
 
 struct FewArgs {
     LayerView L;
@@ -45,7 +45,7 @@ struct FewArgs {
     int batch;
     int W, S;            // waves per row quad, quad streams per workgroup
     int w_inv;           // (w * w_inv) >> 8 == w / W
-    int iters;           // uniform trip count: the longest range of a stream, in trips of the main loop
+    int iters;           // uniform trip count: the longest range of a stream, in quads
     int quads_q, quads_rem;
     int ntiles, nt_inv;  // 512-column tiles of a row; (i * nt_inv) >> 16 == i / ntiles for the job numbers in use
 };
@@ -99,14 +99,14 @@ __device__ __forceinline__ void few_rotate(const TileRaw& raw, int x_dtype, bool
     fwht_lanes<8>(v, bs, lane);
 }
 
-// U segments per wave (wave w of a quad stream owns segments U w .. U w + U - 1 of its rows), Q quads of weight
-// rows per trip of the main loop, TL tile jobs of the rotation per wave (PRE: none, the rows come rotated).
-template <int U, int Q, int TL, bool PRE>
+// SETS sets of four activation rows, U segments per wave (wave w of a quad stream owns segments U w .. U w + U - 1 of
+// its rows), TL tile jobs of the rotation per wave (PRE: none, the rows come rotated).
+template <int SETS, int U, int TL, bool PRE>
 __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
+    static_assert(SETS == 1 || PRE, "more than four activation rows come rotated");
     constexpr int kImage = PRE ? 0 : kFewImageBytes;
-    constexpr int kSums = 16 * Q;                  // (weight row of the trip, activation row) pairs
     __shared__ __align__(16) char smem[kLut256Bytes + kFewPartialBytes + kImage];
-    float* const partial = reinterpret_cast<float*>(smem + kLut256Bytes);     // [2][waves][32]
+    float* const partial = reinterpret_cast<float*>(smem + kLut256Bytes);     // [2][waves][SETS][16]
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -116,7 +116,7 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
     const int unit = wave - stream * a.W;
     const uint32_t laneoff = (uint32_t)lane << 2;
     const int out = a.L.out_features, K = a.L.in_features;
-    const int blk = lane >> 2, q = lane & 3;      // block of the matrix instruction; weight row of the quad and activation row
+    const int blk = lane >> 2, q = lane & 3;      // block of the matrix instruction; weight row of the quad and activation row of a set
 
     int col[U];
     bool act[U];
@@ -143,33 +143,33 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
     for (int u = 0; u < U; ++u) off[u] = act[u] ? (uint32_t)q * (uint32_t)K + (uint32_t)col[u] : kNoFetch;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(a.L.packed_combined) + (size_t)r_base * (size_t)K, 0, 0x7fffffff, 0x00020000);
-    uint4 P[Q][U];                            // one load slot per quad and segment, requested again as soon as it is decoded
+    uint4 P[U];                               // one load slot per segment, requested again as soon as it is decoded
     auto fetch = [&](auto Uc, int r0) {
         constexpr int u = decltype(Uc)::value;
-#pragma unroll
-        for (int k = 0; k < Q; ++k)
-            P[k][u] = few_load16(rs, r0 + 4 * k + q < r_end ? off[u] : kNoFetch, (r0 + 4 * k - r_base) * K);
+        P[u] = few_load16(rs, r0 + q < r_end ? off[u] : kNoFetch, (r0 - r_base) * K);
     };
     auto norm_of = [&](int r0) {
-        const int rn = r0 + ((lane >> 2) & (4 * Q - 1));
+        const int rn = r0 + ((lane >> 2) & 3);
         return a.L.norms[rn < out ? rn : out - 1];
     };
 
     // Small requests first (loads complete in order): the activation tiles this wave rotates, or its columns of
     // the rotated rows; then the norms of the first quad and the first weights.
-    uint32_t xh[U][8];                        // fp16 pairs of activation row q: columns 2 j, 2 j + 1 of segment u
+    uint32_t xh[SETS][U][8];                  // fp16 pairs of activation row q + 4 e: columns 2 j, 2 j + 1 of segment u
     TileRaw raw[PRE ? 1 : TL];
     const int jobs = a.batch * a.ntiles;
     if constexpr (PRE) {
         const char* xr = static_cast<const char*>(a.x);
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const bool on = act[u] && q < a.batch;
-            const uint4* p = reinterpret_cast<const uint4*>(xr + ((size_t)(on ? q : 0) * K + (on ? col[u] : 0)) * 2);
-            const uint4 lo = p[0], hi = p[1];
-            xh[u][0] = lo.x; xh[u][1] = lo.y; xh[u][2] = lo.z; xh[u][3] = lo.w;
-            xh[u][4] = hi.x; xh[u][5] = hi.y; xh[u][6] = hi.z; xh[u][7] = hi.w;
-        }
+        for (int e = 0; e < SETS; ++e)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool on = act[u] && q + 4 * e < a.batch;
+                const uint4* p = reinterpret_cast<const uint4*>(xr + ((size_t)(on ? q + 4 * e : 0) * K + (on ? col[u] : 0)) * 2);
+                const uint4 lo = p[0], hi = p[1];
+                xh[e][u][0] = lo.x; xh[e][u][1] = lo.y; xh[e][u][2] = lo.z; xh[e][u][3] = lo.w;
+                xh[e][u][4] = hi.x; xh[e][u][5] = hi.y; xh[e][u][6] = hi.z; xh[e][u][7] = hi.w;
+            }
     } else {
 #pragma unroll
         for (int k = 0; k < TL; ++k) {            // jobs past the last re-read the start of the first row and are not used
@@ -202,9 +202,11 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
     if constexpr (PRE) {
         __syncthreads();                                       // table visible to every wave
 #pragma unroll
-        for (int u = 0; u < U; ++u)
+        for (int e = 0; e < SETS; ++e)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) xh[u][j] = (act[u] && q < a.batch) ? xh[u][j] : 0u;     // idle lanes contribute 0
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) xh[e][u][j] = (act[u] && q + 4 * e < a.batch) ? xh[e][u][j] : 0u;   // idle lanes contribute 0
     } else {
         char* const image = smem + kLut256Bytes + kFewPartialBytes;               // [batch][K] fp16
         float sg[8];
@@ -227,8 +229,8 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
             const bool on = act[u] && q < a.batch;
             const uint4* p = reinterpret_cast<const uint4*>(image + ((size_t)(on ? q : 0) * K + (on ? col[u] : 0)) * 2);
             const uint4 lo = p[0], hi = p[1];
-            xh[u][0] = on ? lo.x : 0u; xh[u][1] = on ? lo.y : 0u; xh[u][2] = on ? lo.z : 0u; xh[u][3] = on ? lo.w : 0u;
-            xh[u][4] = on ? hi.x : 0u; xh[u][5] = on ? hi.y : 0u; xh[u][6] = on ? hi.z : 0u; xh[u][7] = on ? hi.w : 0u;
+            xh[0][u][0] = on ? lo.x : 0u; xh[0][u][1] = on ? lo.y : 0u; xh[0][u][2] = on ? lo.z : 0u; xh[0][u][3] = on ? lo.w : 0u;
+            xh[0][u][4] = on ? hi.x : 0u; xh[0][u][5] = on ? hi.y : 0u; xh[0][u][6] = on ? hi.z : 0u; xh[0][u][7] = on ? hi.w : 0u;
         }
     }
     // The other load slots are requested behind the barrier: a wave whose requests queue up in the memory pipeline
@@ -249,24 +251,23 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
     };
 
     for (int it = 0; it < a.iters; ++it) {
-        const int r0 = r_begin + 4 * Q * it;
-        const float nrm_next = norm_of(r0 + 4 * Q);
-        few_f4 acc[Q];                                         // results D[i][q] of the lane's block: weight rows r0 + 4 k + i
+        const int r0 = r_begin + 4 * it;
+        const float nrm_next = norm_of(r0 + 4);
+        few_f4 acc[SETS];                                      // results D[i][q] of the lane's block: weight rows r0 + i
 #pragma unroll
-        for (int k = 0; k < Q; ++k) acc[k] = few_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int e = 0; e < SETS; ++e) acc[e] = few_f4{0.0f, 0.0f, 0.0f, 0.0f};
         auto segment = [&](auto Uc) {
             constexpr int u = decltype(Uc)::value;
-            uint4 p[Q];
+            const uint4 p = P[u];
+            fetch(Uc, r0 + 4);
+            const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
-            for (int k = 0; k < Q; ++k) p[k] = P[k][u];
-            fetch(Uc, r0 + 4 * Q);
+            for (int d = 0; d < 4; ++d) {
+                const few_h4 wq = operand(pw[d]);
 #pragma unroll
-            for (int k = 0; k < Q; ++k) {
-                const uint32_t pw[4] = {p[k].x, p[k].y, p[k].z, p[k].w};
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    const few_u2 xb = {xh[u][2 * d], xh[u][2 * d + 1]};
-                    acc[k] = __builtin_amdgcn_mfma_f32_4x4x4f16(operand(pw[d]), __builtin_bit_cast(few_h4, xb), acc[k], 0, 0, 0);
+                for (int e = 0; e < SETS; ++e) {
+                    const few_u2 xb = {xh[e][u][2 * d], xh[e][u][2 * d + 1]};
+                    acc[e] = __builtin_amdgcn_mfma_f32_4x4x4f16(wq, __builtin_bit_cast(few_h4, xb), acc[e], 0, 0, 0);
                 }
             }
         };
@@ -280,35 +281,45 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
         if constexpr (U > 7) segment(std::integral_constant<int, 7>{});
 
         // Sum over the 16 blocks (the columns of the wave): afterwards every lane holds the wave total of weight row
-        // (lane / 4) % (4 Q) of the trip and activation row lane % 4.
-        float v[4 * Q];
+        // (lane / 4) % 4 of the quad and activation row lane % 4 of each set.
+        float total[SETS];
 #pragma unroll
-        for (int k = 0; k < Q; ++k)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) v[4 * k + i] = acc[k][i];
-        const float total = reduce_rec<4 * Q, 4>(v, lane);
-        const int r = r0 + ((lane >> 2) & (4 * Q - 1));
-        const bool owner = lane < kSums && q < a.batch && r < r_end;
-        float t = total;
+        for (int e = 0; e < SETS; ++e) {
+            float v[4] = {acc[e][0], acc[e][1], acc[e][2], acc[e][3]};
+            total[e] = reduce_rec<4, 4>(v, lane);
+        }
+        const int r = r0 + ((lane >> 2) & 3);
+        const bool owner = lane < 16 && r < r_end;
         bool store = owner;
         if (a.W > 1) {                                         // cross-wave sum of the row's segments
             float* const buf_base = partial + (it & 1) * (16 * 32);
-            if (lane < kSums) buf_base[wave * 32 + lane] = total;
+            if (lane < 16) {
+#pragma unroll
+                for (int e = 0; e < SETS; ++e) buf_base[wave * 32 + 16 * e + lane] = total[e];
+            }
             __syncthreads();
             store = owner && unit == 0;
             if (store) {
-                t = 0.0f;
-                for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * 32 + lane];
+#pragma unroll
+                for (int e = 0; e < SETS; ++e) {
+                    float t = 0.0f;
+                    for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * 32 + 16 * e + lane];
+                    total[e] = t;
+                }
             }
         }
-        if (store) store_scalar(a.y, a.y_dtype, (size_t)q * out + r, t * (a.L.inv_scale * nrm));
+        if (store) {
+#pragma unroll
+            for (int e = 0; e < SETS; ++e)
+                if (q + 4 * e < a.batch) store_scalar(a.y, a.y_dtype, (size_t)(q + 4 * e) * out + r, total[e] * (a.L.inv_scale * nrm));
+        }
         nrm = nrm_next;
     }
 }
 
-template <int U, int Q, int TL, bool PRE>
+template <int SETS, int U, int TL, bool PRE>
 __global__ __launch_bounds__(1024) void tq_gemv_few_kernel(FewArgs a) {
-    few_body<U, Q, TL, PRE>(a, (int)blockIdx.x);
+    few_body<SETS, U, TL, PRE>(a, (int)blockIdx.x);
 }
 
 // Two or three layers of equal width on the same activation rows (q, k, v or gate, up), one launch: the
@@ -317,49 +328,59 @@ struct FewGroup {
     FewArgs a[3];
     int first[4];          // layer j owns workgroups first[j] .. first[j + 1] - 1
 };
-template <int U, int TL>
+template <int SETS, int U, int TL, bool PRE>
 __global__ __launch_bounds__(1024) void tq_gemv_few_group_kernel(FewGroup g) {
     const int b = (int)blockIdx.x;
     const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
-    few_body<U, few_quads(U), TL, false>(g.a[j], b - g.first[j]);
+    few_body<SETS, U, TL, PRE>(g.a[j], b - g.first[j]);
 }
 
-// Rotated, scaled activation rows as fp16 [batch, in] for the layers whose images do not fit LDS: one wave per
-// 512-column tile and row.
-__global__ __launch_bounds__(64) void tq_rotate_rows_f16_kernel(const void* x, int x_dtype, int K, uint32_t seed,
-                                                                 uint32_t bs, float scale, uint16_t* out) {
-    const int lane = threadIdx.x, t = blockIdx.y;
+// Rotated, scaled activation rows as fp16 [batch, in] for the calls whose workgroups do not rotate them themselves:
+// one wave per 512-column tile, row and layer (the layers of a group have rotations of their own).
+struct FewRotate {
+    const void* x;
+    int x_dtype, K;
+    uint32_t seed[3], bs[3];
+    float scale[3];
+    uint16_t* out[3];
+};
+__global__ __launch_bounds__(64) void tq_rotate_rows_f16_kernel(FewRotate r) {
+    const int lane = threadIdx.x, t = blockIdx.y, j = blockIdx.z;
     const int c = blockIdx.x * kTile + lane * 8;
-    const TileRaw raw = load_tile_raw(x, x_dtype, (size_t)t * K, c < K ? c : 0);
+    const TileRaw raw = load_tile_raw(r.x, r.x_dtype, (size_t)t * r.K, c < r.K ? c : 0);
     float v[8];
-    rotate_tile(raw, x_dtype, c, c < K, seed, bs, lane, v);
-    if (c < K) *reinterpret_cast<uint4*>(out + (size_t)t * K + c) = few_pack8(v, scale);
+    rotate_tile(raw, r.x_dtype, c, c < r.K, r.seed[j], r.bs[j], lane, v);
+    if (c < r.K) *reinterpret_cast<uint4*>(r.out[j] + (size_t)t * r.K + c) = few_pack8(v, r.scale[j]);
 }
 
-// The shape of a launch: segments per wave, waves per row quad, quad streams, rotation jobs per wave, whether the
-// rows come rotated.  Among the splits of the row's segments over 1 to 16 waves with at most kFewMaxU segments each,
-// the one that keeps most lanes busy (segments that exist, waves that exist; on a tie the one nearest four
-// segments per wave: streams short enough for layers of a few thousand rows, long enough between two barriers).  A function
-// of the width and the batch alone: the order in which a row's products are added depends on it, and a layer must
-// give the same bits in a launch of its own and in one it shares.
-struct FewShape { int U, W, S, threads, tl; bool pre; };
+// The shape of a launch: sets of four activation rows, segments per wave, waves per row quad, quad streams,
+// rotation jobs per wave, whether the rows come rotated.  Among the splits of the row's segments over 1 to 16 waves
+// with at most 8 segments each (4 with two sets: the registers), the one that keeps most lanes busy (segments that
+// exist, waves that exist; on a tie the one nearest four segments per wave: streams short enough for layers of a
+// few thousand rows, long enough between two barriers).  A function of the width and the batch alone: the order in
+// which a row's products are added depends on it, and a layer must give the same bits in a launch of its own and
+// in one it shares.
+struct FewShape { int sets, U, W, S, threads, tl; bool pre; };
 FewShape few_shape(int K, int batch) {
     FewShape s{};
+    s.sets = batch > 4 ? 2 : 1;
+    const int max_u = s.sets == 2 ? 4 : kFewMaxU;
     const int segs = (K + kSegCols - 1) / kSegCols;
     double best = -1.0;
     for (int W = 1; W <= 16; ++W) {
         int U = (segs + W - 1) / W;
-        if (U > kFewMaxU) continue;
+        if (U > max_u) continue;
         if (U < 2) U = 2;
         const int S = 16 / W;
         const double eff = (double)segs / (W * U) * (W * S) / 16.0;
         const bool tie = eff > best - 1e-9 && (U - 4) * (U - 4) < (s.U - 4) * (s.U - 4);
         if (eff > best + 1e-9 || tie) { best = eff; s.U = U; s.W = W; s.S = S; }
     }
+    if (best < 0.0) return s;                                // (wider than 16 waves of max_u segments: W == 0)
     s.threads = s.W * s.S * kWave;
     const int ntiles = (K + kTile - 1) / kTile, waves = s.W * s.S;
     const int per_wave = (batch * ntiles + waves - 1) / waves;
-    s.pre = (size_t)batch * K * 2 > (size_t)kFewImageBytes || per_wave > 6;
+    s.pre = s.sets == 2 || (size_t)batch * K * 2 > (size_t)kFewImageBytes || per_wave > 6;
     s.tl = per_wave <= 3 ? 3 : 6;
     return s;
 }
@@ -371,38 +392,42 @@ void few_ranges(FewArgs& a, const FewShape& s, int grid, int batch) {
     a.w_inv = (256 + s.W - 1) / s.W;
     a.quads_q = quads / ts;
     a.quads_rem = quads % ts;
-    a.iters = (a.quads_q + (a.quads_rem ? 1 : 0) + few_quads(s.U) - 1) / few_quads(s.U);
+    a.iters = a.quads_q + (a.quads_rem ? 1 : 0);
     a.ntiles = (a.L.in_features + kTile - 1) / kTile;
     a.nt_inv = 65536 / a.ntiles + 1;       // exact quotients for job numbers below 16 x 6 (at most 64 tiles per row)
 }
 
-template <int U>
-hipError_t launch_few_u(const FewArgs& a, const FewShape& s, int grid, hipStream_t stream) {
+// GROUP: FewGroup and the kernel that serves several layers; otherwise FewArgs.
+template <int U, bool GROUP, typename Args>
+hipError_t launch_few_u(const Args& a, const FewShape& s, int grid, hipStream_t stream) {
     const dim3 g(grid), b(s.threads);
-    if (s.pre) hipLaunchKernelGGL((tq_gemv_few_kernel<U, few_quads(U), 1, true>), g, b, 0, stream, a);
-    else if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_kernel<U, few_quads(U), 3, false>), g, b, 0, stream, a);
-    else hipLaunchKernelGGL((tq_gemv_few_kernel<U, few_quads(U), 6, false>), g, b, 0, stream, a);
+    if constexpr (GROUP) {
+        if (s.sets == 2) {
+            if constexpr (U <= 4) hipLaunchKernelGGL((tq_gemv_few_group_kernel<2, U, 1, true>), g, b, 0, stream, a);
+            else return hipErrorInvalidValue;                  // few_shape() rules this out
+        }
+        else if (s.pre) hipLaunchKernelGGL((tq_gemv_few_group_kernel<1, U, 1, true>), g, b, 0, stream, a);
+        else if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_group_kernel<1, U, 3, false>), g, b, 0, stream, a);
+        else hipLaunchKernelGGL((tq_gemv_few_group_kernel<1, U, 6, false>), g, b, 0, stream, a);
+    } else {
+        if (s.sets == 2) {
+            if constexpr (U <= 4) hipLaunchKernelGGL((tq_gemv_few_kernel<2, U, 1, true>), g, b, 0, stream, a);
+            else return hipErrorInvalidValue;
+        }
+        else if (s.pre) hipLaunchKernelGGL((tq_gemv_few_kernel<1, U, 1, true>), g, b, 0, stream, a);
+        else if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_kernel<1, U, 3, false>), g, b, 0, stream, a);
+        else hipLaunchKernelGGL((tq_gemv_few_kernel<1, U, 6, false>), g, b, 0, stream, a);
+    }
     return hipGetLastError();
 }
 
-template <int U>
-hipError_t launch_few_group_u(const FewGroup& g, const FewShape& s, int grid, hipStream_t stream) {
-    const dim3 gr(grid), b(s.threads);
-    if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_group_kernel<U, 3>), gr, b, 0, stream, g);
-    else hipLaunchKernelGGL((tq_gemv_few_group_kernel<U, 6>), gr, b, 0, stream, g);
-    return hipGetLastError();
-}
-
-}  // namespace
-
-namespace {
 // What the kernel asks of a layer whatever the launch: shared rotation, centroid sums that fit fp16, blocks of at
 // most 512 columns (a block never leaves the tile a wave rotates), rows of at most 64 tiles.
 bool few_layer_ok(const LayerView& L, int batch) {
     if (batch < 2 || batch > kFewMaxBatch) return false;
     if (L.mode != kSharedLut || !L.packed_combined || !L.fp16_centroids_ok) return false;
     if (!lanes_supported(L.in_features, L.block_size) || L.block_size > (uint32_t)kTile) return false;
-    return L.in_features <= 16 * kFewMaxU * kSegCols;
+    return L.in_features <= 16 * kFewMaxU * kSegCols && few_shape(L.in_features, batch).W > 0;
 }
 // A stream's share of the plane stays below the 2 GB of its buffer descriptor (one stream per CU at least).
 bool few_share_ok(const LayerView& L, int num_cus) {
@@ -410,28 +435,23 @@ bool few_share_ok(const LayerView& L, int num_cus) {
     const long long max_rows = (L.out_features + cus - 1) / cus + 24;
     return (unsigned long long)max_rows * (unsigned long long)L.in_features < (1ull << 31);
 }
+// Where the rotated rows of a call go when its workgroups do not rotate them: the layer's scratch row (rows wider
+// than 16384 columns have one: 2 x in floats = 4 rows of fp16) or a workspace of the caller.
+bool few_uses_scratch_row(const LayerView& L, int batch) { return batch <= 4 && L.xrot_work != nullptr; }
 // Every workgroup rotates all the activation rows for itself: about 0.15 us per 512-column tile and row, whatever
 // the size of the plane, where the small-batch kernel pays 4 us for its second kernel and loses about 0.06 us per MB
 // of plane to its load pattern (same-box comparisons of the two on eleven shapes, weight copies cycled).  Few rows
 // of a wide plane go to the small-batch kernel.  (Up to 40 tiles whatever the plane: the layers of a group, large
-// and small, should agree on the kernel, or the group is run layer by layer.)
-bool few_worth_it(int batch, int K, long long plane_bytes) {
+// and small, should agree on the kernel, or the group is run layer by layer.)  Rows that come rotated cost a kernel
+// of their own, which only a plane of some size repays.
+bool few_worth_it(const FewShape& s, int batch, int K, long long plane_bytes) {
+    // (five to eight rows, same-box comparisons with the small-batch kernel: 27648 x 5120 35.1 against 42.2 us,
+    // 28672 x 8192 47.7 / 59.7, but 14336 x 4096 23.7 / 20.7, 8192 x 8192 23.8 / 21.8, 5120 x 5120 17.1 / 14.3)
+    if (s.pre) return plane_bytes >= (s.sets == 2 ? (96ll << 20) : (64ll << 20));
     const long long jobs = (long long)batch * ((K + kTile - 1) / kTile);
     return jobs <= 40 || jobs * 5 <= 135 + plane_bytes / 500000;           // jobs <= 27 + 0.4 per MB
 }
-}  // namespace
 
-// Two to four rows of any activation type.
-bool gemv_few_supported(const LayerView& L, int batch, int num_cus) {
-    if (!few_layer_ok(L, batch) || !few_share_ok(L, num_cus)) return false;
-    const FewShape s = few_shape(L.in_features, batch);
-    // (rows that come rotated: the scratch row holds them, 2 x in floats = 4 rows of fp16; the rotation is a
-    // kernel of its own, which only a plane of some size repays)
-    if (s.pre) return L.xrot_work != nullptr && (long long)L.out_features * L.in_features >= (64ll << 20);
-    return few_worth_it(batch, L.in_features, (long long)L.out_features * L.in_features);
-}
-
-namespace {
 template <typename F>
 hipError_t few_dispatch_u(int U, F&& f) {
     switch (U) {
@@ -445,42 +465,69 @@ hipError_t few_dispatch_u(int U, F&& f) {
         default: return hipErrorInvalidValue;
     }
 }
+
+// The rotation kernel of a call whose rows come rotated: layer j's rows go to its scratch row or to the j-th part
+// of the workspace; as[j].x is set to them.
+hipError_t few_rotate_rows(FewArgs* as, int n, const void* x, int x_dtype, int batch, void* workspace, hipStream_t stream) {
+    FewRotate r{};
+    r.x = x; r.x_dtype = x_dtype; r.K = as[0].L.in_features;
+    const size_t part = ((size_t)batch * r.K * 2 + 255) & ~(size_t)255;
+    for (int j = 0; j < n; ++j) {
+        const LayerView& L = as[j].L;
+        r.seed[j] = L.seed_primary; r.bs[j] = L.block_size; r.scale[j] = L.inv_sqrt_bs;
+        r.out[j] = few_uses_scratch_row(L, batch) ? reinterpret_cast<uint16_t*>(L.xrot_work)
+                 : workspace ? reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + j * part) : nullptr;
+        if (!r.out[j]) return hipErrorInvalidValue;
+        as[j].x = r.out[j];
+    }
+    hipLaunchKernelGGL(tq_rotate_rows_f16_kernel, dim3((r.K + kTile - 1) / kTile, batch, n), dim3(64), 0, stream, r);
+    return hipGetLastError();
+}
+
 }  // namespace
 
+// Two to eight rows of any activation type.
+bool gemv_few_supported(const LayerView& L, int batch, int num_cus) {
+    if (!few_layer_ok(L, batch) || !few_share_ok(L, num_cus)) return false;
+    return few_worth_it(few_shape(L.in_features, batch), batch, L.in_features, (long long)L.out_features * L.in_features);
+}
+
+// Bytes of workspace a call needs for its rotated rows (0: none).
+size_t gemv_few_workspace_bytes(const LayerView& L, int batch) {
+    if (!few_layer_ok(L, batch) || !few_shape(L.in_features, batch).pre || few_uses_scratch_row(L, batch)) return 0;
+    return ((size_t)batch * L.in_features * 2 + 255) & ~(size_t)255;
+}
+
 hipError_t launch_gemv_few(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
-                           int num_cus, hipStream_t stream) {
+                           void* workspace, int num_cus, hipStream_t stream) {
     const FewShape s = few_shape(L.in_features, batch);
     FewArgs a{};
     a.L = L; a.x = x; a.y = y; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
     if (s.pre) {
-        uint16_t* const xr = reinterpret_cast<uint16_t*>(L.xrot_work);
-        hipLaunchKernelGGL(tq_rotate_rows_f16_kernel, dim3((L.in_features + kTile - 1) / kTile, batch), dim3(64), 0, stream,
-                           x, x_dtype, L.in_features, L.seed_primary, L.block_size, L.inv_sqrt_bs, xr);
-        const hipError_t e = hipGetLastError();
+        const hipError_t e = few_rotate_rows(&a, 1, x, x_dtype, batch, workspace, stream);
         if (e != hipSuccess) return e;
-        a.x = xr;
     }
     const int quads = (L.out_features + 3) / 4;
     int grid = (quads + s.S - 1) / s.S;
     if (grid > num_cus) grid = num_cus;
     if (grid < 1) grid = 1;
     few_ranges(a, s, grid, batch);
-    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value>(a, s, grid, stream); });
+    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, false>(a, s, grid, stream); });
 }
 
-// Layers that can share a launch: two or three of equal width, each taken by the kernel in a launch of its own, whose
-// rows the workgroups rotate themselves.
+// Layers that can share a launch: two or three of equal width, each taken by the kernel in a launch of its own.
 bool gemv_few_group_supported(const LayerView* Ls, int n, int batch, int num_cus) {
     if (n < 2 || n > 3 || num_cus < n) return false;
     for (int j = 0; j < n; ++j) {
         if (Ls[j].in_features != Ls[0].in_features) return false;
         if (!gemv_few_supported(Ls[j], batch, 1)) return false;      // (1 CU: the strictest bound on a stream's share)
     }
-    return !few_shape(Ls[0].in_features, batch).pre;
+    return true;
 }
 
+// workspace: n x gemv_few_workspace_bytes() of the first layer (every layer has a rotation of its own).
 hipError_t launch_gemv_few_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
-                                 int y_dtype, int num_cus, hipStream_t stream) {
+                                 int y_dtype, void* workspace, int num_cus, hipStream_t stream) {
     long long total = 0;
     for (int j = 0; j < n; ++j) total += Ls[j].out_features;
     const FewShape s = few_shape(Ls[0].in_features, batch);
@@ -502,7 +549,11 @@ hipError_t launch_gemv_few_group(const LayerView* Ls, int n, const void* x, int 
         a.L = Ls[j]; a.x = x; a.y = ys[j]; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
         few_ranges(a, s, blocks[j], batch);
     }
-    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_group_u<decltype(Uc)::value>(g, s, used, stream); });
+    if (s.pre) {
+        const hipError_t e = few_rotate_rows(g.a, n, x, x_dtype, batch, workspace, stream);
+        if (e != hipSuccess) return e;
+    }
+    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, true>(g, s, used, stream); });
 }
 
 }  // namespace tq

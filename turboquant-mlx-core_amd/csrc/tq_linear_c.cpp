@@ -373,10 +373,21 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
                  void* y_dev, int y_dtype, hipStream_t stream, const float* gate, void* static_ws, size_t static_cap) {
     const bool lanes = !generic_only && tq::lanes_supported(V.in_features, V.block_size);
     // (the gated store is a feature of the one-row kernels; 16..32 rows: the small-batch kernel where it takes the layer)
-    // (two to four rows on a shared-rotation layer: whole rows per stream, products on the vector ALU, no workspace)
-    if (lanes && !gate && tq::gemv_few_supported(V, batch, device_cu_count()))
-        return hip_ok(tq::launch_gemv_few(V, x_dev, x_dtype, batch, y_dev, y_dtype, device_cu_count(), stream),
+    // (two to eight rows on a shared-rotation layer: whole weight rows per stream, 4 x 4 x 4 matrix blocks; a
+    // workspace only where the rows are rotated by a kernel of their own)
+    if (lanes && !gate && tq::gemv_few_supported(V, batch, device_cu_count())) {
+        const size_t need = tq::gemv_few_workspace_bytes(V, batch);
+        void* few_ws = nullptr;
+        if (need && static_ws) {
+            if (need > static_cap) { set_error("tq_linear_forward_static: the workspace of this call does not fit the static array"); return 1; }
+            few_ws = static_ws;
+        } else if (need) {
+            if (!ensure_stage(&h->d_work, &h->work_bytes, need, stream, &h->retired)) return 1;
+            few_ws = h->d_work;
+        }
+        return hip_ok(tq::launch_gemv_few(V, x_dev, x_dtype, batch, y_dev, y_dtype, few_ws, device_cu_count(), stream),
                       "tq_gemv_few launch") ? 0 : 1;
+    }
     const bool skinny = lanes && !gate && tq::skinny_supported(V, x_dtype, batch);
     const bool prefill = lanes && !skinny && !gate && tq::prefill_supported(V, x_dtype, batch);
     if (!prefill && !skinny && (generic_only || !tq::shape_supported(V.in_features, V.block_size))) {
@@ -518,6 +529,16 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
     } catch (...) { set_error("tq_linear_forward: exception"); return 1; }
 }
 
+namespace {
+// Workspace of the two-to-eight-row kernel for every batch up to max_batch, thrice: the first layer of a group holds
+// the rotated rows of all its layers.
+size_t few_reserve_bytes(const tq::LayerView& V, int max_batch) {
+    size_t need = 0;
+    for (int b = 2; b <= max_batch && b <= 8; ++b) need = std::max(need, 3 * tq::gemv_few_workspace_bytes(V, b));
+    return need;
+}
+}  // namespace
+
 int tq_linear_reserve(tq_linear_t h, int max_batch) {
     try {
         if (!h || max_batch <= 0) { set_error("tq_linear_reserve: bad argument"); return 1; }
@@ -531,6 +552,7 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
                 const size_t small = sk ? tq::skinny_workspace_bytes(P, rows) : 0;
                 const size_t big = max_batch >= 16 ? tq::prefill_reserve_bytes(P, max_batch, device_cu_count()) : 0;
                 work = std::max(work, std::max(small, big));
+                work = std::max(work, few_reserve_bytes(P, max_batch));
                 if (sk) part = std::max(part, tq::skinny_partial_bytes(P, rows));
             }
             if (!ensure_stage(&h->d_work, &h->work_bytes, work, nullptr, &h->retired)) return 1;
@@ -545,7 +567,9 @@ int tq_linear_reserve(tq_linear_t h, int max_batch) {
         const size_t small = sk ? tq::skinny_workspace_bytes(V, rows) : 0;
         const bool pf = tq::lanes_supported(V.in_features, V.block_size) && max_batch >= 16 && tq::prefill_supported(V, tq::kBF16, max_batch);
         const size_t big = pf ? tq::prefill_reserve_bytes(V, max_batch, device_cu_count()) : 0;
-        if ((small || big) && !ensure_stage(&h->d_work, &h->work_bytes, small > big ? small : big, nullptr, &h->retired)) return 1;
+        const size_t few = few_reserve_bytes(V, max_batch);
+        const size_t work = std::max(few, std::max(small, big));
+        if (work && !ensure_stage(&h->d_work, &h->work_bytes, work, nullptr, &h->retired)) return 1;
         if (sk && !ensure_stage(&h->d_partial, &h->partial_bytes, tq::skinny_partial_bytes(V, rows), nullptr, &h->retired)) return 1;
         return 0;
     } catch (...) { set_error("tq_linear_reserve: exception"); return 1; }
@@ -591,9 +615,15 @@ int tq_linear_forward_group(const tq_linear_t* hs, int n, const void* x_dev, int
             }
             return hip_ok(tq::launch_gemv_wide_group(as, n, device_cu_count(), st), "tq_gemv group launch") ? 0 : 1;
         }
-        if (plain && tq::gemv_few_group_supported(views, n, batch, device_cu_count()))
-            return hip_ok(tq::launch_gemv_few_group(views, n, x_dev, x_dtype, batch, y_devs, y_dtype, device_cu_count(), st),
+        if (plain && tq::gemv_few_group_supported(views, n, batch, device_cu_count())) {
+            // (rows that a kernel of its own rotates: one part of the first layer's workspace per layer; allocated on
+            // the first such call, not capturable in a graph, as in tq_linear_forward)
+            const size_t need = n * tq::gemv_few_workspace_bytes(views[0], batch);
+            if (need && !ensure_stage(&hs[0]->d_work, &hs[0]->work_bytes, need, st, &hs[0]->retired)) return 1;
+            return hip_ok(tq::launch_gemv_few_group(views, n, x_dev, x_dtype, batch, y_devs, y_dtype,
+                                                    need ? hs[0]->d_work : nullptr, device_cu_count(), st),
                           "tq_gemv_few group launch") ? 0 : 1;
+        }
         // (a layer that a call of its own would send to the kernel above keeps it: the group is then run layer by layer)
         bool any_few = false;
         for (int j = 0; j < n; ++j) any_few = any_few || tq::gemv_few_supported(views[j], batch, device_cu_count());
@@ -790,7 +820,10 @@ int tq_mlp_forward(tq_mlp_t m, const void* x_dev, int x_dtype, int batch, void* 
         if (plain && tq::gemv_few_group_supported(both, 2, batch, device_cu_count())) {
             // two to four rows: gate and up share one launch of the kernel that reads whole rows
             void* outs[2] = {m->d_gate, m->d_up};
-            if (!hip_ok(tq::launch_gemv_few_group(both, 2, x_dev, x_dtype, batch, outs, tq::kF32, device_cu_count(), st),
+            const size_t need = 2 * tq::gemv_few_workspace_bytes(both[0], batch);      // (sized by tq_mlp_create)
+            if (need && !ensure_stage(&m->gate->d_work, &m->gate->work_bytes, need, st, &m->gate->retired)) return 1;
+            if (!hip_ok(tq::launch_gemv_few_group(both, 2, x_dev, x_dtype, batch, outs, tq::kF32,
+                                                  need ? m->gate->d_work : nullptr, device_cu_count(), st),
                         "tq_gemv_few group launch")) return 1;
         } else if (plain && !any_few && tq::skinny_group_supported(both, 2, x_dtype, batch, device_cu_count())) {
             // gate and up share the small-batch kernel and its reduction (workspaces sized by tq_mlp_create)
