@@ -482,13 +482,27 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     # five to eight rows: two sets of four on the same decoded weights, planes of 96 MB and more
     (19701, 5120, 512, 8), (12300, 8192, 256, 5), (6200, 16384, 512, 7), (66000, 1536, 512, 6), (49500, 2048, 128, 8)])
 def test_two_to_eight_rows_whole_row_kernel(tq, oracle, out, inf, bs, batch):
+    _whole_row_kernel_case(tq, oracle, "shared", out, inf, bs, batch)
+
+
+@pytest.mark.parametrize("mode,out,inf,bs,batch", [
+    # nibble planes of 96 MB and more: dual rotation (primary segments, then residual ones; two to four units of 512
+    # columns per wave), five to eight rows where the row's units fill 14 waves and more, and primary only
+    ("dual", 19701, 5120, 512, 4), ("dual", 12300, 8192, 256, 3), ("dual", 12300, 8192, 512, 7), ("dual", 33000, 3072, 128, 2),
+    ("dual", 6200, 16384, 512, 4), ("dual", 25000, 4096, 512, 8), ("dual", 9000, 11264, 256, 3),
+    ("primary_only", 39400, 5120, 512, 4), ("primary_only", 50000, 4096, 256, 6)])
+def test_two_to_eight_rows_whole_row_kernel_nibble_planes(tq, oracle, mode, out, inf, bs, batch):
+    _whole_row_kernel_case(tq, oracle, mode, out, inf, bs, batch)
+
+
+def _whole_row_kernel_case(tq, oracle, mode, out, inf, bs, batch):
     """2..8 rows on a shared-rotation layer: the kernel that reads whole weight rows per stream (four weight rows by
     four activation rows per v_mfma_f32_4x4x4_16b_f16 block, fp16 weights and rotated activations, fp32 sums, the
     cross-wave sum inside the workgroup).  1e-3 relative L2 against the oracle for every activation type (5e-3 with a
     bf16 output), every activation row by itself, every row equal to its batch-1 result within the same bound, and
     the same bits on a second call.  Planes of more than 40 MB: a sample of the weight rows (the first and last
     quads, every 61st row) against the oracle, all of them for finiteness."""
-    qw, cb = _packed_layer(oracle, out, inf, bs, "shared", out + inf + batch)
+    qw, cb = _packed_layer(oracle, out, inf, bs, mode, out + inf + batch)
     x32 = np.random.default_rng(batch + inf).standard_normal((batch, inf)).astype(np.float32)
     xbits = oracle.f32_to_bf16_bits(x32)
     rows = np.arange(out) if out * inf <= 40 << 20 else \

@@ -304,9 +304,11 @@ def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):
         layer.close()
 
 
-@pytest.mark.parametrize("outs,in_f,bs,batch", [((9900, 9850), 10240, 512, 8),     # two sets of four rows: 96 MB and more per layer
-                                                ((4700, 4800, 4690), 14336, 256, 4)])   # images that do not fit LDS
-def test_forward_group_rows_rotated_by_a_kernel_of_their_own(tq, oracle, outs, in_f, bs, batch):
+@pytest.mark.parametrize("outs,in_f,bs,batch,dual", [((9900, 9850), 10240, 512, 8, False),     # two sets of four rows: 96 MB and more per layer
+                                                     ((4700, 4800, 4690), 14336, 256, 4, False),   # images that do not fit LDS
+                                                     ((19701, 19800), 5120, 512, 3, True),         # nibble planes: two rotations per layer
+                                                     ((12300, 12400), 8192, 256, 6, True)])
+def test_forward_group_rows_rotated_by_a_kernel_of_their_own(tq, oracle, outs, in_f, bs, batch, dual):
     """tq_linear_forward_group where the two-to-eight-row kernel takes rows that come rotated: one rotation launch
     writes every layer's rotation (each layer has a seed of its own) into its part of the first layer's workspace.
     Bit-identical to separate calls, twice in a row; a sample of the rows against the dense product."""
@@ -318,7 +320,7 @@ def test_forward_group_rows_rotated_by_a_kernel_of_their_own(tq, oracle, outs, i
         pp = rng.integers(0, 256, size=(o, in_f // 2)).astype(np.uint8)
         pr = rng.integers(0, 256, size=(o, in_f // 2)).astype(np.uint8)
         norms = (rng.random(o) + 0.5).astype(np.float32)
-        qw = oracle.QuantizedWeight(pp, pr, norms, np.array([rng.integers(1, 2 ** 32), 0, bs], np.uint32))
+        qw = oracle.QuantizedWeight(pp, pr, norms, np.array([rng.integers(1, 2 ** 32), rng.integers(1, 2 ** 32) if dual else 0, bs], np.uint32))
         qws.append(qw)
         layers.append(tq.TurboQuantLinear(in_f, o, qw, cb, cb, bs))
     xbits = oracle.f32_to_bf16_bits(np.random.default_rng(batch).standard_normal((batch, in_f)).astype(np.float32))

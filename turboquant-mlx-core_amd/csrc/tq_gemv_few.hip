@@ -48,6 +48,7 @@ struct FewArgs {
     int iters;           // uniform trip count: the longest range of a stream, in quads
     int quads_q, quads_rem;
     int ntiles, nt_inv;  // 512-column tiles of a row; (i * nt_inv) >> 16 == i / ntiles for the job numbers in use
+    int planes, segs;    // nibble planes: planes of the layer (1 or 2) and 512-column segments of a plane
 };
 
 typedef _Float16 few_h4 __attribute__((ext_vector_type(4)));
@@ -322,6 +323,194 @@ __global__ __launch_bounds__(1024) void tq_gemv_few_kernel(FewArgs a) {
     few_body<SETS, U, TL, PRE>(a, (int)blockIdx.x);
 }
 
+// Nibble planes (dual rotation: two planes, each with its own rotation and 16-entry table; primary only: one).  The
+// same scheme on a plane of two weights per byte: a segment is 256 bytes of a row, 512 columns; a lane's 16 bytes are
+// 32 columns; the table is indexed by a whole byte and an entry holds the fp16 centroids of both its nibbles (low
+// nibble = even column), i.e. half an A operand, so four weights cost two table reads and no pack.  Both planes'
+// tables share the 64 KB one took: an entry holds 32 lane columns of the primary plane's value, then 32 of the
+// residual plane's, and lanes l and l + 32 share a column (the LDS serves a wave's 32-bit reads in two halves of 32
+// lanes, so they never meet).  The units of a row are its primary segments, then its residual segments; wave w of a
+// quad stream owns units U w .. U w + U - 1 and multiplies each with the activations of that plane's rotation, and
+// the cross-wave sum adds the planes.  The rows always come rotated ([plane][batch][in] fp16): every CU rotating
+// every row twice costs more than the rotation kernel.
+template <int SETS, int U>
+__device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int block) {
+    __shared__ __align__(16) char smem[kLut256Bytes + kFewPartialBytes];
+    float* const partial = reinterpret_cast<float*>(smem + kLut256Bytes);     // [2][waves][SETS][16]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int stream = (wave * a.w_inv) >> 8;
+    const int unit = wave - stream * a.W;
+    const int out = a.L.out_features, K = a.L.in_features;
+    const int pitch = K >> 1;                     // bytes of a row of a plane
+    const int blk = lane >> 2, q = lane & 3;
+    const int units = a.planes * a.segs;
+
+    int col[U], plane[U];
+    bool act[U];
+    uint32_t laneoff[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int g = unit * U + u;
+        plane[u] = g >= a.segs ? 1 : 0;           // wave-uniform
+        col[u] = (g - plane[u] * a.segs) * 512 + 32 * blk;
+        act[u] = g < units && col[u] < K;
+        laneoff[u] = ((uint32_t)(lane & 31) << 2) | ((uint32_t)plane[u] << 7);
+    }
+
+    const int gs = block * a.S + stream;
+    const int q_begin = gs * a.quads_q + (gs < a.quads_rem ? gs : a.quads_rem);
+    const int q_end = q_begin + a.quads_q + (gs < a.quads_rem ? 1 : 0);
+    const int r_begin = 4 * q_begin;
+    const int r_end = 4 * q_end < out ? 4 * q_end : out;
+    const int r_base = r_begin < out ? r_begin : out - 1;
+
+    constexpr uint32_t kNoFetch = 0x80000000u;
+    uint32_t off[U];
+    __amdgpu_buffer_rsrc_t rs[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        off[u] = act[u] ? (uint32_t)q * (uint32_t)pitch + (uint32_t)(col[u] >> 1) : kNoFetch;
+        const uint8_t* const base = (plane[u] && a.planes == 2) ? a.L.packed_residual : a.L.packed_primary;
+        rs[u] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(base) + (size_t)r_base * (size_t)pitch, 0, 0x7fffffff, 0x00020000);
+    }
+    uint4 P[U];
+    auto fetch = [&](auto Uc, int r0) {
+        constexpr int u = decltype(Uc)::value;
+        P[u] = few_load16(rs[u], r0 + q < r_end ? off[u] : kNoFetch, (r0 - r_base) * pitch);
+    };
+    auto norm_of = [&](int r0) {
+        const int rn = r0 + ((lane >> 2) & 3);
+        return a.L.norms[rn < out ? rn : out - 1];
+    };
+
+    // The lane's columns of the rotated rows of its units' planes, then the norms and the first weights.
+    uint32_t xh[SETS][U][16];                 // fp16 pairs of activation row q + 4 e: columns 2 j, 2 j + 1 of unit u
+    {
+        const char* xr = static_cast<const char*>(a.x);
+#pragma unroll
+        for (int e = 0; e < SETS; ++e)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool on = act[u] && q + 4 * e < a.batch;
+                const size_t row = on ? (size_t)plane[u] * a.batch + q + 4 * e : 0;
+                const uint4* p = reinterpret_cast<const uint4*>(xr + (row * K + (on ? col[u] : 0)) * 2);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint4 t = p[k];
+                    xh[e][u][4 * k] = t.x; xh[e][u][4 * k + 1] = t.y; xh[e][u][4 * k + 2] = t.z; xh[e][u][4 * k + 3] = t.w;
+                }
+            }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    float nrm = norm_of(r_begin);
+    fetch(std::integral_constant<int, 0>{}, r_begin);
+    if constexpr (U > 1) fetch(std::integral_constant<int, 1>{}, r_begin);
+    if constexpr (U > 2) fetch(std::integral_constant<int, 2>{}, r_begin);
+    if constexpr (U > 3) fetch(std::integral_constant<int, 3>{}, r_begin);
+
+    // Byte-pair tables of both planes -> LDS.  (Both planes' entries are made from scalar loads and chosen per lane
+    // afterwards: a choice between the two addresses instead becomes a vector load, which queues behind the
+    // weight requests above.)
+    {
+        typedef const __attribute__((address_space(4))) float cfloat;
+        cfloat* const tab = (cfloat*)a.L.tables;
+        uint32_t* const dst = reinterpret_cast<uint32_t*>(smem) + lane;
+        const bool second = lane >= 32;
+        auto pair_entry = [&](int base, int c, int e) {
+            const uint32_t h = (uint32_t)float_to_f16_bits(tab[base + c]);
+            const uint32_t l = (uint32_t)float_to_f16_bits(tab[base + e]);
+            return (uint32_t)__builtin_amdgcn_readfirstlane((int)((h << 16) | l));
+        };
+        for (int c = wave; c < 16; c += nwaves) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t u0 = pair_entry(0, c, e), u1 = pair_entry(16, c, e);
+                dst[(c * 16 + e) * kWave] = second ? u1 : u0;
+            }
+        }
+    }
+    __syncthreads();                                           // tables visible to every wave
+#pragma unroll
+    for (int e = 0; e < SETS; ++e)
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) xh[e][u][j] = (act[u] && q + 4 * e < a.batch) ? xh[e][u][j] : 0u;   // idle lanes contribute 0
+
+    for (int it = 0; it < a.iters; ++it) {
+        const int r0 = r_begin + 4 * it;
+        const float nrm_next = norm_of(r0 + 4);
+        few_f4 acc[SETS];
+#pragma unroll
+        for (int e = 0; e < SETS; ++e) acc[e] = few_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        auto segment = [&](auto Uc) {
+            constexpr int u = decltype(Uc)::value;
+            const uint4 p = P[u];
+            fetch(Uc, r0 + 4);
+            const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {                      // dword d: columns 8 d .. 8 d + 7 of the lane's 32
+                const few_u2 w0 = {*reinterpret_cast<const uint32_t*>(smem + entry_addr<0>(pw[d], laneoff[u])),
+                                   *reinterpret_cast<const uint32_t*>(smem + entry_addr<1>(pw[d], laneoff[u]))};
+                const few_u2 w1 = {*reinterpret_cast<const uint32_t*>(smem + entry_addr<2>(pw[d], laneoff[u])),
+                                   *reinterpret_cast<const uint32_t*>(smem + entry_addr<3>(pw[d], laneoff[u]))};
+#pragma unroll
+                for (int e = 0; e < SETS; ++e) {
+                    const few_u2 x0 = {xh[e][u][4 * d], xh[e][u][4 * d + 1]}, x1 = {xh[e][u][4 * d + 2], xh[e][u][4 * d + 3]};
+                    acc[e] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(few_h4, w0), __builtin_bit_cast(few_h4, x0), acc[e], 0, 0, 0);
+                    acc[e] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(few_h4, w1), __builtin_bit_cast(few_h4, x1), acc[e], 0, 0, 0);
+                }
+            }
+        };
+        segment(std::integral_constant<int, 0>{});
+        if constexpr (U > 1) segment(std::integral_constant<int, 1>{});
+        if constexpr (U > 2) segment(std::integral_constant<int, 2>{});
+        if constexpr (U > 3) segment(std::integral_constant<int, 3>{});
+
+        float total[SETS];
+#pragma unroll
+        for (int e = 0; e < SETS; ++e) {
+            float v[4] = {acc[e][0], acc[e][1], acc[e][2], acc[e][3]};
+            total[e] = reduce_rec<4, 4>(v, lane);
+        }
+        const int r = r0 + ((lane >> 2) & 3);
+        const bool owner = lane < 16 && r < r_end;
+        bool store = owner;
+        if (a.W > 1) {
+            float* const buf_base = partial + (it & 1) * (16 * 32);
+            if (lane < 16) {
+#pragma unroll
+                for (int e = 0; e < SETS; ++e) buf_base[wave * 32 + 16 * e + lane] = total[e];
+            }
+            __syncthreads();
+            store = owner && unit == 0;
+            if (store) {
+#pragma unroll
+                for (int e = 0; e < SETS; ++e) {
+                    float t = 0.0f;
+                    for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * 32 + 16 * e + lane];
+                    total[e] = t;
+                }
+            }
+        }
+        if (store) {
+#pragma unroll
+            for (int e = 0; e < SETS; ++e)
+                if (q + 4 * e < a.batch) store_scalar(a.y, a.y_dtype, (size_t)(q + 4 * e) * out + r, total[e] * (a.L.inv_scale * nrm));
+        }
+        nrm = nrm_next;
+    }
+}
+
+template <int SETS, int U>
+__global__ __launch_bounds__(1024) void tq_gemv_few_nibble_kernel(FewArgs a) {
+    few_nibble_body<SETS, U>(a, (int)blockIdx.x);
+}
+
 // Two or three layers of equal width on the same activation rows (q, k, v or gate, up), one launch: the
 // workgroups are shared out over the layers by rows.
 struct FewGroup {
@@ -334,15 +523,22 @@ __global__ __launch_bounds__(1024) void tq_gemv_few_group_kernel(FewGroup g) {
     const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
     few_body<SETS, U, TL, PRE>(g.a[j], b - g.first[j]);
 }
+template <int SETS, int U>
+__global__ __launch_bounds__(1024) void tq_gemv_few_nibble_group_kernel(FewGroup g) {
+    const int b = (int)blockIdx.x;
+    const int j = b >= g.first[2] ? 2 : (b >= g.first[1] ? 1 : 0);
+    few_nibble_body<SETS, U>(g.a[j], b - g.first[j]);
+}
 
 // Rotated, scaled activation rows as fp16 [batch, in] for the calls whose workgroups do not rotate them themselves:
-// one wave per 512-column tile, row and layer (the layers of a group have rotations of their own).
+// one wave per 512-column tile, row and rotation (the layers of a group have rotations of their own, a dual-rotation
+// layer two).
 struct FewRotate {
     const void* x;
     int x_dtype, K;
-    uint32_t seed[3], bs[3];
-    float scale[3];
-    uint16_t* out[3];
+    uint32_t seed[6], bs[6];
+    float scale[6];
+    uint16_t* out[6];
 };
 __global__ __launch_bounds__(64) void tq_rotate_rows_f16_kernel(FewRotate r) {
     const int lane = threadIdx.x, t = blockIdx.y, j = blockIdx.z;
@@ -353,34 +549,41 @@ __global__ __launch_bounds__(64) void tq_rotate_rows_f16_kernel(FewRotate r) {
     if (c < r.K) *reinterpret_cast<uint4*>(r.out[j] + (size_t)t * r.K + c) = few_pack8(v, r.scale[j]);
 }
 
-// The shape of a launch: sets of four activation rows, segments per wave, waves per row quad, quad streams,
-// rotation jobs per wave, whether the rows come rotated.  Among the splits of the row's segments over 1 to 16 waves
-// with at most 8 segments each (4 with two sets: the registers), the one that keeps most lanes busy (segments that
-// exist, waves that exist; on a tie the one nearest four segments per wave: streams short enough for layers of a
-// few thousand rows, long enough between two barriers).  A function of the width and the batch alone: the order in
-// which a row's products are added depends on it, and a layer must give the same bits in a launch of its own and
-// in one it shares.
+bool few_nibble(const LayerView& L) { return L.mode == kDual || L.mode == kPrimaryOnly; }
+int few_planes(const LayerView& L) { return L.mode == kDual ? 2 : 1; }
+
+// The shape of a launch: sets of four activation rows, units per wave, waves per row quad, quad streams, rotation
+// jobs per wave, whether the rows come rotated.  A unit is a 256-byte segment of a row of a plane (256 columns of the
+// byte plane, 512 of a nibble plane; a dual-rotation row has its primary segments, then its residual ones).  Among
+// the splits of the row's units over 1 to 16 waves with no more units each than the registers hold (byte plane: 8,
+// with two sets 4; nibble planes, twice the activations per unit: 4 and 2), the one that keeps most lanes busy (units
+// that exist, waves that exist; on a tie the one nearest four units per wave: streams short enough for layers of a
+// few thousand rows, long enough between two barriers).  A function of the layer's width and mode and the batch
+// alone: the order in which a row's products are added depends on it, and a layer must give the same bits in a launch
+// of its own and in one it shares.  W == 0: no such split.
 struct FewShape { int sets, U, W, S, threads, tl; bool pre; };
-FewShape few_shape(int K, int batch) {
+FewShape few_shape(const LayerView& L, int batch) {
     FewShape s{};
+    const int K = L.in_features;
+    const bool nib = few_nibble(L);
     s.sets = batch > 4 ? 2 : 1;
-    const int max_u = s.sets == 2 ? 4 : kFewMaxU;
-    const int segs = (K + kSegCols - 1) / kSegCols;
+    const int max_u = nib ? (s.sets == 2 ? 2 : 4) : (s.sets == 2 ? 4 : kFewMaxU);
+    const int units = nib ? few_planes(L) * ((K + 511) / 512) : (K + kSegCols - 1) / kSegCols;
     double best = -1.0;
     for (int W = 1; W <= 16; ++W) {
-        int U = (segs + W - 1) / W;
+        int U = (units + W - 1) / W;
         if (U > max_u) continue;
         if (U < 2) U = 2;
         const int S = 16 / W;
-        const double eff = (double)segs / (W * U) * (W * S) / 16.0;
+        const double eff = (double)units / (W * U) * (W * S) / 16.0;
         const bool tie = eff > best - 1e-9 && (U - 4) * (U - 4) < (s.U - 4) * (s.U - 4);
         if (eff > best + 1e-9 || tie) { best = eff; s.U = U; s.W = W; s.S = S; }
     }
-    if (best < 0.0) return s;                                // (wider than 16 waves of max_u segments: W == 0)
+    if (best < 0.0) return s;
     s.threads = s.W * s.S * kWave;
     const int ntiles = (K + kTile - 1) / kTile, waves = s.W * s.S;
     const int per_wave = (batch * ntiles + waves - 1) / waves;
-    s.pre = s.sets == 2 || (size_t)batch * K * 2 > (size_t)kFewImageBytes || per_wave > 6;
+    s.pre = nib || s.sets == 2 || (size_t)batch * K * 2 > (size_t)kFewImageBytes || per_wave > 6;
     s.tl = per_wave <= 3 ? 3 : 6;
     return s;
 }
@@ -395,16 +598,31 @@ void few_ranges(FewArgs& a, const FewShape& s, int grid, int batch) {
     a.iters = a.quads_q + (a.quads_rem ? 1 : 0);
     a.ntiles = (a.L.in_features + kTile - 1) / kTile;
     a.nt_inv = 65536 / a.ntiles + 1;       // exact quotients for job numbers below 16 x 6 (at most 64 tiles per row)
+    a.planes = few_planes(a.L);
+    a.segs = (a.L.in_features + 511) / 512;
 }
 
-// GROUP: FewGroup and the kernel that serves several layers; otherwise FewArgs.
-template <int U, bool GROUP, typename Args>
+// GROUP: FewGroup and the kernels that serve several layers; otherwise FewArgs.  NIB: nibble planes.
+template <int U, bool GROUP, bool NIB, typename Args>
 hipError_t launch_few_u(const Args& a, const FewShape& s, int grid, hipStream_t stream) {
     const dim3 g(grid), b(s.threads);
-    if constexpr (GROUP) {
+    if constexpr (NIB) {
+        if constexpr (U > 4) return hipErrorInvalidValue;      // few_shape() rules this out
+        else if constexpr (GROUP) {
+            if (s.sets == 2) {
+                if constexpr (U <= 2) hipLaunchKernelGGL((tq_gemv_few_nibble_group_kernel<2, U>), g, b, 0, stream, a);
+                else return hipErrorInvalidValue;
+            } else hipLaunchKernelGGL((tq_gemv_few_nibble_group_kernel<1, U>), g, b, 0, stream, a);
+        } else {
+            if (s.sets == 2) {
+                if constexpr (U <= 2) hipLaunchKernelGGL((tq_gemv_few_nibble_kernel<2, U>), g, b, 0, stream, a);
+                else return hipErrorInvalidValue;
+            } else hipLaunchKernelGGL((tq_gemv_few_nibble_kernel<1, U>), g, b, 0, stream, a);
+        }
+    } else if constexpr (GROUP) {
         if (s.sets == 2) {
             if constexpr (U <= 4) hipLaunchKernelGGL((tq_gemv_few_group_kernel<2, U, 1, true>), g, b, 0, stream, a);
-            else return hipErrorInvalidValue;                  // few_shape() rules this out
+            else return hipErrorInvalidValue;
         }
         else if (s.pre) hipLaunchKernelGGL((tq_gemv_few_group_kernel<1, U, 1, true>), g, b, 0, stream, a);
         else if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_group_kernel<1, U, 3, false>), g, b, 0, stream, a);
@@ -421,13 +639,17 @@ hipError_t launch_few_u(const Args& a, const FewShape& s, int grid, hipStream_t 
     return hipGetLastError();
 }
 
-// What the kernel asks of a layer whatever the launch: shared rotation, centroid sums that fit fp16, blocks of at
-// most 512 columns (a block never leaves the tile a wave rotates), rows of at most 64 tiles.
+// What the kernels ask of a layer whatever the launch: shared rotation (the byte plane) or nibble planes, centroids
+// that fit fp16, blocks of at most 512 columns (a block never leaves the tile a wave rotates), rows of at most 64
+// tiles that some split covers.
 bool few_layer_ok(const LayerView& L, int batch) {
     if (batch < 2 || batch > kFewMaxBatch) return false;
-    if (L.mode != kSharedLut || !L.packed_combined || !L.fp16_centroids_ok) return false;
+    if (!L.fp16_centroids_ok) return false;
+    if (L.mode == kSharedLut) { if (!L.packed_combined) return false; }
+    else if (few_nibble(L)) { if (!L.packed_primary || (L.mode == kDual && !L.packed_residual)) return false; }
+    else return false;
     if (!lanes_supported(L.in_features, L.block_size) || L.block_size > (uint32_t)kTile) return false;
-    return L.in_features <= 16 * kFewMaxU * kSegCols && few_shape(L.in_features, batch).W > 0;
+    return L.in_features <= 16 * kFewMaxU * kSegCols && few_shape(L, batch).W > 0;
 }
 // A stream's share of the plane stays below the 2 GB of its buffer descriptor (one stream per CU at least).
 bool few_share_ok(const LayerView& L, int num_cus) {
@@ -435,19 +657,25 @@ bool few_share_ok(const LayerView& L, int num_cus) {
     const long long max_rows = (L.out_features + cus - 1) / cus + 24;
     return (unsigned long long)max_rows * (unsigned long long)L.in_features < (1ull << 31);
 }
-// Where the rotated rows of a call go when its workgroups do not rotate them: the layer's scratch row (rows wider
-// than 16384 columns have one: 2 x in floats = 4 rows of fp16) or a workspace of the caller.
-bool few_uses_scratch_row(const LayerView& L, int batch) { return batch <= 4 && L.xrot_work != nullptr; }
+// Where the rotated rows of a call go when its workgroups do not rotate them: the layer's scratch row (shared-
+// rotation rows wider than 16384 columns have one: 2 x in floats = 4 rows of fp16) or a workspace of the caller.
+bool few_uses_scratch_row(const LayerView& L, int batch) { return !few_nibble(L) && batch <= 4 && L.xrot_work != nullptr; }
 // Every workgroup rotates all the activation rows for itself: about 0.15 us per 512-column tile and row, whatever
 // the size of the plane, where the small-batch kernel pays 4 us for its second kernel and loses about 0.06 us per MB
 // of plane to its load pattern (same-box comparisons of the two on eleven shapes, weight copies cycled).  Few rows
 // of a wide plane go to the small-batch kernel.  (Up to 40 tiles whatever the plane: the layers of a group, large
 // and small, should agree on the kernel, or the group is run layer by layer.)  Rows that come rotated cost a kernel
-// of their own, which only a plane of some size repays.
-bool few_worth_it(const FewShape& s, int batch, int K, long long plane_bytes) {
+// of their own (4.6 to 4.8 us), which only a plane of some size repays.
+bool few_worth_it(const LayerView& L, const FewShape& s, int batch) {
+    const int K = L.in_features;
+    const long long plane_bytes = (long long)L.out_features * K * (few_nibble(L) ? few_planes(L) : 2) / 2;
     // (five to eight rows, same-box comparisons with the small-batch kernel: 27648 x 5120 35.1 against 42.2 us,
     // 28672 x 8192 47.7 / 59.7, but 14336 x 4096 23.7 / 20.7, 8192 x 8192 23.8 / 21.8, 5120 x 5120 17.1 / 14.3)
-    if (s.pre) return plane_bytes >= (s.sets == 2 ? (96ll << 20) : (64ll << 20));
+    // (nibble planes, two to four rows: 27648 x 5120 34.6 against 40.2 us, 28672 x 8192 47.9 / 62.0, but 8192 x 8192
+    // 23.9 / 21.7; five to eight: 28672 x 8192 59.8 / 68.1, but 27648 x 5120, whose 20 units make two per wave of 10
+    // waves, 56.2 / 44.4: two sets want a workgroup of 14 waves and more)
+    if (s.sets == 2 && s.W * s.S < 14) return false;
+    if (s.pre) return plane_bytes >= ((s.sets == 2 || few_nibble(L)) ? (96ll << 20) : (64ll << 20));
     const long long jobs = (long long)batch * ((K + kTile - 1) / kTile);
     return jobs <= 40 || jobs * 5 <= 135 + plane_bytes / 500000;           // jobs <= 27 + 0.4 per MB
 }
@@ -466,21 +694,30 @@ hipError_t few_dispatch_u(int U, F&& f) {
     }
 }
 
-// The rotation kernel of a call whose rows come rotated: layer j's rows go to its scratch row or to the j-th part
-// of the workspace; as[j].x is set to them.
+size_t few_rotated_bytes(const LayerView& L, int batch) {
+    return ((size_t)few_planes(L) * batch * L.in_features * 2 + 255) & ~(size_t)255;
+}
+
+// The rotation kernel of a call whose rows come rotated: layer j's rows ([plane][batch][in]) go to its scratch row
+// or to the j-th part of the workspace; as[j].x is set to them.
 hipError_t few_rotate_rows(FewArgs* as, int n, const void* x, int x_dtype, int batch, void* workspace, hipStream_t stream) {
     FewRotate r{};
     r.x = x; r.x_dtype = x_dtype; r.K = as[0].L.in_features;
-    const size_t part = ((size_t)batch * r.K * 2 + 255) & ~(size_t)255;
+    const size_t part = few_rotated_bytes(as[0].L, batch);
+    const int planes = few_planes(as[0].L);
     for (int j = 0; j < n; ++j) {
         const LayerView& L = as[j].L;
-        r.seed[j] = L.seed_primary; r.bs[j] = L.block_size; r.scale[j] = L.inv_sqrt_bs;
-        r.out[j] = few_uses_scratch_row(L, batch) ? reinterpret_cast<uint16_t*>(L.xrot_work)
-                 : workspace ? reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + j * part) : nullptr;
-        if (!r.out[j]) return hipErrorInvalidValue;
-        as[j].x = r.out[j];
+        uint16_t* const base = few_uses_scratch_row(L, batch) ? reinterpret_cast<uint16_t*>(L.xrot_work)
+                             : workspace ? reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + j * part) : nullptr;
+        if (!base) return hipErrorInvalidValue;
+        for (int p = 0; p < planes; ++p) {
+            r.seed[j * planes + p] = p ? L.seed_residual : L.seed_primary;
+            r.bs[j * planes + p] = L.block_size; r.scale[j * planes + p] = L.inv_sqrt_bs;
+            r.out[j * planes + p] = base + (size_t)p * batch * r.K;
+        }
+        as[j].x = base;
     }
-    hipLaunchKernelGGL(tq_rotate_rows_f16_kernel, dim3((r.K + kTile - 1) / kTile, batch, n), dim3(64), 0, stream, r);
+    hipLaunchKernelGGL(tq_rotate_rows_f16_kernel, dim3((r.K + kTile - 1) / kTile, batch, n * planes), dim3(64), 0, stream, r);
     return hipGetLastError();
 }
 
@@ -489,48 +726,50 @@ hipError_t few_rotate_rows(FewArgs* as, int n, const void* x, int x_dtype, int b
 // Two to eight rows of any activation type.
 bool gemv_few_supported(const LayerView& L, int batch, int num_cus) {
     if (!few_layer_ok(L, batch) || !few_share_ok(L, num_cus)) return false;
-    return few_worth_it(few_shape(L.in_features, batch), batch, L.in_features, (long long)L.out_features * L.in_features);
+    return few_worth_it(L, few_shape(L, batch), batch);
 }
 
 // Bytes of workspace a call needs for its rotated rows (0: none).
 size_t gemv_few_workspace_bytes(const LayerView& L, int batch) {
-    if (!few_layer_ok(L, batch) || !few_shape(L.in_features, batch).pre || few_uses_scratch_row(L, batch)) return 0;
-    return ((size_t)batch * L.in_features * 2 + 255) & ~(size_t)255;
+    if (!few_layer_ok(L, batch) || !few_shape(L, batch).pre || few_uses_scratch_row(L, batch)) return 0;
+    return few_rotated_bytes(L, batch);
 }
 
 hipError_t launch_gemv_few(const LayerView& L, const void* x, int x_dtype, int batch, void* y, int y_dtype,
                            void* workspace, int num_cus, hipStream_t stream) {
-    const FewShape s = few_shape(L.in_features, batch);
+    const FewShape s = few_shape(L, batch);
     FewArgs a{};
     a.L = L; a.x = x; a.y = y; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
-    if (s.pre) {
-        const hipError_t e = few_rotate_rows(&a, 1, x, x_dtype, batch, workspace, stream);
-        if (e != hipSuccess) return e;
-    }
     const int quads = (L.out_features + 3) / 4;
     int grid = (quads + s.S - 1) / s.S;
     if (grid > num_cus) grid = num_cus;
     if (grid < 1) grid = 1;
     few_ranges(a, s, grid, batch);
-    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, false>(a, s, grid, stream); });
+    if (s.pre) {
+        const hipError_t e = few_rotate_rows(&a, 1, x, x_dtype, batch, workspace, stream);
+        if (e != hipSuccess) return e;
+    }
+    if (few_nibble(L))
+        return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, false, true>(a, s, grid, stream); });
+    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, false, false>(a, s, grid, stream); });
 }
 
-// Layers that can share a launch: two or three of equal width, each taken by the kernel in a launch of its own.
+// Layers that can share a launch: two or three of equal width and mode, each taken by the kernel in a launch of its own.
 bool gemv_few_group_supported(const LayerView* Ls, int n, int batch, int num_cus) {
     if (n < 2 || n > 3 || num_cus < n) return false;
     for (int j = 0; j < n; ++j) {
-        if (Ls[j].in_features != Ls[0].in_features) return false;
+        if (Ls[j].in_features != Ls[0].in_features || Ls[j].mode != Ls[0].mode) return false;
         if (!gemv_few_supported(Ls[j], batch, 1)) return false;      // (1 CU: the strictest bound on a stream's share)
     }
     return true;
 }
 
-// workspace: n x gemv_few_workspace_bytes() of the first layer (every layer has a rotation of its own).
+// workspace: n x gemv_few_workspace_bytes() of the first layer (every layer has rotations of its own).
 hipError_t launch_gemv_few_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
                                  int y_dtype, void* workspace, int num_cus, hipStream_t stream) {
     long long total = 0;
     for (int j = 0; j < n; ++j) total += Ls[j].out_features;
-    const FewShape s = few_shape(Ls[0].in_features, batch);
+    const FewShape s = few_shape(Ls[0], batch);
     // Workgroups per layer in proportion to its rows.
     int blocks[3] = {0, 0, 0}, used = 0;
     for (int j = 0; j < n; ++j) {
@@ -553,7 +792,9 @@ hipError_t launch_gemv_few_group(const LayerView* Ls, int n, const void* x, int 
         const hipError_t e = few_rotate_rows(g.a, n, x, x_dtype, batch, workspace, stream);
         if (e != hipSuccess) return e;
     }
-    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, true>(g, s, used, stream); });
+    if (few_nibble(Ls[0]))
+        return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, true, true>(g, s, used, stream); });
+    return few_dispatch_u(s.U, [&](auto Uc) { return launch_few_u<decltype(Uc)::value, true, false>(g, s, used, stream); });
 }
 
 }  // namespace tq
