@@ -163,6 +163,51 @@ def test_reserved_layer_is_captured_and_replayed(tq, oracle, mode, out, inf, bs,
     hip.close()
 
 
+@pytest.mark.parametrize("dual,out,inf,bs,batches", [(False, 12300, 8192, 512, (3, 8)),     # rows rotated in the kernel; two sets of rows, rotated by a kernel of their own
+                                                     (False, 4700, 14336, 256, (4,)),        # images that do not fit LDS
+                                                     (True, 19701, 5120, 512, (2, 4))])      # nibble planes: two rotations
+def test_whole_row_kernel_with_rotated_rows_is_captured_and_replayed(tq, oracle, dual, out, inf, bs, batches):
+    """The kernel for two to eight rows where a kernel of its own rotates the rows into the layer's workspace: after
+    tq_linear_reserve both launches of a call are captured, and every replay gives the bits of the eager call (a
+    sample of whose rows is checked against the oracle)."""
+    o, hip = oracle, _Hip()
+    rng = np.random.default_rng(out)
+    cb = o.generate_codebook(4)
+    pp = rng.integers(0, 256, size=(out, inf // 2)).astype(np.uint8)
+    pr = rng.integers(0, 256, size=(out, inf // 2)).astype(np.uint8)
+    norms = (rng.random(out) + 0.5).astype(np.float32)
+    qw = o.QuantizedWeight(pp, pr, norms, np.array([rng.integers(1, 2 ** 32), rng.integers(1, 2 ** 32) if dual else 0, bs], np.uint32))
+    layer = tq.TurboQuantLinear(inf, out, qw, cb, cb, bs)
+    layer.reserve(max(batches))
+    xbits = {b: _bits(o, rng, b, inf) for b in batches}
+    xs = {b: hip.upload(xbits[b]) for b in batches}
+    eager = {b: hip.alloc(b * out * 4) for b in batches}
+    replayed = {b: hip.alloc(b * out * 4) for b in batches}
+    for b in batches:
+        layer.forward_device(xs[b], tq.BF16, b, eager[b], tq.F32, hip.stream)
+    want = {b: hip.download(eager[b], (b, out)) for b in batches}
+    rows = np.unique(np.concatenate([np.arange(5), np.arange(out - 5, out), np.arange(0, out, 173)]))
+    sub = o.QuantizedWeight(pp[rows], pr[rows], norms[rows], qw.seeds)
+    w_ref = o.dequantize_weight_cpu(sub, cb, cb, bs)
+    for b in batches:
+        assert _rel(want[b][:, rows], o.matmul_xwT(o.bf16_bits_to_f32(xbits[b]), w_ref, acc_double=True)) < 1e-3
+    hip.begin_capture()
+    for b in batches:
+        layer.forward_device(xs[b], tq.BF16, b, replayed[b], tq.F32, hip.stream)
+    graph = hip.end_capture()
+    for turn in range(3):
+        for b in batches:
+            hip.fill(replayed[b], b * out * 4)                 # eager work between the replays
+        other = batches[turn % len(batches)]
+        layer.forward_device(xs[other], tq.BF16, other, eager[other], tq.F32, None)
+        hip.replay(graph[1])
+        for b in batches:
+            assert np.array_equal(hip.download(replayed[b], (b, out)), want[b]), f"replay {turn}, batch {b}"
+    hip.drop(graph)
+    layer.close()
+    hip.close()
+
+
 def test_growth_is_refused_while_capturing_and_capture_survives(tq, oracle):
     o, hip = oracle, _Hip()
     out, inf, bs = 320, 1024, 512
