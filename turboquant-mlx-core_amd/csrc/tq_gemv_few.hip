@@ -67,10 +67,48 @@ __device__ __forceinline__ uint4 few_pack8(const float (&v)[8], float s) {
     o.w = (uint32_t)float_to_f16_bits(v[6] * s) | ((uint32_t)float_to_f16_bits(v[7] * s) << 16);
     return o;
 }
+// The same for values that carry their scale already: four packed conversions (round to nearest even, as above).
+__device__ __forceinline__ uint4 few_pack8(const float (&v)[8]) {
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    uint4 o;
+    o.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[0], v[1]}, h2));
+    o.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[2], v[3]}, h2));
+    o.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[4], v[5]}, h2));
+    o.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[6], v[7]}, h2));
+    return o;
+}
+
+// One butterfly stage across lanes l and l ^ 16 (or 32) for two values at once: v_permlane16_swap / _permlane32_swap
+// exchange rows (halves) between two registers, so a swap, a sum, a difference and a second swap serve both values,
+// four instructions where lane_xor + select + fma take six.  Lower lane a + b, upper lane a - b with a the lower
+// lane's value: the bits of butterfly_lanes.
+template <int MASK>
+__device__ __forceinline__ void few_butterfly_pair(float& a, float& b) {
+    static_assert(MASK == 16 || MASK == 32, "row and half swaps");
+    const unsigned ua = __builtin_bit_cast(unsigned, a), ub = __builtin_bit_cast(unsigned, b);
+    float lo, hi;
+    if constexpr (MASK == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(ua, ub, false, false);
+        lo = __builtin_bit_cast(float, (unsigned)r[0]); hi = __builtin_bit_cast(float, (unsigned)r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap(ua, ub, false, false);
+        lo = __builtin_bit_cast(float, (unsigned)r[0]); hi = __builtin_bit_cast(float, (unsigned)r[1]);
+    }
+    const float sum = lo + hi, dif = lo - hi;
+    const unsigned us = __builtin_bit_cast(unsigned, sum), ud = __builtin_bit_cast(unsigned, dif);
+    if constexpr (MASK == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(us, ud, false, false);
+        a = __builtin_bit_cast(float, (unsigned)r[0]); b = __builtin_bit_cast(float, (unsigned)r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap(us, ud, false, false);
+        a = __builtin_bit_cast(float, (unsigned)r[0]); b = __builtin_bit_cast(float, (unsigned)r[1]);
+    }
+}
 
 // rotate_tile() with the signs handed in: blocks are at most one tile wide and tiles start at multiples of 512, so
 // the sign of a column depends on its position inside the tile alone, and a wave computes its eight once for all
-// the tiles it rotates (the hash is a quarter of the instructions of a rotation).
+// the tiles it rotates (the hash is a quarter of the instructions of a rotation).  The signs may carry a scale.
 __device__ __forceinline__ void few_rotate(const TileRaw& raw, int x_dtype, bool active, const float (&sg)[8],
                                            uint32_t bs, int lane, float (&v)[8]) {
     if (active) {
@@ -97,7 +135,33 @@ __device__ __forceinline__ void few_rotate(const TileRaw& raw, int x_dtype, bool
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = 0.0f;
     }
-    fwht_lanes<8>(v, bs, lane);
+    // fwht_lanes<8> with the stages across 16 and 32 lanes done two values at a time.
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1) {
+        if ((uint32_t)h < bs) {
+#pragma unroll
+            for (int i = 0; i < 8; i += 2 * h) {
+#pragma unroll
+                for (int k = i; k < i + h; ++k) {
+                    const float p = v[k], q = v[k + h];
+                    v[k] = p + q;
+                    v[k + h] = p - q;
+                }
+            }
+        }
+    }
+    if (8u < bs) butterfly_lanes<1, 8>(v, lane);
+    if (16u < bs) butterfly_lanes<2, 8>(v, lane);
+    if (32u < bs) butterfly_lanes<4, 8>(v, lane);
+    if (64u < bs) butterfly_lanes<8, 8>(v, lane);
+    if (128u < bs) {
+#pragma unroll
+        for (int k = 0; k < 8; k += 2) few_butterfly_pair<16>(v[k], v[k + 1]);
+    }
+    if (256u < bs) {
+#pragma unroll
+        for (int k = 0; k < 8; k += 2) few_butterfly_pair<32>(v[k], v[k + 1]);
+    }
 }
 
 // SETS sets of four activation rows, U segments per wave (wave w of a quad stream owns segments U w .. U w + U - 1 of
@@ -212,7 +276,8 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
         char* const image = smem + kLut256Bytes + kFewPartialBytes;               // [batch][K] fp16
         float sg[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) sg[j] = sign_of(a.L.seed_primary, (uint32_t)(lane * 8 + j) & (a.L.block_size - 1));
+        for (int j = 0; j < 8; ++j)        // (with the scale 1 / sqrt(bs): the rotation is linear)
+            sg[j] = sign_of(a.L.seed_primary, (uint32_t)(lane * 8 + j) & (a.L.block_size - 1)) * a.L.inv_sqrt_bs;
 #pragma unroll
         for (int k = 0; k < TL; ++k) {
             const int job = wave + k * nwaves;
@@ -221,7 +286,7 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
                 const int c = (job - tok * a.ntiles) * kTile + lane * 8;
                 float v[8];
                 few_rotate(raw[k], a.x_dtype, c < K, sg, a.L.block_size, lane, v);
-                if (c < K) *reinterpret_cast<uint4*>(image + ((size_t)tok * K + c) * 2) = few_pack8(v, a.L.inv_sqrt_bs);
+                if (c < K) *reinterpret_cast<uint4*>(image + ((size_t)tok * K + c) * 2) = few_pack8(v);
             }
         }
         __syncthreads();                                       // images and table visible to every wave
