@@ -470,7 +470,7 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     # the workgroups rotate the activation rows themselves: 2..7 segments of 256 columns per wave, one wave per row
     # quad (no cross-wave sum) or several
     (64, 256, 64, 2), (70, 1536, 512, 3), (64, 768, 256, 4), (66, 2048, 512, 2), (61, 1024, 64, 3),
-    (64, 2560, 512, 4), (63, 1280, 256, 2), (65, 4352, 256, 3), (64, 3328, 256, 4), (67, 1792, 256, 2),
+    (64, 2560, 512, 4), (63, 1280, 256, 2), (65, 4352, 256, 3), (64, 3328, 256, 4), (67, 1792, 256, 2), (64, 4608, 512, 2),
     # fewer rows than a quad, ragged quads, widths that are not a multiple of a segment, many streams per workgroup
     (3, 1024, 64, 4), (1281, 5120, 512, 3), (6913, 5120, 512, 4), (130, 2816, 256, 4), (77, 1344, 64, 2),
     (3000, 2848, 32, 3), (16500, 2304, 256, 4),
@@ -480,7 +480,8 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     # images that do not fit LDS (a workspace)
     (4096, 17408, 512, 3), (3500, 24576, 512, 4), (2600, 27648, 512, 4), (2600, 32768, 512, 2), (5000, 14336, 512, 4),
     # five to eight rows: two sets of four on the same decoded weights, planes of 96 MB and more
-    (19701, 5120, 512, 8), (12300, 8192, 256, 5), (6200, 16384, 512, 7), (66000, 1536, 512, 6), (49500, 2048, 128, 8)])
+    (19701, 5120, 512, 8), (12300, 8192, 256, 5), (6200, 16384, 512, 7), (66000, 1536, 512, 6), (49500, 2048, 128, 8),
+    (197000, 512, 64, 6)])
 def test_two_to_eight_rows_whole_row_kernel(tq, oracle, out, inf, bs, batch):
     _whole_row_kernel_case(tq, oracle, "shared", out, inf, bs, batch)
 
