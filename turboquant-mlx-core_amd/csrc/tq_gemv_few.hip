@@ -67,15 +67,14 @@ __device__ __forceinline__ uint4 few_pack8(const float (&v)[8], float s) {
     o.w = (uint32_t)float_to_f16_bits(v[6] * s) | ((uint32_t)float_to_f16_bits(v[7] * s) << 16);
     return o;
 }
-// The same for values that carry their scale already: four packed conversions (round to nearest even, as above).
+// The same for values that carry their scale already: four packed conversions (round to nearest even, saturating
+// like the above).
 __device__ __forceinline__ uint4 few_pack8(const float (&v)[8]) {
-    typedef float f2 __attribute__((ext_vector_type(2)));
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     uint4 o;
-    o.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[0], v[1]}, h2));
-    o.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[2], v[3]}, h2));
-    o.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[4], v[5]}, h2));
-    o.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){v[6], v[7]}, h2));
+    o.x = pack_f16_saturating(v[0], v[1]);
+    o.y = pack_f16_saturating(v[2], v[3]);
+    o.z = pack_f16_saturating(v[4], v[5]);
+    o.w = pack_f16_saturating(v[6], v[7]);
     return o;
 }
 
