@@ -554,7 +554,7 @@ def main():
     L.tq_linear_forward_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_int,
                                           C.POINTER(C.c_void_p), C.c_int, C.c_void_p]
     def grouped(sets, tag):
-        for batch in (1, 4, 8, 32):
+        for batch in (1, 2, 4, 8, 32):
             xg = {i_: torch.randn(batch, i_, device="cuda", generator=g).to(torch.bfloat16) for i_ in (5120, 27648)}
             yg = {n_: torch.empty(batch, out_of[n_], device="cuda", dtype=torch.float32) for n_ in sets[0]}
             turn = [0]
