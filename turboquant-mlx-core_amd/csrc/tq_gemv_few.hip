@@ -1,15 +1,16 @@
-// Fused TQ8 dequant + matrix-vector products for gfx950, two to eight activation rows, shared-rotation layers
-// (one byte per weight), blocks of at most 512 columns.
+// Fused TQ8 dequant + matrix-vector products for gfx950, two to eight activation rows, blocks of at most 512
+// columns: shared-rotation layers (one byte per weight) and, further down, nibble planes (dual rotation, primary only).
 //
 // The batch-1 kernel (tq_gemv_wide.hip) reads the plane in whole rows and runs at the rate of its table reads.  The
 // small-batch kernel (tq_skinny.hip) puts the activation rows on v_mfma_f32_16x16x32_f16, whose operand layout
 // wants 16 weight rows per load instruction, 64 bytes of each; it cuts K over the workgroups and adds the parts in a
 // second kernel.  Four activation rows fit v_mfma_f32_4x4x4_16b_f16 instead (five to eight: two such sets on the
-// same decoded weights): 16 independent 4 x 4 x 4 blocks per instruction, block = lane / 4.  The four lanes of a block hold the same 16 columns of four consecutive weight
-// rows (A operand: four decoded weights per step) and of the four activation rows (B operand), so
-//   * a load instruction of a wave fetches 256 contiguous bytes of each of four rows (whole cache lines), a wave
-//     covers U such segments of its four rows, and the waves of a row stream cover the whole row: no cut along K,
-//     the cross-wave sum stays inside the workgroup and there is no second kernel;
+// same decoded weights): 16 independent 4 x 4 x 4 blocks per instruction, block = lane / 4.  The four lanes of a
+// block hold the same 16 columns of four consecutive weight rows (A operand: four decoded weights per step) and of
+// the four activation rows (B operand), so
+//   * a load instruction of a wave fetches 256 contiguous bytes of each of four rows (whole cache lines, streaming
+//     hint), a wave covers U such segments of its four rows, and the waves of a row stream cover the whole row: no
+//     cut along K, the cross-wave sum stays inside the workgroup and there is no second kernel;
 //   * a decoded weight costs one address permute, one table read and half a pack (as in the small-batch kernel)
 //     whatever the number of activation rows; the products are four matrix instructions per 16 bytes of a lane;
 //   * the kernel keeps the batch-1 kernel's shape: one workgroup of up to 16 waves per CU, lane-private table
@@ -17,8 +18,9 @@
 //     they are rounded, as in the small-batch and prefill kernels), every load slot requested again as soon as it
 //     has been decoded.
 // The activation rows are rotated once per CU (the waves share out the 512-column tiles of all rows and hand the
-// result over through fp16 images in LDS), or, where the images do not fit or there are more than four rows (every
-// CU rotating every row costs 0.15 us per tile and row), by a small kernel of its own into a workspace.
+// result over through fp16 images in LDS), or, where the images do not fit, there are more than four rows (every
+// CU rotating every row costs 0.15 us per tile and row) or the layer has nibble planes, by a small kernel of its
+// own into the layer's scratch row or a workspace.
 // Sums are fp32.  The reference has no batched path (src/dequantizer.cpp:545-549: batch is a grid dimension of its
 // per-row kernel).
 #include "tq_device.h"
