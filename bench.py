@@ -211,6 +211,42 @@ def timeline(tq, torch):
         torch.cuda.empty_cache()
 
 
+def rows_table(tq, torch):
+    """us per tq_linear_forward call against the number of rows; one line per shape and rotation."""
+    L = tq.lib()
+    rows = (1, 2, 3, 4, 5, 8, 16, 32)
+    print("rows                          " + "".join(f"{r:>8d}" for r in rows))
+    for shared in (True, False):
+        for outp, inp in ((151936, 2048), (27648, 5120), (5120, 27648)):
+            copies = -(-600_000_000 // (outp * inp)) + 1
+            hs = [make_layer(tq, torch, outp, inp, 512, seed=700 + i, sigma=0.01, shared=shared,
+                             per_layer_codebooks=False, tails=False)[0] for i in range(copies)]
+            res = []
+            for m in rows:
+                x = torch.randn(m, inp, device="cuda").to(torch.bfloat16)
+                y = torch.empty(m, outp, device="cuda", dtype=torch.float32)
+
+                def run(n):
+                    for i in range(n):
+                        if L.tq_linear_forward(hs[i % copies], x.data_ptr(), tq.BF16, m, y.data_ptr(), tq.F32, None) != 0:
+                            raise RuntimeError(tq.last_error())
+                t_end = time.perf_counter() + 0.1          # the clocks settle over tens of milliseconds
+                while time.perf_counter() < t_end:
+                    run(copies)
+                    torch.cuda.synchronize()
+                st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                st.record()
+                run(8 * copies)
+                en.record()
+                torch.cuda.synchronize()
+                res.append(st.elapsed_time(en) * 1e3 / (8 * copies))
+            tag = f"{outp}x{inp} {'shared' if shared else 'dual'} ({copies} copies)"
+            print(f"{tag:30s}" + "".join(f"{v:8.1f}" for v in res), flush=True)
+            for h in hs:
+                L.tq_linear_free(h)
+            torch.cuda.empty_cache()
+
+
 def cpu_baseline(torch, tensors, out, inf, bs, x_f32):
     """Reference CPU path (dequantize_weight_cpu + fp32 matmul, restated in oracle/) on the
     host cores of this box, whole layer, single thread as the reference's serial loops."""
@@ -255,6 +291,11 @@ def main():
                          "(`make ablations`; MASK as in csrc/tq_prefill_panel.hip, 0 = the product library).  Meant to "
                          "run under rocprofv3 --pmc: the results are wrong by construction, the cycle counters of "
                          "the kernel are what is compared")
+    ap.add_argument("--rows-table", action="store_true",
+                    help="instead of the benchmark: time of one tq_linear_forward call against the number of activation "
+                         "rows (1..32) on the lm_head and the two large decoder projections, shared and dual rotation, "
+                         "bf16 in / fp32 out, eager launches timed with HIP events, weight copies cycled so that the "
+                         "planes come from HBM (more than 600 MB per shape)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy three times (reference reading for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -274,6 +315,9 @@ def main():
     torch.cuda.set_device(0)
     if args.timeline:
         timeline(tq, torch)
+        return
+    if args.rows_table:
+        rows_table(tq, torch)
         return
     if args.prefill_ablations is not None:
         mask = int(args.prefill_ablations)

@@ -443,10 +443,13 @@ __device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int bloc
         const uint8_t* const base = (plane[u] && a.planes == 2) ? a.L.packed_residual : a.L.packed_primary;
         rs[u] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(base) + (size_t)r_base * (size_t)pitch, 0, 0x7fffffff, 0x00020000);
     }
-    uint4 P[U];
-    auto fetch = [&](auto Uc, int r0) {
-        constexpr int u = decltype(Uc)::value;
-        P[u] = few_load16(rs[u], r0 + q < r_end ? off[u] : kNoFetch, (r0 - r_base) * pitch);
+    // Load slots: one per unit, requested again as soon as it has been decoded; two units per wave (two sets of rows)
+    // would leave 2 KB per wave in flight, so they keep the slots of two trips.
+    constexpr int D = U <= 2 ? 2 : 1;
+    uint4 P[D][U];
+    auto fetch = [&](auto Dc, auto Uc, int r0) {
+        constexpr int d = decltype(Dc)::value, u = decltype(Uc)::value;
+        P[d][u] = few_load16(rs[u], r0 + q < r_end ? off[u] : kNoFetch, (r0 - r_base) * pitch);
     };
     auto norm_of = [&](int r0) {
         const int rn = r0 + ((lane >> 2) & 3);
@@ -473,10 +476,16 @@ __device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int bloc
     }
     __builtin_amdgcn_sched_barrier(0);
     float nrm = norm_of(r_begin);
-    fetch(std::integral_constant<int, 0>{}, r_begin);
-    if constexpr (U > 1) fetch(std::integral_constant<int, 1>{}, r_begin);
-    if constexpr (U > 2) fetch(std::integral_constant<int, 2>{}, r_begin);
-    if constexpr (U > 3) fetch(std::integral_constant<int, 3>{}, r_begin);
+    using D0 = std::integral_constant<int, 0>;
+    using D1 = std::integral_constant<int, D - 1>;
+    fetch(D0{}, std::integral_constant<int, 0>{}, r_begin);
+    if constexpr (U > 1) fetch(D0{}, std::integral_constant<int, 1>{}, r_begin);
+    if constexpr (U > 2) fetch(D0{}, std::integral_constant<int, 2>{}, r_begin);
+    if constexpr (U > 3) fetch(D0{}, std::integral_constant<int, 3>{}, r_begin);
+    if constexpr (D == 2) {
+        fetch(D1{}, std::integral_constant<int, 0>{}, r_begin + 4);
+        if constexpr (U > 1) fetch(D1{}, std::integral_constant<int, 1>{}, r_begin + 4);
+    }
 
     // Byte-pair tables of both planes -> LDS.  (Both planes' entries are made from scalar loads and chosen per lane
     // afterwards: a choice between the two addresses instead becomes a vector load, which queues behind the
@@ -507,7 +516,7 @@ __device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int bloc
 #pragma unroll
             for (int j = 0; j < 16; ++j) xh[e][u][j] = (act[u] && q + 4 * e < a.batch) ? xh[e][u][j] : 0u;   // idle lanes contribute 0
 
-    for (int it = 0; it < a.iters; ++it) {
+    auto trip = [&](auto Dc, int it) {
         const int r0 = r_begin + 4 * it;
         const float nrm_next = norm_of(r0 + 4);
         few_f4 acc[SETS];
@@ -515,8 +524,8 @@ __device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int bloc
         for (int e = 0; e < SETS; ++e) acc[e] = few_f4{0.0f, 0.0f, 0.0f, 0.0f};
         auto segment = [&](auto Uc) {
             constexpr int u = decltype(Uc)::value;
-            const uint4 p = P[u];
-            fetch(Uc, r0 + 4);
+            const uint4 p = P[decltype(Dc)::value][u];
+            fetch(Dc, Uc, r0 + 4 * D);
             const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
             for (int d = 0; d < 4; ++d) {                      // dword d: columns 8 d .. 8 d + 7 of the lane's 32
@@ -569,7 +578,13 @@ __device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int bloc
                 if (q + 4 * e < a.batch) store_scalar(a.y, a.y_dtype, (size_t)(q + 4 * e) * out + r, total[e] * (a.L.inv_scale * nrm));
         }
         nrm = nrm_next;
+    };
+    int it = 0;
+    for (; it + D <= a.iters; it += D) {
+        trip(D0{}, it);
+        if constexpr (D == 2) trip(D1{}, it + 1);
     }
+    if (it < a.iters) trip(D0{}, it);
 }
 
 template <int SETS, int U>
