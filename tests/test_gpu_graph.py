@@ -163,7 +163,7 @@ def test_reserved_layer_is_captured_and_replayed(tq, oracle, mode, out, inf, bs,
     hip.close()
 
 
-@pytest.mark.parametrize("dual,out,inf,bs,batches", [(False, 12300, 8192, 512, (3, 8)),     # rows rotated in the kernel; two sets of rows, rotated by a kernel of their own
+@pytest.mark.parametrize("dual,out,inf,bs,batches", [(False, 12300, 8192, 512, (3, 8, 11)),     # rows rotated in the kernel; two sets of rows, rotated by a kernel of their own
                                                      (False, 4700, 14336, 256, (4,)),        # images that do not fit LDS
                                                      (True, 19701, 5120, 512, (2, 4))])      # nibble planes: two rotations
 def test_whole_row_kernel_with_rotated_rows_is_captured_and_replayed(tq, oracle, dual, out, inf, bs, batches):

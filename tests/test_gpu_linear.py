@@ -465,7 +465,7 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     layer.close()
 
 
-# ------------------------------------------------------------------ two to eight rows, whole weight rows per stream
+# ------------------------------------------------------------------ two to twelve rows, whole weight rows per stream
 @pytest.mark.parametrize("out,inf,bs,batch", [
     # the workgroups rotate the activation rows themselves: 2..7 segments of 256 columns per wave, one wave per row
     # quad (no cross-wave sum) or several
@@ -481,8 +481,10 @@ def test_small_batch_mfma_path_matches_oracle_and_batch1(tq, oracle, mode, out, 
     (4096, 17408, 512, 3), (3500, 24576, 512, 4), (2600, 27648, 512, 4), (2600, 32768, 512, 2), (5000, 14336, 512, 4),
     # five to eight rows: two sets of four on the same decoded weights, planes of 96 MB and more
     (19701, 5120, 512, 8), (12300, 8192, 256, 5), (6200, 16384, 512, 7), (66000, 1536, 512, 6), (49500, 2048, 128, 8),
-    (197000, 512, 64, 6)])
-def test_two_to_eight_rows_whole_row_kernel(tq, oracle, out, inf, bs, batch):
+    (197000, 512, 64, 6),
+    # nine to twelve rows: three sets, two segments per wave, rows of eight waves and more
+    (12300, 8192, 512, 9), (25000, 4096, 256, 12), (12400, 8192, 128, 11), (13200, 7680, 256, 10)])
+def test_two_to_twelve_rows_whole_row_kernel(tq, oracle, out, inf, bs, batch):
     _whole_row_kernel_case(tq, oracle, "shared", out, inf, bs, batch)
 
 
@@ -492,12 +494,12 @@ def test_two_to_eight_rows_whole_row_kernel(tq, oracle, out, inf, bs, batch):
     ("dual", 19701, 5120, 512, 4), ("dual", 12300, 8192, 256, 3), ("dual", 12300, 8192, 512, 7), ("dual", 33000, 3072, 128, 2),
     ("dual", 6200, 16384, 512, 4), ("dual", 25000, 4096, 512, 8), ("dual", 9000, 11264, 256, 3),
     ("primary_only", 39400, 5120, 512, 4), ("primary_only", 50000, 4096, 256, 6)])
-def test_two_to_eight_rows_whole_row_kernel_nibble_planes(tq, oracle, mode, out, inf, bs, batch):
+def test_two_to_twelve_rows_whole_row_kernel_nibble_planes(tq, oracle, mode, out, inf, bs, batch):
     _whole_row_kernel_case(tq, oracle, mode, out, inf, bs, batch)
 
 
 def _whole_row_kernel_case(tq, oracle, mode, out, inf, bs, batch):
-    """2..8 rows on a shared-rotation layer: the kernel that reads whole weight rows per stream (four weight rows by
+    """2..12 rows (nibble planes: 2..8): the kernel that reads whole weight rows per stream (four weight rows by
     four activation rows per v_mfma_f32_4x4x4_16b_f16 block, fp16 weights and rotated activations, fp32 sums, the
     cross-wave sum inside the workgroup).  1e-3 relative L2 against the oracle for every activation type (5e-3 with a
     bf16 output), every activation row by itself, every row equal to its batch-1 result within the same bound, and

@@ -307,7 +307,8 @@ def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):
 @pytest.mark.parametrize("outs,in_f,bs,batch,dual", [((9900, 9850), 10240, 512, 8, False),     # two sets of four rows: 96 MB and more per layer
                                                      ((4700, 4800, 4690), 14336, 256, 4, False),   # images that do not fit LDS
                                                      ((19701, 19800), 5120, 512, 3, True),         # nibble planes: two rotations per layer
-                                                     ((12300, 12400), 8192, 256, 6, True)])
+                                                     ((12300, 12400), 8192, 256, 6, True),
+                                                     ((12300, 12500), 8192, 512, 10, False)])      # three sets of four rows
 def test_forward_group_rows_rotated_by_a_kernel_of_their_own(tq, oracle, outs, in_f, bs, batch, dual):
     """tq_linear_forward_group where the two-to-eight-row kernel takes rows that come rotated: one rotation launch
     writes every layer's rotation (each layer has a seed of its own) into its part of the first layer's workspace.

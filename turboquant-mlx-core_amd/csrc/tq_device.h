@@ -83,7 +83,7 @@ hipError_t launch_skinny(const LayerView& L, const void* x, int x_dtype, int bat
 bool skinny_group_supported(const LayerView* Ls, int n, int x_dtype, int batch, int num_cus);
 hipError_t launch_skinny_group(const LayerView* Ls, int n, const void* x, int x_dtype, int batch, void* const* ys,
                                int y_dtype, float* const* partials, int num_cus, hipStream_t stream);
-// Two to eight rows on shared-rotation layers (tq_gemv_few.hip): the batch-1 kernel's shape (whole weight rows per
+// Two to twelve rows (tq_gemv_few.hip): the batch-1 kernel's shape (whole weight rows per
 // stream, no cut along K, no second kernel), four weight rows by four activation rows per 4x4x4 matrix block.
 // workspace: gemv_few_workspace_bytes() (0 for most calls of up to four rows: the workgroups rotate the rows
 // themselves); a group needs that of its first layer once per layer.

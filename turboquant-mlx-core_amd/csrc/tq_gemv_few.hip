@@ -1,11 +1,11 @@
-// Fused TQ8 dequant + matrix-vector products for gfx950, two to eight activation rows, blocks of at most 512
+// Fused TQ8 dequant + matrix-vector products for gfx950, two to twelve activation rows, blocks of at most 512
 // columns: shared-rotation layers (one byte per weight) and, further down, nibble planes (dual rotation, primary only).
 //
 // The batch-1 kernel (tq_gemv_wide.hip) reads the plane in whole rows and runs at the rate of its table reads.  The
 // small-batch kernel (tq_skinny.hip) puts the activation rows on v_mfma_f32_16x16x32_f16, whose operand layout
 // wants 16 weight rows per load instruction, 64 bytes of each; it cuts K over the workgroups and adds the parts in a
-// second kernel.  Four activation rows fit v_mfma_f32_4x4x4_16b_f16 instead (five to eight: two such sets on the
-// same decoded weights): 16 independent 4 x 4 x 4 blocks per instruction, block = lane / 4.  The four lanes of a
+// second kernel.  Four activation rows fit v_mfma_f32_4x4x4_16b_f16 instead (five to twelve: two or three such sets on
+// the same decoded weights): 16 independent 4 x 4 x 4 blocks per instruction, block = lane / 4.  The four lanes of a
 // block hold the same 16 columns of four consecutive weight rows (A operand: four decoded weights per step) and of
 // the four activation rows (B operand), so
 //   * a load instruction of a wave fetches 256 contiguous bytes of each of four rows (whole cache lines, streaming
@@ -31,10 +31,11 @@ namespace tq {
 namespace {
 
 constexpr int kSegCols = 256;                    // columns of a segment: 16 blocks x 16 columns
-constexpr int kFewMaxBatch = 8;
+constexpr int kFewMaxBatch = 12;                 // byte plane; nibble planes: 8
 constexpr int kFewImageBytes = 88 * 1024;        // fp16 images of the activation rows in LDS
 constexpr int kFewMaxU = 8;
-constexpr int kFewPartialBytes = 2 * 16 * 32 * 4;   // [2 buffers][<= 16 waves][16 sums x 2 sets of activation rows]
+constexpr int kFewSumStride = 48;                 // floats per wave in the cross-wave buffer: 16 sums x up to 3 sets of rows
+constexpr int kFewPartialBytes = 2 * 16 * kFewSumStride * 4;   // [2 buffers][<= 16 waves][kFewSumStride]
 
 // (Two quads of weight rows per trip of the main loop, for twice the loads in flight and half the cross-wave sums,
 // measured no faster on the large layers and slower on the small ones, whose streams have one or two quads.)
@@ -209,10 +210,16 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
     for (int u = 0; u < U; ++u) off[u] = act[u] ? (uint32_t)q * (uint32_t)K + (uint32_t)col[u] : kNoFetch;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(a.L.packed_combined) + (size_t)r_base * (size_t)K, 0, 0x7fffffff, 0x00020000);
-    uint4 P[U];                               // one load slot per segment, requested again as soon as it is decoded
-    auto fetch = [&](auto Uc, int r0) {
-        constexpr int u = decltype(Uc)::value;
-        P[u] = few_load16(rs, r0 + q < r_end ? off[u] : kNoFetch, (r0 - r_base) * K);
+    // One load slot per segment, requested again as soon as it is decoded.  Two segments per wave (three sets of
+    // rows) would leave 2 KB per wave in flight, so they keep the slots of two trips.  (With three and four
+    // segments per wave two trips were slower: 27648 x 5120 28.2 / 29.4 / 31.5 against 27.4 / 28.8 / 30.4 us.)
+    constexpr int D = U <= 2 ? 2 : 1;
+    using D0 = std::integral_constant<int, 0>;
+    using D1 = std::integral_constant<int, D - 1>;
+    uint4 P[D][U];
+    auto fetch = [&](auto Dc, auto Uc, int r0) {
+        constexpr int d = decltype(Dc)::value, u = decltype(Uc)::value;
+        P[d][u] = few_load16(rs, r0 + q < r_end ? off[u] : kNoFetch, (r0 - r_base) * K);
     };
     auto norm_of = [&](int r0) {
         const int rn = r0 + ((lane >> 2) & 3);
@@ -248,10 +255,14 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
     }
     __builtin_amdgcn_sched_barrier(0);
     float nrm = norm_of(r_begin);
-    fetch(std::integral_constant<int, 0>{}, r_begin);
-    if constexpr (U > 1) fetch(std::integral_constant<int, 1>{}, r_begin);
-    if constexpr (U > 2) fetch(std::integral_constant<int, 2>{}, r_begin);
-    if constexpr (U > 3) fetch(std::integral_constant<int, 3>{}, r_begin);
+    fetch(D0{}, std::integral_constant<int, 0>{}, r_begin);
+    if constexpr (U > 1) fetch(D0{}, std::integral_constant<int, 1>{}, r_begin);
+    if constexpr (U > 2) fetch(D0{}, std::integral_constant<int, 2>{}, r_begin);
+    if constexpr (U > 3) fetch(D0{}, std::integral_constant<int, 3>{}, r_begin);
+    if constexpr (D == 2) {
+        fetch(D1{}, std::integral_constant<int, 0>{}, r_begin + 4);
+        if constexpr (U > 1) fetch(D1{}, std::integral_constant<int, 1>{}, r_begin + 4);
+    }
 
     // Decode table -> LDS, one private column per lane: fp16 value in the upper half of the entry.  Values through
     // scalar loads (a vector memory instruction holds the CU's address unit for 16 cycles, and 16 waves share it).
@@ -302,10 +313,10 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
     }
     // The other load slots are requested behind the barrier: a wave whose requests queue up in the memory pipeline
     // would otherwise keep the whole workgroup waiting there.
-    if constexpr (U > 4) fetch(std::integral_constant<int, 4>{}, r_begin);
-    if constexpr (U > 5) fetch(std::integral_constant<int, 5>{}, r_begin);
-    if constexpr (U > 6) fetch(std::integral_constant<int, 6>{}, r_begin);
-    if constexpr (U > 7) fetch(std::integral_constant<int, 7>{}, r_begin);
+    if constexpr (U > 4) fetch(D0{}, std::integral_constant<int, 4>{}, r_begin);
+    if constexpr (U > 5) fetch(D0{}, std::integral_constant<int, 5>{}, r_begin);
+    if constexpr (U > 6) fetch(D0{}, std::integral_constant<int, 6>{}, r_begin);
+    if constexpr (U > 7) fetch(D0{}, std::integral_constant<int, 7>{}, r_begin);
 
     // Four weights of this lane's row -> one A operand (entries are fp32 patterns with the fp16 value in the upper half).
     auto operand = [&](uint32_t w) {
@@ -317,7 +328,7 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
         return __builtin_bit_cast(few_h4, r);
     };
 
-    for (int it = 0; it < a.iters; ++it) {
+    auto trip = [&](auto Dc, int it) {
         const int r0 = r_begin + 4 * it;
         const float nrm_next = norm_of(r0 + 4);
         few_f4 acc[SETS];                                      // results D[i][q] of the lane's block: weight rows r0 + i
@@ -325,8 +336,8 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
         for (int e = 0; e < SETS; ++e) acc[e] = few_f4{0.0f, 0.0f, 0.0f, 0.0f};
         auto segment = [&](auto Uc) {
             constexpr int u = decltype(Uc)::value;
-            const uint4 p = P[u];
-            fetch(Uc, r0 + 4);
+            const uint4 p = P[decltype(Dc)::value][u];
+            fetch(Dc, Uc, r0 + 4 * D);
             const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
@@ -359,10 +370,10 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
         const bool owner = lane < 16 && r < r_end;
         bool store = owner;
         if (a.W > 1) {                                         // cross-wave sum of the row's segments
-            float* const buf_base = partial + (it & 1) * (16 * 32);
+            float* const buf_base = partial + (it & 1) * (16 * kFewSumStride);
             if (lane < 16) {
 #pragma unroll
-                for (int e = 0; e < SETS; ++e) buf_base[wave * 32 + 16 * e + lane] = total[e];
+                for (int e = 0; e < SETS; ++e) buf_base[wave * kFewSumStride + 16 * e + lane] = total[e];
             }
             __syncthreads();
             store = owner && unit == 0;
@@ -370,7 +381,7 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
 #pragma unroll
                 for (int e = 0; e < SETS; ++e) {
                     float t = 0.0f;
-                    for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * 32 + 16 * e + lane];
+                    for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * kFewSumStride + 16 * e + lane];
                     total[e] = t;
                 }
             }
@@ -381,7 +392,13 @@ __device__ __forceinline__ void few_body(const FewArgs& a, const int block) {
                 if (q + 4 * e < a.batch) store_scalar(a.y, a.y_dtype, (size_t)(q + 4 * e) * out + r, total[e] * (a.L.inv_scale * nrm));
         }
         nrm = nrm_next;
+    };
+    int it = 0;
+    for (; it + D <= a.iters; it += D) {
+        trip(D0{}, it);
+        if constexpr (D == 2) trip(D1{}, it + 1);
     }
+    if (it < a.iters) trip(D0{}, it);
 }
 
 template <int SETS, int U, int TL, bool PRE>
@@ -556,10 +573,10 @@ __device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int bloc
         const bool owner = lane < 16 && r < r_end;
         bool store = owner;
         if (a.W > 1) {
-            float* const buf_base = partial + (it & 1) * (16 * 32);
+            float* const buf_base = partial + (it & 1) * (16 * kFewSumStride);
             if (lane < 16) {
 #pragma unroll
-                for (int e = 0; e < SETS; ++e) buf_base[wave * 32 + 16 * e + lane] = total[e];
+                for (int e = 0; e < SETS; ++e) buf_base[wave * kFewSumStride + 16 * e + lane] = total[e];
             }
             __syncthreads();
             store = owner && unit == 0;
@@ -567,7 +584,7 @@ __device__ __forceinline__ void few_nibble_body(const FewArgs& a, const int bloc
 #pragma unroll
                 for (int e = 0; e < SETS; ++e) {
                     float t = 0.0f;
-                    for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * 32 + 16 * e + lane];
+                    for (int w = 0; w < a.W; ++w) t += buf_base[(stream * a.W + w) * kFewSumStride + 16 * e + lane];
                     total[e] = t;
                 }
             }
@@ -647,8 +664,8 @@ FewShape few_shape(const LayerView& L, int batch) {
     FewShape s{};
     const int K = L.in_features;
     const bool nib = few_nibble(L);
-    s.sets = batch > 4 ? 2 : 1;
-    const int max_u = nib ? (s.sets == 2 ? 2 : 4) : (s.sets == 2 ? 4 : kFewMaxU);
+    s.sets = (batch + 3) / 4;
+    const int max_u = nib ? (s.sets == 2 ? 2 : 4) : (s.sets >= 3 ? 2 : s.sets == 2 ? 4 : kFewMaxU);
     const int units = nib ? few_planes(L) * ((K + 511) / 512) : (K + kSegCols - 1) / kSegCols;
     auto efficiency = [&](int W, int& U) {
         U = (units + W - 1) / W;
@@ -673,7 +690,7 @@ FewShape few_shape(const LayerView& L, int batch) {
     s.threads = s.W * s.S * kWave;
     const int ntiles = (K + kTile - 1) / kTile, waves = s.W * s.S;
     const int per_wave = (batch * ntiles + waves - 1) / waves;
-    s.pre = nib || s.sets == 2 || (size_t)batch * K * 2 > (size_t)kFewImageBytes || per_wave > 6;
+    s.pre = nib || s.sets >= 2 || (size_t)batch * K * 2 > (size_t)kFewImageBytes || per_wave > 6;
     s.tl = per_wave <= 3 ? 3 : 6;
     return s;
 }
@@ -710,7 +727,11 @@ hipError_t launch_few_u(const Args& a, const FewShape& s, int grid, hipStream_t 
             } else hipLaunchKernelGGL((tq_gemv_few_nibble_kernel<1, U>), g, b, 0, stream, a);
         }
     } else if constexpr (GROUP) {
-        if (s.sets == 2) {
+        if (s.sets == 3) {
+            if constexpr (U <= 2) hipLaunchKernelGGL((tq_gemv_few_group_kernel<3, U, 1, true>), g, b, 0, stream, a);
+            else return hipErrorInvalidValue;
+        }
+        else if (s.sets == 2) {
             if constexpr (U <= 4) hipLaunchKernelGGL((tq_gemv_few_group_kernel<2, U, 1, true>), g, b, 0, stream, a);
             else return hipErrorInvalidValue;
         }
@@ -718,7 +739,11 @@ hipError_t launch_few_u(const Args& a, const FewShape& s, int grid, hipStream_t 
         else if (s.tl == 3) hipLaunchKernelGGL((tq_gemv_few_group_kernel<1, U, 3, false>), g, b, 0, stream, a);
         else hipLaunchKernelGGL((tq_gemv_few_group_kernel<1, U, 6, false>), g, b, 0, stream, a);
     } else {
-        if (s.sets == 2) {
+        if (s.sets == 3) {
+            if constexpr (U <= 2) hipLaunchKernelGGL((tq_gemv_few_kernel<3, U, 1, true>), g, b, 0, stream, a);
+            else return hipErrorInvalidValue;
+        }
+        else if (s.sets == 2) {
             if constexpr (U <= 4) hipLaunchKernelGGL((tq_gemv_few_kernel<2, U, 1, true>), g, b, 0, stream, a);
             else return hipErrorInvalidValue;
         }
@@ -733,7 +758,7 @@ hipError_t launch_few_u(const Args& a, const FewShape& s, int grid, hipStream_t 
 // that fit fp16, blocks of at most 512 columns (a block never leaves the tile a wave rotates), rows of at most 64
 // tiles that some split covers.
 bool few_layer_ok(const LayerView& L, int batch) {
-    if (batch < 2 || batch > kFewMaxBatch) return false;
+    if (batch < 2 || batch > (few_nibble(L) ? 8 : kFewMaxBatch)) return false;
     if (!L.fp16_centroids_ok) return false;
     if (L.mode == kSharedLut) { if (!L.packed_combined) return false; }
     else if (few_nibble(L)) { if (!L.packed_primary || (L.mode == kDual && !L.packed_residual)) return false; }
@@ -764,8 +789,13 @@ bool few_worth_it(const LayerView& L, const FewShape& s, int batch) {
     // (nibble planes, two to four rows: 27648 x 5120 34.6 against 40.2 us, 28672 x 8192 47.9 / 62.0, but 8192 x 8192
     // 23.9 / 21.7; five to eight: 28672 x 8192 59.8 / 68.1, but 27648 x 5120, whose 20 units make two per wave of 10
     // waves, 56.2 / 44.4: two sets want a workgroup of 14 waves and more)
-    if (s.sets == 2 && s.W * s.S < 14) return false;
-    if (s.pre) return plane_bytes >= ((s.sets == 2 || few_nibble(L)) ? (96ll << 20) : (64ll << 20));
+    // (nine to twelve rows, three sets, two segments per wave: 28672 x 8192 53.9 / 55.3 against 59.8 / 63.2 us at 9 / 12
+    // rows, 65536 x 4096 60.4 / 62.0 against 70.2 / 74.3, but the lm_head of 2048 columns, four waves per row and four
+    // streams, 94.1 / 95.5 against 87.9 / 94.1: rows of eight waves and more.  Four sets, 128 registers and ten spilled,
+    // took 104-111 us where the small-batch kernel takes 65-103.)
+    if (s.sets >= 2 && s.W * s.S < 14) return false;
+    if (s.sets == 3 && s.W < 8) return false;
+    if (s.pre) return plane_bytes >= ((s.sets >= 2 || few_nibble(L)) ? (96ll << 20) : (64ll << 20));
     const long long jobs = (long long)batch * ((K + kTile - 1) / kTile);
     return jobs <= 40 || jobs * 5 <= 135 + plane_bytes / 500000;           // jobs <= 27 + 0.4 per MB
 }
@@ -813,7 +843,7 @@ hipError_t few_rotate_rows(FewArgs* as, int n, const void* x, int x_dtype, int b
 
 }  // namespace
 
-// Two to eight rows of any activation type.
+// Two to twelve rows (nibble planes: eight) of any activation type.
 bool gemv_few_supported(const LayerView& L, int batch, int num_cus) {
     if (!few_layer_ok(L, batch) || !few_share_ok(L, num_cus)) return false;
     return few_worth_it(L, few_shape(L, batch), batch);

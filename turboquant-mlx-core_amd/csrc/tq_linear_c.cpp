@@ -373,7 +373,7 @@ int forward_view(tq_linear_s* h, const tq::LayerView& V, bool generic_only, cons
                  void* y_dev, int y_dtype, hipStream_t stream, const float* gate, void* static_ws, size_t static_cap) {
     const bool lanes = !generic_only && tq::lanes_supported(V.in_features, V.block_size);
     // (the gated store is a feature of the one-row kernels; 16..32 rows: the small-batch kernel where it takes the layer)
-    // (two to eight rows on a shared-rotation layer: whole weight rows per stream, 4 x 4 x 4 matrix blocks; a
+    // (two to twelve rows: whole weight rows per stream, 4 x 4 x 4 matrix blocks; a
     // workspace only where the rows are rotated by a kernel of their own)
     if (lanes && !gate && tq::gemv_few_supported(V, batch, device_cu_count())) {
         const size_t need = tq::gemv_few_workspace_bytes(V, batch);
@@ -530,11 +530,11 @@ int tq_linear_forward(tq_linear_t h, const void* x_dev, int x_dtype, int batch,
 }
 
 namespace {
-// Workspace of the two-to-eight-row kernel for every batch up to max_batch, thrice: the first layer of a group holds
+// Workspace of the whole-row kernel (2..12 rows) for every batch up to max_batch, thrice: the first layer of a group holds
 // the rotated rows of all its layers.
 size_t few_reserve_bytes(const tq::LayerView& V, int max_batch) {
     size_t need = 0;
-    for (int b = 2; b <= max_batch && b <= 8; ++b) need = std::max(need, 3 * tq::gemv_few_workspace_bytes(V, b));
+    for (int b = 2; b <= max_batch && b <= 12; ++b) need = std::max(need, 3 * tq::gemv_few_workspace_bytes(V, b));
     return need;
 }
 }  // namespace
