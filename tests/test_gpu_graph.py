@@ -167,7 +167,7 @@ def test_reserved_layer_is_captured_and_replayed(tq, oracle, mode, out, inf, bs,
                                                      (False, 4700, 14336, 256, (4,)),        # images that do not fit LDS
                                                      (True, 19701, 5120, 512, (2, 4))])      # nibble planes: two rotations
 def test_whole_row_kernel_with_rotated_rows_is_captured_and_replayed(tq, oracle, dual, out, inf, bs, batches):
-    """The kernel for two to eight rows where a kernel of its own rotates the rows into the layer's workspace: after
+    """The kernel for two to twelve rows where a kernel of its own rotates the rows into the layer's workspace: after
     tq_linear_reserve both launches of a call are captured, and every replay gives the bits of the eager call (a
     sample of whose rows is checked against the oracle)."""
     o, hip = oracle, _Hip()

@@ -310,7 +310,7 @@ def test_forward_group_small_batches(tq, oracle, shared, batch, outs, in_f, bs):
                                                      ((12300, 12400), 8192, 256, 6, True),
                                                      ((12300, 12500), 8192, 512, 10, False)])      # three sets of four rows
 def test_forward_group_rows_rotated_by_a_kernel_of_their_own(tq, oracle, outs, in_f, bs, batch, dual):
-    """tq_linear_forward_group where the two-to-eight-row kernel takes rows that come rotated: one rotation launch
+    """tq_linear_forward_group where the kernel for two to twelve rows takes rows that come rotated: one rotation launch
     writes every layer's rotation (each layer has a seed of its own) into its part of the first layer's workspace.
     Bit-identical to separate calls, twice in a row; a sample of the rows against the dense product."""
     hip = _Hip()

@@ -113,7 +113,7 @@ struct tq_linear_s {
 };
 
 // Workspace of the matrix-core paths for callers that cannot allocate (tq_linear_forward_static):
-// rotated activations (tile images, or the fp16 rows of the two-to-eight-row kernel) followed by the per-chunk
+// rotated activations (tile images, or the fp16 rows of the whole-row kernel for 2..12 rows) followed by the per-chunk
 // partial products of the small-batch kernels.  One copy per GPU, held until the process ends; every call on a GPU shares it, so calls
 // that overlap on one GPU race.  Nothing in it has to start at zero: the kernels write every element
 // they later read (rows past the batch are computed from whatever is there and never stored).
